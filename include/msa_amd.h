@@ -1,0 +1,162 @@
+/*
+ * msa_amd — C ABI of the MI355X (gfx950) routing / sparse-attention hot path of MSA.
+ *
+ * The reference (EverMind-AI/MSA) is pure Python: its "FFI" for this path is a set of torch
+ * op sequences inside three Python call sites.  Each entry point below replaces one of those
+ * sequences and cites it (paths relative to the reference checkout).  A Python maintainer binds
+ * these with ctypes (see msa_amd/_lib.py) and passes `tensor.data_ptr()`.
+ *
+ * Conventions
+ *   - every function returns 0 (MSA_OK) or a negative MSA_E* code and never throws;
+ *     msa_last_error() gives the message of the calling thread's last failure;
+ *   - pointers are DEVICE pointers unless the name ends in `_host`;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); all work is
+ *     enqueued on it and nothing synchronises unless stated;
+ *   - no entry point allocates device memory: scratch comes in as `workspace`, sized by the
+ *     matching *_workspace_bytes() function;
+ *   - activations are token-major [T, H, D]; pooled tensors and the bank are chunk-major
+ *     [C, Hkv, D]; document indices are 0-based in bank order; D must be 128;
+ *   - dtype: MSA_BF16 (storage bf16, fp32 accumulation) or MSA_F32.
+ */
+#ifndef MSA_AMD_H
+#define MSA_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MSA_OK 0
+#define MSA_EINVAL (-1)   /* bad argument (shape, null pointer, unsupported value) */
+#define MSA_EHIP (-2)     /* a HIP runtime call failed */
+#define MSA_ESIZE (-3)    /* workspace or output capacity too small */
+#define MSA_ESTATE (-4)   /* bank layer not set / handle misuse */
+
+#define MSA_BF16 0
+#define MSA_F32 1
+
+#define MSA_MODE_COSINE 0      /* q L2-normalised per head here, K_r expected normalised, scale 1 */
+#define MSA_MODE_SCALED_DOT 1  /* raw dot product times `scale` (head_dim^-0.5 in the reference) */
+
+const char* msa_last_error(void);
+int msa_abi_version(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Chunk table of a packed block.  Replaces the nonzero / unique_consecutive / cumsum /
+ * repeat_interleave chain of src/msa/memory_sparse_attention.py:138-163 and the per-document
+ * ceil(len / P) of src/prefill.py:225.
+ *   doc_start[n_docs+1]: token offset of each document in the packed block (doc_start[0] may be
+ *   > 0: template tokens in front belong to no chunk).  Document d has ceil(len_d / P) chunks.
+ * Outputs (capacity `chunk_cap` entries each, writes beyond it are suppressed):
+ *   doc_chunk_off[n_docs+1], chunk_start[C] (first token), chunk_len[C] (1..P),
+ *   chunk_doc[C] (0-based document), n_chunks_out[1] (int64, total C for the caller to verify). */
+int msa_chunk_table(const int32_t* doc_start, int32_t n_docs, int32_t P, int64_t chunk_cap,
+                    int32_t* doc_chunk_off, int32_t* chunk_start, int32_t* chunk_len,
+                    int32_t* chunk_doc, int64_t* n_chunks_out, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Chunk-mean pooling of K, V and K_r.  Replaces sequence_pooling_kv
+ * (src/msa/memory_sparse_attention.py:467-486), the inline K_r pooling (:178-190) and the
+ * optional normalise (:192-194); with `rope_cos` it also fuses the rotary of :133 into the K read.
+ *   k, v, kr: [T, H, D] token-major, any of them may be NULL (skipped with its output).
+ *   Sums are direct fp32 segment sums; a partial last chunk is divided by its true length.
+ *   rope_cos / rope_sin: fp32 [rope_rows, D/2] tables or NULL.  When given, K is rotated
+ *   (half-split layout) at position (token - first token of its document) before pooling and
+ *   `max_doc_len` must not exceed rope_rows.  `doc_start` is only read in that case.
+ *   normalize_kr != 0: pooled K_r is divided by max(||.||_2, 1e-12) per (chunk, head). */
+int msa_pool_chunks(const void* k, const void* v, const void* kr, int32_t dtype, int64_t T,
+                    int32_t H, int32_t D, const int32_t* chunk_start, const int32_t* chunk_len,
+                    const int32_t* chunk_doc, int64_t C, const int32_t* doc_start,
+                    const float* rope_cos, const float* rope_sin, int32_t rope_rows,
+                    int32_t max_doc_len, int32_t normalize_kr, void* k_out, void* v_out,
+                    void* kr_out, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Memory bank.  Replaces Memory._init_block_data / BlockDesc / _generate_slice
+ * (src/msa_service.py:191-231, 481-492, 644-695): K_r resident in HBM, pooled K / V in pinned
+ * host memory, documents as contiguous chunk ranges.  The handle copies the two tables; the
+ * per-layer tensors stay owned by the caller and must outlive the handle's use of them.
+ *   doc_chunk_off_host[n_docs+1] (int32, first entry 0, last entry C), doc_global_id_host[n_docs]. */
+typedef struct msa_bank msa_bank;
+int msa_bank_create(msa_bank** out, int32_t n_layers, int64_t C, int32_t Hkv, int32_t D,
+                    int32_t dtype, const int32_t* doc_chunk_off_host,
+                    const int64_t* doc_global_id_host, int64_t n_docs);
+/* kr_dev: device [C, Hkv, D]; k_host / v_host: pinned host [C, Hkv, D] (may be NULL for a
+ * scoring-only bank). */
+int msa_bank_set_layer(msa_bank* bank, int32_t layer, const void* kr_dev, const void* k_host,
+                       const void* v_host);
+int msa_bank_destroy(msa_bank* bank);
+
+/* ---------------------------------------------------------------------------------------------
+ * Router scoring + top-k.  Replaces MSAService._gather_querys' scaling / regrouping
+ * (src/msa_service.py:1095-1100) and Memory.prefill_stage2 (:703-828): matmul, pad-token mask,
+ * mean over the Hq heads, max over query tokens, max over a document's chunks, top-k.
+ *   q: [B, S, Hq, D] (token-major, NOT pre-scaled), qmask_u8: [B, S] (1 = scored token) or NULL.
+ *   msa_chunk_scores writes chunk_scores[B, C] fp32 (-inf where a query has no scored token).
+ *   msa_route_topk writes scores_out[B, topk] (descending; ties by lower document index),
+ *   doc_out[B, topk] (0-based, -1 past the number of documents) and doc_global_out[B, topk]
+ *   (doc_global_id[doc], -1 likewise).  topk <= 64. */
+size_t msa_route_workspace_bytes(int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D,
+                                 int64_t C, int64_t n_docs, int32_t topk);
+int msa_chunk_scores(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8,
+                     int32_t B, int32_t S, int32_t Hq, int32_t mode, float scale,
+                     float* chunk_scores, void* workspace, size_t workspace_bytes, void* stream);
+int msa_route_topk(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8,
+                   int32_t B, int32_t S, int32_t Hq, int32_t mode, float scale, int32_t topk,
+                   float* scores_out, int32_t* doc_out, int64_t* doc_global_out, void* workspace,
+                   size_t workspace_bytes, void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Gather of the selected documents' pooled K / V from pinned host memory.  Replaces the
+ * index_select fetch and per-sample regroup of MSAService.doc_query
+ * (src/msa_service.py:1203-1262, 1289-1312).
+ *   doc_sel_host[B, k]: 0-based documents (-1 = none).  Per sample, documents are laid out in
+ *   ascending bank order, each once.  msa_gather_plan fills cu_sel_host[B+1] (prefix sums of
+ *   selected chunk counts).  msa_gather_kv enqueues one hipMemcpyAsync per contiguous document
+ *   run and tensor on `copy_stream` into k_out / v_out [cu_sel[B], Hkv, D]; the caller orders
+ *   consumers after the stream (event or synchronise). */
+int msa_gather_plan(const msa_bank* bank, const int32_t* doc_sel_host, int32_t B, int32_t k,
+                    int64_t* cu_sel_host);
+int msa_gather_kv(const msa_bank* bank, int32_t layer, const int32_t* doc_sel_host, int32_t B,
+                  int32_t k, void* k_out, void* v_out, int64_t out_capacity_chunks,
+                  void* copy_stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Context assembly.  Replaces the ragged scatter of src/msa/memory_sparse_attention.py:282-329
+ * and the compact cache of :344-351: for every sample b writes
+ *   [ prefix (n_prefix rows) | mem rows cu_sel[b]..cu_sel[b+1] | local rows cu_local[b]..cu_local[b+1] ]
+ * into kcache / vcache [B, Lcap, Hkv, D] starting at row 0 of the sample, and kv_len[b].
+ * Rows are [Hkv, D]; cu_sel / cu_local are device int32 [B+1]. */
+int msa_assemble_context(const void* prefix_k, const void* prefix_v, int32_t n_prefix,
+                         const void* mem_k, const void* mem_v, const int32_t* cu_sel,
+                         const void* local_k, const void* local_v, const int32_t* cu_local,
+                         int32_t B, int32_t Hkv, int32_t D, int32_t dtype, void* kcache,
+                         void* vcache, int32_t Lcap, int32_t* kv_len, void* stream);
+
+/* Appends one new K / V row per sample at kv_len[b] and increments kv_len[b]
+ * (the torch.cat of src/msa/memory_sparse_attention.py:372-373, done in place). */
+int msa_cache_append(const void* k_new, const void* v_new, int32_t B, int32_t Hkv, int32_t D,
+                     int32_t dtype, void* kcache, void* vcache, int32_t Lcap, int32_t* kv_len,
+                     void* stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * GQA attention of ragged query rows over per-sample KV ranges.  Replaces repeat_kv + SDPA of the
+ * decode step (src/msa/memory_sparse_attention.py:389-399) and, with several query rows per
+ * sample, the causal varlen attention of stage 2 (:334-339).
+ *   q: [sum Sq, Hq, D] with cu_q[B+1] (NULL = one row per sample); k / v: rows [Hkv, D];
+ *   sample b's keys are rows kv_off[b] .. kv_off[b] + kv_len[b].  causal != 0: query row i of a
+ *   sample with Sq rows sees the first kv_len - Sq + i + 1 keys (bottom-right aligned).
+ *   out: [sum Sq, Hq, D].  max_sq / max_kv bound the per-sample sizes (grid sizing only). */
+size_t msa_attn_workspace_bytes(int32_t total_q, int32_t Hq, int32_t D, int32_t max_kv);
+int msa_sparse_attn(const void* q, const int32_t* cu_q, const void* k, const void* v,
+                    const int64_t* kv_off, const int32_t* kv_len, int32_t B, int32_t total_q,
+                    int32_t max_sq, int32_t max_kv, int32_t Hq, int32_t Hkv, int32_t D,
+                    int32_t dtype, float scale, int32_t causal, void* out, void* workspace,
+                    size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MSA_AMD_H */

@@ -1,0 +1,53 @@
+"""Builds ``libmsa_amd.so`` (the C-ABI library) from ``csrc/*.hip`` for gfx950 with hipcc.
+
+``python -m msa_amd.build`` compiles in-tree; the library then travels with the source tree.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libmsa_amd.so")
+ARCH = "gfx950"
+# packed fp32 VALU ops are switched off for all device code of this library
+FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
+         "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
+
+
+def sources():
+    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def _compile(src: str) -> str:
+    obj = src[:-4] + ".o"
+    cmd = ["hipcc", *FLAGS, "-c", src, "-o", obj]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in r.stderr.splitlines() if noise not in l)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {src}:\n{err}")
+    if err.strip():
+        sys.stderr.write(err + "\n")
+    return obj
+
+
+def build(jobs: int = 8) -> str:
+    """Compiles every source (always, even if the library exists) and links the shared library."""
+    srcs = sources()
+    with ThreadPoolExecutor(max_workers=min(jobs, len(srcs))) as ex:
+        objs = list(ex.map(_compile, srcs))
+    tmp = LIB + ".tmp"
+    r = subprocess.run(["hipcc", "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", tmp],
+                       capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stderr}")
+    os.replace(tmp, LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build())

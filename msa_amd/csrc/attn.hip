@@ -1,0 +1,230 @@
+// GQA attention of ragged query rows over per-sample KV ranges (decode and stage-2 prefill).
+//
+// Split-KV: workgroup (query row, KV head, split) streams its slice of K and V once and serves all
+// G query heads of that KV head from the same loads.  A wavefront takes 4 keys per step (16 lanes
+// per key, 8 head-dim elements per lane); every (key slot, dim slice) lane keeps an independent
+// online-softmax state (m, l, acc[G][8]) that is merged across slots, wavefronts and finally
+// splits (second kernel).  K / V rows are [Hkv, 128].
+#include <algorithm>
+
+#include "common.h"
+
+namespace {
+
+constexpr int kAttnWaves = 4;
+constexpr int kSplitKeys = 256;   // keys per workgroup
+constexpr int kMaxG = 8;
+
+template <typename T>
+__device__ __forceinline__ void ld8(const T* p, float (&x)[8]) {
+  if constexpr (sizeof(T) == 2) {
+    const uint4 w = *reinterpret_cast<const uint4*>(p);
+    x[0] = bf16lo(w.x); x[1] = bf16hi(w.x); x[2] = bf16lo(w.y); x[3] = bf16hi(w.y);
+    x[4] = bf16lo(w.z); x[5] = bf16hi(w.z); x[6] = bf16lo(w.w); x[7] = bf16hi(w.w);
+  } else {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    const float4 b = *reinterpret_cast<const float4*>(p + 4);
+    x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+  }
+}
+
+// Finds the sample owning query row `row` in cu_q (B is small: linear scan is fine and uniform).
+__device__ __forceinline__ int find_sample(const int32_t* cu_q, int B, int row) {
+  int b = 0;
+  while (b + 1 < B && cu_q[b + 1] <= row) ++b;
+  return b;
+}
+
+template <typename T, int G>
+__global__ __launch_bounds__(kAttnWaves * 64) void attn_partial_kernel(
+    const T* __restrict__ q, const int32_t* __restrict__ cu_q, const T* __restrict__ k, const T* __restrict__ v,
+    const int64_t* __restrict__ kv_off, const int32_t* __restrict__ kv_len, int32_t B, int32_t Hq, int32_t Hkv,
+    float scale_log2e, int32_t causal, int32_t n_split, float* __restrict__ part_ml, float* __restrict__ part_acc) {
+  __shared__ float sm_m[kAttnWaves][G], sm_l[kAttnWaves][G];
+  __shared__ float sm_acc[kAttnWaves][G][kHeadDim];
+
+  const int row = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
+  const int b = cu_q ? find_sample(cu_q, B, row) : row;
+  const int q_first = cu_q ? cu_q[b] : row;
+  const int sq = cu_q ? cu_q[b + 1] - q_first : 1;
+  const int L = kv_len[b];
+  const int visible = causal ? max(0, L - sq + (row - q_first) + 1) : L;
+  const int key0 = split * kSplitKeys;
+  const int key1 = min(visible, key0 + kSplitKeys);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int slot = lane >> 4, j = lane & 15;
+  const int64_t base = kv_off[b];
+  const int row_elems = Hkv * kHeadDim;
+
+  float qv[G][8];
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    ld8<T>(q + ((int64_t)row * Hq + g * G + h) * kHeadDim + 8 * j, qv[h]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qv[h][i] *= scale_log2e;      // scores in log2 units: exp2f below
+  }
+
+  float m[G], l[G], acc[G][8];
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    m[h] = -INFINITY; l[h] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
+  }
+
+  for (int kk = key0 + wave * 4 + slot; kk < key1; kk += kAttnWaves * 4) {
+    const int64_t off = (base + kk) * row_elems + g * kHeadDim + 8 * j;
+    float kx[8], vx[8];
+    ld8<T>(k + off, kx);
+    ld8<T>(v + off, vx);
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      float s = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) s += qv[h][i] * kx[i];
+      s += __shfl_xor(s, 1); s += __shfl_xor(s, 2); s += __shfl_xor(s, 4); s += __shfl_xor(s, 8);
+      const float mn = fmaxf(m[h], s);
+      const float alpha = exp2f(m[h] - mn);     // first key: exp2f(-inf) = 0
+      const float p = exp2f(s - mn);
+      m[h] = mn;
+      l[h] = l[h] * alpha + p;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[h][i] = acc[h][i] * alpha + p * vx[i];
+    }
+  }
+
+  // merge the 4 key slots of the wavefront (lanes differing in bits 4 and 5)
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+#pragma unroll
+    for (int x = 16; x <= 32; x <<= 1) {
+      const float mo = __shfl_xor(m[h], x), lo = __shfl_xor(l[h], x);
+      const float mn = fmaxf(m[h], mo);
+      const float a = mn == -INFINITY ? 0.f : exp2f(m[h] - mn), bo = mn == -INFINITY ? 0.f : exp2f(mo - mn);
+      l[h] = l[h] * a + lo * bo;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[h][i] = acc[h][i] * a + __shfl_xor(acc[h][i], x) * bo;
+      m[h] = mn;
+    }
+  }
+  if (slot == 0) {
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      if (j == 0) { sm_m[wave][h] = m[h]; sm_l[wave][h] = l[h]; }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sm_acc[wave][h][8 * j + i] = acc[h][i];
+    }
+  }
+  __syncthreads();
+
+  // merge the wavefronts; thread (h, d) for h < G
+  for (int idx = tid; idx < G * kHeadDim; idx += kAttnWaves * 64) {
+    const int h = idx / kHeadDim, d = idx % kHeadDim;
+    float mn = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kAttnWaves; ++w) mn = fmaxf(mn, sm_m[w][h]);
+    float lt = 0.f, at = 0.f;
+#pragma unroll
+    for (int w = 0; w < kAttnWaves; ++w) {
+      const float a = mn == -INFINITY ? 0.f : exp2f(sm_m[w][h] - mn);
+      lt += sm_l[w][h] * a;
+      at += sm_acc[w][h][d] * a;
+    }
+    const int64_t o = ((int64_t)row * Hq + g * G + h) * n_split + split;
+    part_acc[o * kHeadDim + d] = at;
+    if (d == 0) { part_ml[o * 2] = mn; part_ml[o * 2 + 1] = lt; }
+  }
+}
+
+// One workgroup of 128 threads per (query row, head): merge the splits and normalise.
+template <typename T>
+__global__ __launch_bounds__(kHeadDim) void attn_combine_kernel(const float* __restrict__ part_ml,
+                                                                const float* __restrict__ part_acc, int32_t n_split,
+                                                                T* __restrict__ out) {
+  const int64_t rh = blockIdx.x;   // row * Hq + head
+  const int d = threadIdx.x;
+  float mn = -INFINITY;
+  for (int s = 0; s < n_split; ++s) mn = fmaxf(mn, part_ml[(rh * n_split + s) * 2]);
+  float lt = 0.f, at = 0.f;
+  for (int s = 0; s < n_split; ++s) {
+    const float ms = part_ml[(rh * n_split + s) * 2];
+    const float a = ms == -INFINITY ? 0.f : exp2f(ms - mn);
+    lt += part_ml[(rh * n_split + s) * 2 + 1] * a;
+    at += part_acc[(rh * n_split + s) * kHeadDim + d] * a;
+  }
+  const float o = lt > 0.f ? at / lt : 0.f;     // a row that sees no key yields zeros
+  if constexpr (sizeof(T) == 2) out[rh * kHeadDim + d] = f32_to_bf16(o);
+  else out[rh * kHeadDim + d] = o;
+}
+
+inline int splits_for(int32_t max_kv) { return std::max(1, (max_kv + kSplitKeys - 1) / kSplitKeys); }
+
+template <typename T>
+int launch_attn(const void* q, const int32_t* cu_q, const void* k, const void* v, const int64_t* kv_off,
+                const int32_t* kv_len, int32_t B, int32_t total_q, int32_t Hq, int32_t Hkv, float scale,
+                int32_t causal, int32_t n_split, void* out, float* part_ml, float* part_acc, hipStream_t st) {
+  const int G = Hq / Hkv;
+  dim3 grid((unsigned)total_q, (unsigned)Hkv, (unsigned)n_split);
+  const float sl2 = scale * 1.4426950408889634f;
+#define MSA_ATTN_CASE(GG)                                                                                          \
+  case GG:                                                                                                         \
+    attn_partial_kernel<T, GG><<<grid, kAttnWaves * 64, 0, st>>>(                                                  \
+        static_cast<const T*>(q), cu_q, static_cast<const T*>(k), static_cast<const T*>(v), kv_off, kv_len, B, Hq, \
+        Hkv, sl2, causal, n_split, part_ml, part_acc);                                                             \
+    break;
+  switch (G) {
+    MSA_ATTN_CASE(1)
+    MSA_ATTN_CASE(2)
+    MSA_ATTN_CASE(4)
+    MSA_ATTN_CASE(8)
+    default:
+      msa_set_error("msa_sparse_attn: GQA group size %d unsupported (1, 2, 4, 8)", G);
+      return MSA_EINVAL;
+  }
+#undef MSA_ATTN_CASE
+  MSA_LAUNCH_CHECK();
+  attn_combine_kernel<T><<<(unsigned)((int64_t)total_q * Hq), kHeadDim, 0, st>>>(part_ml, part_acc, n_split,
+                                                                                 static_cast<T*>(out));
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
+
+}  // namespace
+
+extern "C" size_t msa_attn_workspace_bytes(int32_t total_q, int32_t Hq, int32_t D, int32_t max_kv) {
+  if (total_q <= 0 || Hq <= 0 || D <= 0 || max_kv <= 0) return 0;
+  const size_t n = (size_t)total_q * Hq * splits_for(max_kv);
+  return align_up(n * 2 * sizeof(float), 256) + align_up(n * D * sizeof(float), 256);
+}
+
+extern "C" int msa_sparse_attn(const void* q, const int32_t* cu_q, const void* k, const void* v,
+                               const int64_t* kv_off, const int32_t* kv_len, int32_t B, int32_t total_q,
+                               int32_t max_sq, int32_t max_kv, int32_t Hq, int32_t Hkv, int32_t D, int32_t dtype,
+                               float scale, int32_t causal, void* out, void* workspace, size_t workspace_bytes,
+                               void* stream) {
+  MSA_REQUIRE(q && k && v && kv_off && kv_len && out && workspace, "msa_sparse_attn: null pointer");
+  MSA_REQUIRE(D == kHeadDim, "msa_sparse_attn: head dim %d unsupported (need %d)", D, kHeadDim);
+  MSA_REQUIRE(B > 0 && total_q > 0 && max_sq > 0 && max_kv > 0, "msa_sparse_attn: bad sizes");
+  MSA_REQUIRE(cu_q != nullptr || total_q == B, "msa_sparse_attn: cu_q is required when total_q != B");
+  MSA_REQUIRE(Hkv > 0 && Hq % Hkv == 0 && Hq / Hkv <= kMaxG, "msa_sparse_attn: Hq=%d Hkv=%d unsupported", Hq, Hkv);
+  MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "msa_sparse_attn: bad dtype %d", dtype);
+  MSA_REQUIRE(scale > 0.f, "msa_sparse_attn: scale must be positive");
+  MSA_REQUIRE((int64_t)total_q * Hq < (int64_t)1 << 31 && total_q < 65536 * 32, "msa_sparse_attn: too many rows");
+  const int n_split = splits_for(max_kv);
+  MSA_REQUIRE(n_split <= 65535, "msa_sparse_attn: max_kv=%d too large", max_kv);
+  const size_t need = msa_attn_workspace_bytes(total_q, Hq, D, max_kv);
+  if (need > workspace_bytes) {
+    msa_set_error("msa_sparse_attn: workspace of %zu bytes, need %zu", workspace_bytes, need);
+    return MSA_ESIZE;
+  }
+  const size_t n = (size_t)total_q * Hq * n_split;
+  float* part_ml = static_cast<float*>(workspace);
+  float* part_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + align_up(n * 2 * sizeof(float), 256));
+  hipStream_t st = as_stream(stream);
+  if (dtype == MSA_BF16)
+    return launch_attn<bf16_t>(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, n_split, out,
+                               part_ml, part_acc, st);
+  return launch_attn<float>(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, n_split, out, part_ml,
+                            part_acc, st);
+}

@@ -1,0 +1,82 @@
+// Shared helpers for the gfx950 kernels: error plumbing, bf16 bit tricks, ordered float keys.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/msa_amd.h"
+
+void msa_set_error(const char* fmt, ...);
+
+#define MSA_REQUIRE(cond, ...)                \
+  do {                                        \
+    if (!(cond)) {                            \
+      msa_set_error(__VA_ARGS__);             \
+      return MSA_EINVAL;                      \
+    }                                         \
+  } while (0)
+
+#define MSA_HIP(call)                                                                  \
+  do {                                                                                 \
+    hipError_t e__ = (call);                                                           \
+    if (e__ != hipSuccess) {                                                           \
+      msa_set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e__), __FILE__,  \
+                    __LINE__);                                                         \
+      return MSA_EHIP;                                                                 \
+    }                                                                                  \
+  } while (0)
+
+#define MSA_LAUNCH_CHECK() MSA_HIP(hipGetLastError())
+
+typedef uint16_t bf16_t;  // raw bf16 bits
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t x) { return __uint_as_float(((uint32_t)x) << 16); }
+
+// round-to-nearest-even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+}
+__device__ __forceinline__ float bf16lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// Monotone float -> uint32 map (larger float = larger key); key 0 is below every real number.
+__device__ __forceinline__ uint32_t f32_to_key(float f) {
+  uint32_t u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_to_f32(uint32_t k) {
+  uint32_t u = (k & 0x80000000u) ? (k & 0x7fffffffu) : ~k;
+  return __uint_as_float(u);
+}
+
+static inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
+static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+static inline size_t elem_bytes(int dtype) { return dtype == MSA_F32 ? 4 : 2; }
+
+constexpr int kHeadDim = 128;
+
+// Bank handle (bank.hip).  Tables live on both sides; per-layer tensors are borrowed.
+struct msa_bank {
+  int32_t n_layers;
+  int64_t C;
+  int32_t Hkv;
+  int32_t D;
+  int32_t dtype;
+  int64_t n_docs;
+  int32_t device;
+  int32_t* doc_chunk_off_dev;   // [n_docs+1]
+  int64_t* doc_global_id_dev;   // [n_docs]
+  int32_t* doc_chunk_off_host;  // [n_docs+1]
+  int64_t* doc_global_id_host;  // [n_docs]
+  const void** kr_dev;          // [n_layers]
+  const void** k_host;
+  const void** v_host;
+};

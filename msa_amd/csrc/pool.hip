@@ -1,0 +1,235 @@
+// Chunk-mean pooling of K / V / K_r over ragged documents (HBM-bound streaming kernel).
+//
+// One workgroup per (chunk, tensor).  A token row [H, 128] is covered by H*8 lanes; lane (h, j)
+// owns d in [8j, 8j+8) and [64+8j, 64+8j+8) — the two halves the half-split rotary pairs — so the
+// optional RoPE on K needs no cross-lane traffic.  256 threads cover R = 256 / (H*8) token rows
+// per step, accumulate in fp32 registers, and fold the R partial rows through LDS at the end.
+#include "common.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+
+struct PoolArgs {
+  const void* in[3];
+  void* out[3];
+  int rope[3];       // rotate this tensor while reading
+  int normalize[3];  // L2-normalise this tensor's pooled rows
+  int n_tensors;
+  int64_t T;
+  int32_t H;
+  const int32_t* chunk_start;
+  const int32_t* chunk_len;
+  const int32_t* chunk_doc;
+  const int32_t* doc_start;
+  const float* rope_cos;
+  const float* rope_sin;
+  int32_t rope_rows;
+};
+
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float (&x)[8]);
+
+template <>
+__device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float (&x)[8]) {
+  const uint4 w = *reinterpret_cast<const uint4*>(p);
+  x[0] = bf16lo(w.x); x[1] = bf16hi(w.x); x[2] = bf16lo(w.y); x[3] = bf16hi(w.y);
+  x[4] = bf16lo(w.z); x[5] = bf16hi(w.z); x[6] = bf16lo(w.w); x[7] = bf16hi(w.w);
+}
+template <>
+__device__ __forceinline__ void load8<float>(const float* p, float (&x)[8]) {
+  const float4 a = *reinterpret_cast<const float4*>(p);
+  const float4 b = *reinterpret_cast<const float4*>(p + 4);
+  x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+}
+
+template <typename T>
+__device__ __forceinline__ void store8(T* p, const float (&x)[8]);
+template <>
+__device__ __forceinline__ void store8<bf16_t>(bf16_t* p, const float (&x)[8]) {
+  uint4 w;
+  w.x = pack_bf16x2(x[0], x[1]); w.y = pack_bf16x2(x[2], x[3]);
+  w.z = pack_bf16x2(x[4], x[5]); w.w = pack_bf16x2(x[6], x[7]);
+  *reinterpret_cast<uint4*>(p) = w;
+}
+template <>
+__device__ __forceinline__ void store8<float>(float* p, const float (&x)[8]) {
+  *reinterpret_cast<float4*>(p) = make_float4(x[0], x[1], x[2], x[3]);
+  *reinterpret_cast<float4*>(p + 4) = make_float4(x[4], x[5], x[6], x[7]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kThreads) void pool_chunks_kernel(PoolArgs a) {
+  __shared__ float fold[kThreads * 16];
+
+  const int c = blockIdx.x;
+  const int slot = blockIdx.y;
+  const T* __restrict__ in = static_cast<const T*>(a.in[slot]);
+  T* __restrict__ out = static_cast<T*>(a.out[slot]);
+  const bool rope = a.rope[slot] != 0;
+
+  const int U = a.H * 8;          // lanes per token row
+  const int R = kThreads / U;     // token rows per step
+  const int tid = threadIdx.x;
+  const int r = tid / U, u = tid % U;
+  const bool active = r < R;
+  const int h = u >> 3, j = u & 7;
+  const int row_elems = a.H * kHeadDim;
+  const int col_lo = h * kHeadDim + 8 * j, col_hi = col_lo + 64;
+
+  const int32_t t0 = a.chunk_start[c];
+  const int32_t len = a.chunk_len[c];
+
+  float acc_lo[8], acc_hi[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc_lo[i] = acc_hi[i] = 0.f;
+
+  // rotary state of this lane's 8 frequencies at its current token, advanced by R positions per step
+  float rc[8], rs[8], sc[8], ss[8];
+  if (rope && active) {
+    const int32_t pos0 = t0 - a.doc_start[a.chunk_doc[c]] + r;
+    const int32_t p = min(pos0, a.rope_rows - 1), st = min(R, a.rope_rows - 1);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      rc[i] = a.rope_cos[(int64_t)p * 64 + 8 * j + i];
+      rs[i] = a.rope_sin[(int64_t)p * 64 + 8 * j + i];
+      sc[i] = a.rope_cos[(int64_t)st * 64 + 8 * j + i];
+      ss[i] = a.rope_sin[(int64_t)st * 64 + 8 * j + i];
+    }
+  }
+
+  if (active) {
+    constexpr int kUnroll = 4;
+    for (int base = 0; base < len; base += R * kUnroll) {
+      float xl[kUnroll][8], xh[kUnroll][8];
+      bool ok[kUnroll];
+#pragma unroll
+      for (int q = 0; q < kUnroll; ++q) {
+        const int off = base + q * R + r;
+        const int64_t t = (int64_t)t0 + off;
+        ok[q] = off < len && t < a.T;
+        if (ok[q]) {
+          const T* p = in + t * row_elems;
+          load8<T>(p + col_lo, xl[q]);
+          load8<T>(p + col_hi, xh[q]);
+        }
+      }
+#pragma unroll
+      for (int q = 0; q < kUnroll; ++q) {
+        if (rope) {
+          if (ok[q]) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              acc_lo[i] += xl[q][i] * rc[i] - xh[q][i] * rs[i];
+              acc_hi[i] += xh[q][i] * rc[i] + xl[q][i] * rs[i];
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {   // advance the angle by R positions
+            const float nc = rc[i] * sc[i] - rs[i] * ss[i];
+            rs[i] = rs[i] * sc[i] + rc[i] * ss[i];
+            rc[i] = nc;
+          }
+        } else if (ok[q]) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            acc_lo[i] += xl[q][i];
+            acc_hi[i] += xh[q][i];
+          }
+        }
+      }
+    }
+  }
+
+  // fold the R partial rows: fold[(r * U + u) * 16 + i]
+  if (active) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      fold[(r * U + u) * 16 + i] = acc_lo[i];
+      fold[(r * U + u) * 16 + 8 + i] = acc_hi[i];
+    }
+  }
+  __syncthreads();
+  if (tid < U) {
+    const float inv = 1.0f / (float)len;
+    float lo[8], hi[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lo[i] = hi[i] = 0.f;
+    for (int rr = 0; rr < R; ++rr) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        lo[i] += fold[(rr * U + tid) * 16 + i];
+        hi[i] += fold[(rr * U + tid) * 16 + 8 + i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { lo[i] *= inv; hi[i] *= inv; }
+    if (a.normalize[slot]) {
+      float ssq = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ssq += lo[i] * lo[i] + hi[i] * hi[i];
+      // the 8 lanes of one head are consecutive: butterfly over the low 3 lane bits
+      ssq += __shfl_xor(ssq, 1);
+      ssq += __shfl_xor(ssq, 2);
+      ssq += __shfl_xor(ssq, 4);
+      const float sc2 = 1.0f / fmaxf(sqrtf(ssq), 1e-12f);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) { lo[i] *= sc2; hi[i] *= sc2; }
+    }
+    T* o = out + (int64_t)c * row_elems;
+    store8<T>(o + col_lo, lo);
+    store8<T>(o + col_hi, hi);
+  }
+}
+
+}  // namespace
+
+extern "C" int msa_pool_chunks(const void* k, const void* v, const void* kr, int32_t dtype, int64_t T, int32_t H,
+                               int32_t D, const int32_t* chunk_start, const int32_t* chunk_len,
+                               const int32_t* chunk_doc, int64_t C, const int32_t* doc_start, const float* rope_cos,
+                               const float* rope_sin, int32_t rope_rows, int32_t max_doc_len, int32_t normalize_kr,
+                               void* k_out, void* v_out, void* kr_out, void* stream) {
+  MSA_REQUIRE(D == kHeadDim, "msa_pool_chunks: head dim %d unsupported (need %d)", D, kHeadDim);
+  MSA_REQUIRE(H > 0 && H <= 32 && (kThreads % (H * 8)) == 0, "msa_pool_chunks: H=%d must divide 32", H);
+  MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "msa_pool_chunks: bad dtype %d", dtype);
+  MSA_REQUIRE(T > 0 && T < (int64_t)1 << 31, "msa_pool_chunks: T=%lld out of range", (long long)T);
+  MSA_REQUIRE(C >= 0 && C < (int64_t)1 << 31, "msa_pool_chunks: C=%lld out of range", (long long)C);
+  MSA_REQUIRE(chunk_start && chunk_len && chunk_doc, "msa_pool_chunks: null chunk table");
+  MSA_REQUIRE((k == nullptr) == (k_out == nullptr) && (v == nullptr) == (v_out == nullptr) &&
+                  (kr == nullptr) == (kr_out == nullptr),
+              "msa_pool_chunks: each input needs its output and vice versa");
+  const bool rope = rope_cos != nullptr || rope_sin != nullptr;
+  if (rope) {
+    MSA_REQUIRE(rope_cos && rope_sin && doc_start, "msa_pool_chunks: rotary needs cos, sin and doc_start");
+    MSA_REQUIRE(k != nullptr, "msa_pool_chunks: rotary requested without K");
+    MSA_REQUIRE(max_doc_len > 0 && max_doc_len <= rope_rows,
+                "msa_pool_chunks: max_doc_len=%d exceeds the rotary table (%d rows)", max_doc_len, rope_rows);
+    MSA_REQUIRE(rope_rows > kThreads / (H * 8), "msa_pool_chunks: rotary table too short (%d rows)", rope_rows);
+  }
+  if (C == 0) return MSA_OK;
+
+  PoolArgs a{};
+  int n = 0;
+  auto add = [&](const void* in, void* out, int rp, int nm) {
+    if (!in) return;
+    a.in[n] = in; a.out[n] = out; a.rope[n] = rp; a.normalize[n] = nm; ++n;
+  };
+  add(k, k_out, rope ? 1 : 0, 0);
+  add(v, v_out, 0, 0);
+  add(kr, kr_out, 0, normalize_kr ? 1 : 0);
+  MSA_REQUIRE(n > 0, "msa_pool_chunks: nothing to pool");
+  for (int i = 0; i < n; ++i)
+    MSA_REQUIRE(((uintptr_t)a.in[i] & 15) == 0 && ((uintptr_t)a.out[i] & 15) == 0,
+                "msa_pool_chunks: tensors must be 16-byte aligned");
+  a.n_tensors = n; a.T = T; a.H = H;
+  a.chunk_start = chunk_start; a.chunk_len = chunk_len; a.chunk_doc = chunk_doc; a.doc_start = doc_start;
+  a.rope_cos = rope_cos; a.rope_sin = rope_sin; a.rope_rows = rope_rows;
+
+  dim3 grid((unsigned)C, (unsigned)n);
+  if (dtype == MSA_BF16)
+    pool_chunks_kernel<bf16_t><<<grid, kThreads, 0, as_stream(stream)>>>(a);
+  else
+    pool_chunks_kernel<float><<<grid, kThreads, 0, as_stream(stream)>>>(a);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}

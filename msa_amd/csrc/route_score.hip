@@ -1,0 +1,378 @@
+// Router scoring: pre-summed query tiles against the HBM-resident pooled K_r bank.
+//
+// score[b, c] = max over scored tokens t of (scale / Hq) * sum_h q'[b,t,h] . kr[c, h / G]
+//             = max_t (scale / Hq) * Qs[b,t,:] . kr[c,:]        with Qs[b,t,g,:] = sum_{h in g} q'[b,t,h,:]
+// (the mean over heads is linear, so the G query heads of one KV group are summed first).  That is
+// an NT GEMM  [B*S_pad, Hkv*D] x [C, Hkv*D]^T  whose output is never written: each 32-row MFMA
+// block is reduced to a column max over its scored rows in registers and merged into
+// chunk_key[B, C] (order-preserving uint32 keys) with atomicMax.
+#include <algorithm>
+
+#include "common.h"
+
+namespace {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
+
+// ------------------------------------------------------------------------------------------
+// Prologue: normalise (cosine mode), sum the G heads of each KV group, cast, build row masks.
+// One workgroup of Hkv*16 lanes per (b, padded token); lane (g, j) owns 8 contiguous d of group g.
+// ------------------------------------------------------------------------------------------
+template <typename TIn, typename TOut>
+__global__ void presum_queries_kernel(const TIn* __restrict__ q, const uint8_t* __restrict__ qmask, int32_t B,
+                                      int32_t S, int32_t S_pad, int32_t Hq, int32_t Hkv, int32_t normalize,
+                                      TOut* __restrict__ qs, uint32_t* __restrict__ row_bits) {
+  const int row = blockIdx.x;              // b * S_pad + s
+  const int b = row / S_pad, s = row % S_pad;
+  const int G = Hq / Hkv;
+  const int g = threadIdx.x >> 4, j = threadIdx.x & 15;
+  const bool valid = s < S && (qmask == nullptr || qmask[(int64_t)b * S + s] != 0);
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  if (valid) {
+    for (int hh = 0; hh < G; ++hh) {
+      const TIn* p = q + (((int64_t)b * S + s) * Hq + (g * G + hh)) * kHeadDim + 8 * j;
+      float x[8];
+      if constexpr (sizeof(TIn) == 2) {
+        const uint4 w = *reinterpret_cast<const uint4*>(p);
+        x[0] = bf16lo(w.x); x[1] = bf16hi(w.x); x[2] = bf16lo(w.y); x[3] = bf16hi(w.y);
+        x[4] = bf16lo(w.z); x[5] = bf16hi(w.z); x[6] = bf16lo(w.w); x[7] = bf16hi(w.w);
+      } else {
+        const float4 u = *reinterpret_cast<const float4*>(p);
+        const float4 v = *reinterpret_cast<const float4*>(p + 4);
+        x[0] = u.x; x[1] = u.y; x[2] = u.z; x[3] = u.w; x[4] = v.x; x[5] = v.y; x[6] = v.z; x[7] = v.w;
+      }
+      float inv = 1.f;
+      if (normalize) {
+        float ssq = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ssq += x[i] * x[i];
+        ssq += __shfl_xor(ssq, 1); ssq += __shfl_xor(ssq, 2);     // the 16 lanes of one group
+        ssq += __shfl_xor(ssq, 4); ssq += __shfl_xor(ssq, 8);
+        inv = 1.0f / fmaxf(sqrtf(ssq), 1e-12f);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += x[i] * inv;
+    }
+  }
+  TOut* o = qs + ((int64_t)row * Hkv + g) * kHeadDim + 8 * j;
+  if constexpr (sizeof(TOut) == 2) {
+    uint4 w;
+    w.x = pack_bf16x2(acc[0], acc[1]); w.y = pack_bf16x2(acc[2], acc[3]);
+    w.z = pack_bf16x2(acc[4], acc[5]); w.w = pack_bf16x2(acc[6], acc[7]);
+    *reinterpret_cast<uint4*>(o) = w;
+  } else {
+    *reinterpret_cast<float4*>(o) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    *reinterpret_cast<float4*>(o + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+  }
+  if (threadIdx.x == 0 && valid) atomicOr(&row_bits[row >> 5], 1u << (row & 31));
+}
+
+__global__ void fill_u32_kernel(uint32_t* __restrict__ p, int64_t n, uint32_t v) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = v;
+}
+
+// ------------------------------------------------------------------------------------------
+// MFMA operand traits.  LDS rows hold 128 bytes of K (64 bf16 or 32 fp32) plus 16 bytes of pad,
+// which makes the 16-byte / 4-byte operand reads of a 32-row block bank-conflict free.
+// ------------------------------------------------------------------------------------------
+constexpr int kRowBytes = 128;
+constexpr int kRowStride = kRowBytes + 16;
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<bf16_t> {
+  static constexpr int kSub = 4;   // 32x32x16 steps per 64-element K tile
+  static __device__ __forceinline__ floatx16_t run(const char* a, const char* b, int sub, int half, floatx16_t c) {
+    const bf16x8_t fa = *reinterpret_cast<const bf16x8_t*>(a + sub * 32 + half * 16);
+    const bf16x8_t fb = *reinterpret_cast<const bf16x8_t*>(b + sub * 32 + half * 16);
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mma<float> {
+  static constexpr int kSub = 16;  // 32x32x2 steps per 32-element K tile
+  static __device__ __forceinline__ floatx16_t run(const char* a, const char* b, int sub, int half, floatx16_t c) {
+    const float fa = *reinterpret_cast<const float*>(a + sub * 8 + half * 4);
+    const float fb = *reinterpret_cast<const float*>(b + sub * 8 + half * 4);
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb, c, 0, 0, 0);
+  }
+};
+
+// Workgroup tile BM x BN, WAVES_M x WAVES_N wavefronts, each owning TM x TN blocks of 32 x 32.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
+    const T* __restrict__ qs,            // [M_rows, K]  pre-summed queries, M_rows = B * S_pad
+    const T* __restrict__ kr,            // [C, K]
+    const uint32_t* __restrict__ row_bits,  // [ceil(M_alloc / 32)] scored-row bitmask
+    uint32_t* __restrict__ chunk_key,    // [B, C]
+    int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t tiles_m, int32_t tiles_n) {
+  constexpr int kThreads = WAVES_M * WAVES_N * 64;
+  constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
+  constexpr int TM = WM / 32, TN = WN / 32;
+  constexpr int kVecA = BM * 8 / kThreads, kVecB = BN * 8 / kThreads;   // 16-byte vectors per thread per tile
+  static_assert(BM * 8 % kThreads == 0 && BN * 8 % kThreads == 0, "tile/threads mismatch");
+
+  extern __shared__ __align__(16) char lds[];
+  constexpr int kBufBytes = (BM + BN) * kRowStride;   // [A tile | B tile] per buffer, two buffers
+
+  // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so give each XCD one
+  // contiguous run of tiles with the M tiles of a K_r tile adjacent; K_r then comes from HBM once
+  // per XCD and the other M tiles hit that XCD's L2.
+  const int total = tiles_m * tiles_n;
+  const int per_xcd = (total + 7) / 8;
+  const int logical = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (logical >= total) return;
+  const int tile_n = logical / tiles_m, tile_m = logical % tiles_m;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int half = lane >> 5, l32 = lane & 31;
+
+  const int64_t row_bytes_g = (int64_t)K * sizeof(T);
+  const char* ga = reinterpret_cast<const char*>(qs);
+  const char* gb = reinterpret_cast<const char*>(kr);
+
+  uint4 ra[kVecA], rb[kVecB];
+  auto load_tile = [&](int kt) {
+#pragma unroll
+    for (int i = 0; i < kVecA; ++i) {
+      const int v = tid + i * kThreads, r = v >> 3, c = v & 7;
+      const int m = m0 + r;
+      ra[i] = m < M_rows ? *reinterpret_cast<const uint4*>(ga + m * row_bytes_g + (int64_t)kt * kRowBytes + c * 16)
+                         : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < kVecB; ++i) {
+      const int v = tid + i * kThreads, r = v >> 3, c = v & 7;
+      const int n = n0 + r;
+      rb[i] = n < C ? *reinterpret_cast<const uint4*>(gb + n * row_bytes_g + (int64_t)kt * kRowBytes + c * 16)
+                    : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store_tile = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < kVecA; ++i) {
+      const int v = tid + i * kThreads, r = v >> 3, c = v & 7;
+      *reinterpret_cast<uint4*>(lds + buf * kBufBytes + r * kRowStride + c * 16) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < kVecB; ++i) {
+      const int v = tid + i * kThreads, r = v >> 3, c = v & 7;
+      *reinterpret_cast<uint4*>(lds + buf * kBufBytes + (BM + r) * kRowStride + c * 16) = rb[i];
+    }
+  };
+
+  floatx16_t acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+  const int k_tiles = (int)(row_bytes_g / kRowBytes);
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < k_tiles) load_tile(kt + 1);
+    const char* pa = lds + buf * kBufBytes + (wm * WM + l32) * kRowStride;
+    const char* pb = lds + buf * kBufBytes + (BM + wn * WN + l32) * kRowStride;
+#pragma unroll
+    for (int sub = 0; sub < Mma<T>::kSub; ++sub) {
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = Mma<T>::run(pa + i * 32 * kRowStride, pb + j * 32 * kRowStride, sub, half, acc[i][j]);
+    }
+    if (kt + 1 < k_tiles) {
+      store_tile(buf ^ 1);   // the other buffer was last read one iteration ago, behind the barrier below
+      __syncthreads();
+    }
+  }
+
+  // Epilogue.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of its 32x32 block.
+#pragma unroll
+  for (int j = 0; j < TN; ++j) {
+    const int n = n0 + wn * WN + j * 32 + l32;
+    float run = -INFINITY;
+    bool any = false;
+    int run_q = -1;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int blk = (m0 + wm * WM + i * 32) >> 5;      // global 32-row block index
+      const int qid = blk / blocks_per_query;
+      const uint32_t bits = row_bits[blk];               // 0 for blocks past M_rows (buffer is padded)
+      if (qid != run_q) {
+        if (any && half == 0 && n < C) atomicMax(&chunk_key[(int64_t)run_q * C + n], f32_to_key(run));
+        run = -INFINITY; any = false; run_q = qid;
+      }
+      if (bits != 0) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int r = 8 * (e >> 2) + 4 * half + (e & 3);
+          if (bits & (1u << r)) mx = fmaxf(mx, acc[i][j][e]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        run = fmaxf(run, mx);
+        any = true;
+      }
+    }
+    if (any && half == 0 && n < C) atomicMax(&chunk_key[(int64_t)run_q * C + n], f32_to_key(run));
+  }
+}
+
+// chunk_key -> fp32 scores (times scale / Hq); key 0 (query without a scored token) -> -inf.
+__global__ void decode_scores_kernel(const uint32_t* __restrict__ key, int64_t n, float mul,
+                                     float* __restrict__ out) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const uint32_t k = key[i];
+    out[i] = k == 0 ? -INFINITY : key_to_f32(k) * mul;
+  }
+}
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
+int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* chunk_key, int32_t M_rows,
+                int32_t C, int32_t K, int32_t blocks_per_query, hipStream_t st) {
+  const int tiles_m = (M_rows + BM - 1) / BM, tiles_n = (C + BN - 1) / BN;
+  const int total = tiles_m * tiles_n;
+  const int grid = (total + 7) / 8 * 8;
+  const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
+  auto kern = score_gemm_kernel<T, BM, BN, WAVES_M, WAVES_N>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    MSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)lds));
+    attr_set = true;
+  }
+  kern<<<grid, WAVES_M * WAVES_N * 64, lds, st>>>(static_cast<const T*>(qs), static_cast<const T*>(kr), row_bits,
+                                                  chunk_key, M_rows, C, K, blocks_per_query, tiles_m, tiles_n);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
+
+}  // namespace
+
+// ------------------------------------------------------------------------------------------
+// Workspace layout (shared with topk.hip through route_internal.h)
+// ------------------------------------------------------------------------------------------
+#include "route_internal.h"
+
+RouteWorkspace route_workspace_layout(int32_t B, int32_t S, int32_t Hkv, int32_t D, int64_t C, int64_t n_docs,
+                                      int32_t topk, int32_t dtype) {
+  RouteWorkspace w{};
+  w.S_pad = (S + 31) / 32 * 32;
+  w.M_rows = B * w.S_pad;
+  const int64_t m_alloc = ((int64_t)w.M_rows + 255) / 256 * 256;   // every M tile may read whole mask words
+  size_t off = 0;
+  w.off_qs = off;       off = align_up(off + (size_t)w.M_rows * Hkv * D * elem_bytes(dtype), 256);
+  w.off_row_bits = off; off = align_up(off + (size_t)(m_alloc / 32) * sizeof(uint32_t), 256);
+  w.off_chunk_key = off; off = align_up(off + (size_t)B * C * sizeof(uint32_t), 256);
+  w.topk_blocks = topk_blocks_for(n_docs);
+  w.off_cand = off;     off = align_up(off + (size_t)B * w.topk_blocks * kTopkMax * sizeof(uint64_t), 256);
+  w.bytes = off;
+  return w;
+}
+
+extern "C" size_t msa_route_workspace_bytes(int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D, int64_t C,
+                                            int64_t n_docs, int32_t topk) {
+  (void)Hq;
+  if (B <= 0 || S <= 0 || Hkv <= 0 || D <= 0 || C <= 0 || n_docs <= 0) return 0;
+  // sized for fp32 queries so one workspace serves both dtypes
+  return route_workspace_layout(B, S, Hkv, D, C, n_docs, topk, MSA_F32).bytes;
+}
+
+int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
+                         int32_t S, int32_t Hq, int32_t mode, float scale, void* workspace, size_t workspace_bytes,
+                         hipStream_t st, RouteWorkspace* layout_out, float* mul_out, const char* who) {
+  MSA_REQUIRE(bank != nullptr, "%s: null bank", who);
+  MSA_REQUIRE(layer >= 0 && layer < bank->n_layers, "%s: layer %d out of range", who, layer);
+  if (bank->kr_dev[layer] == nullptr) {
+    msa_set_error("%s: layer %d has no K_r set", who, layer);
+    return MSA_ESTATE;
+  }
+  MSA_REQUIRE(q != nullptr && workspace != nullptr, "%s: null pointer", who);
+  MSA_REQUIRE(B > 0 && B <= 4096 && S > 0 && S <= 65536, "%s: B=%d S=%d out of range", who, B, S);
+  MSA_REQUIRE(Hq > 0 && Hq % bank->Hkv == 0, "%s: Hq=%d not a multiple of Hkv=%d", who, Hq, bank->Hkv);
+  MSA_REQUIRE(bank->Hkv <= 16, "%s: Hkv=%d unsupported (max 16)", who, bank->Hkv);
+  MSA_REQUIRE(mode == MSA_MODE_COSINE || mode == MSA_MODE_SCALED_DOT, "%s: bad mode %d", who, mode);
+  MSA_REQUIRE(((uintptr_t)q & 15) == 0 && ((uintptr_t)workspace & 255) == 0, "%s: q / workspace misaligned", who);
+  const float sc = mode == MSA_MODE_COSINE ? 1.0f : scale;
+  MSA_REQUIRE(sc > 0.f && sc < INFINITY, "%s: scale must be positive and finite", who);
+  MSA_REQUIRE((int64_t)B * ((S + 31) / 32 * 32) < (int64_t)1 << 24, "%s: too many query rows", who);
+
+  const RouteWorkspace w = route_workspace_layout(B, S, bank->Hkv, bank->D, bank->C, bank->n_docs, kTopkMax, bank->dtype);
+  if (w.bytes > workspace_bytes) {
+    msa_set_error("%s: workspace of %zu bytes, need %zu", who, workspace_bytes, w.bytes);
+    return MSA_ESIZE;
+  }
+  char* ws = static_cast<char*>(workspace);
+  void* qs = ws + w.off_qs;
+  uint32_t* row_bits = reinterpret_cast<uint32_t*>(ws + w.off_row_bits);
+  uint32_t* chunk_key = reinterpret_cast<uint32_t*>(ws + w.off_chunk_key);
+  const int64_t m_alloc = ((int64_t)w.M_rows + 255) / 256 * 256;
+
+  // row masks and chunk keys start at zero (both live in one contiguous span of the workspace)
+  const int64_t zero_words = (int64_t)((w.off_cand - w.off_row_bits) / sizeof(uint32_t));
+  (void)m_alloc;
+  fill_u32_kernel<<<(int)std::min<int64_t>((zero_words + 1023) / 1024, 4096), 256, 0, st>>>(row_bits, zero_words, 0u);
+  MSA_LAUNCH_CHECK();
+
+  const int normalize = mode == MSA_MODE_COSINE ? 1 : 0;
+  const int pthreads = bank->Hkv * 16;
+  if (bank->dtype == MSA_BF16)
+    presum_queries_kernel<bf16_t, bf16_t><<<w.M_rows, pthreads, 0, st>>>(
+        static_cast<const bf16_t*>(q), qmask_u8, B, S, w.S_pad, Hq, bank->Hkv, normalize, static_cast<bf16_t*>(qs),
+        row_bits);
+  else
+    presum_queries_kernel<float, float><<<w.M_rows, pthreads, 0, st>>>(
+        static_cast<const float*>(q), qmask_u8, B, S, w.S_pad, Hq, bank->Hkv, normalize, static_cast<float*>(qs),
+        row_bits);
+  MSA_LAUNCH_CHECK();
+
+  const int32_t K = bank->Hkv * bank->D;
+  const int32_t bpq = w.S_pad / 32;
+  int rc;
+  if (bank->dtype == MSA_BF16) {
+    if (w.M_rows <= 128)
+      rc = launch_gemm<bf16_t, 128, 128, 2, 2>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C,
+                                              K, bpq, st);
+    else
+      rc = launch_gemm<bf16_t, 256, 128, 2, 2>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C,
+                                              K, bpq, st);
+  } else {
+    rc = launch_gemm<float, 128, 128, 2, 2>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C, K,
+                                            bpq, st);
+  }
+  if (rc != MSA_OK) return rc;
+  *layout_out = w;
+  *mul_out = sc / (float)Hq;
+  return MSA_OK;
+}
+
+extern "C" int msa_chunk_scores(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
+                                int32_t S, int32_t Hq, int32_t mode, float scale, float* chunk_scores,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+  MSA_REQUIRE(chunk_scores != nullptr, "msa_chunk_scores: null output");
+  RouteWorkspace w;
+  float mul;
+  hipStream_t st = as_stream(stream);
+  int rc = route_scores_to_keys(bank, layer, q, qmask_u8, B, S, Hq, mode, scale, workspace, workspace_bytes, st, &w,
+                                &mul, "msa_chunk_scores");
+  if (rc != MSA_OK) return rc;
+  const int64_t n = (int64_t)B * bank->C;
+  const uint32_t* key = reinterpret_cast<const uint32_t*>(static_cast<char*>(workspace) + w.off_chunk_key);
+  decode_scores_kernel<<<(int)std::min<int64_t>((n + 255) / 256, 8192), 256, 0, st>>>(key, n, mul, chunk_scores);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}

@@ -1,0 +1,271 @@
+"""Torch-tensor front end of the C ABI (``include/msa_amd.h``).
+
+PyTorch is used here only to own device / pinned memory and to name streams; every computation
+below happens in the HIP library.  All functions enqueue on the current torch stream unless a
+stream is given, and raise :class:`msa_amd._lib.MsaError` on any failure.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import MODE_COSINE, MODE_SCALED_DOT, check, dtype_code, ptr
+
+MODES = {"cosine": MODE_COSINE, "scaled_dot": MODE_SCALED_DOT}
+
+
+def _stream(stream: Optional[torch.cuda.Stream] = None) -> int:
+    return (stream or torch.cuda.current_stream()).cuda_stream
+
+
+def _need_cuda(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise ValueError("expected a device tensor (the HIP path has no CPU fallback)")
+        if t is not None and not t.is_contiguous():
+            raise ValueError("expected a contiguous tensor")
+
+
+# ------------------------------------------------------------------------------ chunk table
+@dataclass
+class ChunkTable:
+    """Device-side chunking of one packed block (all int32 tensors)."""
+    doc_start: torch.Tensor       # [n_docs + 1] token offsets
+    doc_chunk_off: torch.Tensor   # [n_docs + 1]
+    chunk_start: torch.Tensor     # [C]
+    chunk_len: torch.Tensor       # [C]
+    chunk_doc: torch.Tensor       # [C] 0-based
+    n_chunks: torch.Tensor        # [1] int64, written by the kernel
+    P: int
+    max_doc_len: int
+
+    @property
+    def C(self) -> int:
+        return self.chunk_start.numel()
+
+
+def chunk_table(doc_lens: Sequence[int], P: int, first_token: int = 0, device="cuda") -> ChunkTable:
+    """Builds the chunk table on the device from host-side document lengths (the host only sizes
+    the outputs: ``C = sum(ceil(len / P))``, as src/prefill.py:225 does)."""
+    lib = _lib.load()
+    lens = [int(x) for x in doc_lens]
+    if not lens or min(lens) <= 0:
+        raise ValueError("every document needs at least one token")
+    n_chunks = sum((n + P - 1) // P for n in lens)
+    starts = torch.tensor([first_token] + lens, dtype=torch.int64).cumsum(0).to(torch.int32)
+    doc_start = starts.to(device)
+    n_docs = len(lens)
+    i32 = dict(dtype=torch.int32, device=device)
+    t = ChunkTable(doc_start, torch.empty(n_docs + 1, **i32), torch.empty(n_chunks, **i32),
+                   torch.empty(n_chunks, **i32), torch.empty(n_chunks, **i32),
+                   torch.zeros(1, dtype=torch.int64, device=device), P, max(lens))
+    check(lib.msa_chunk_table(ptr(t.doc_start), n_docs, P, n_chunks, ptr(t.doc_chunk_off), ptr(t.chunk_start),
+                              ptr(t.chunk_len), ptr(t.chunk_doc), ptr(t.n_chunks), _stream()), "msa_chunk_table")
+    return t
+
+
+# ------------------------------------------------------------------------------ pooling
+def rope_tables(n_rows: int, D: int, theta: float, device="cuda") -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp32 ``[n_rows, D/2]`` cos / sin tables, computed the way Qwen3RotaryEmbedding does (fp32
+    inv_freq, fp32 angles)."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, D, 2, dtype=torch.int64).float() / D))
+    ang = torch.arange(n_rows, dtype=torch.float32)[:, None] * inv_freq[None, :]
+    return ang.cos().contiguous().to(device), ang.sin().contiguous().to(device)
+
+
+def pool_chunks(k: Optional[torch.Tensor], v: Optional[torch.Tensor], kr: Optional[torch.Tensor], table: ChunkTable,
+                rope: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, normalize_kr: bool = False):
+    """Chunk means of token-major ``[T, H, D]`` tensors -> chunk-major ``[C, H, D]`` (same dtype).
+    ``rope=(cos, sin)`` rotates K at per-document positions while reading it."""
+    lib = _lib.load()
+    ref = next(t for t in (k, v, kr) if t is not None)
+    _need_cuda(k, v, kr)
+    T, H, D = ref.shape
+    for t in (k, v, kr):
+        if t is not None and (t.shape != ref.shape or t.dtype != ref.dtype):
+            raise ValueError("K, V and K_r must share shape and dtype")
+    outs = [None if t is None else torch.empty((table.C, H, D), dtype=ref.dtype, device=ref.device) for t in (k, v, kr)]
+    cos, sin = rope if rope is not None else (None, None)
+    if rope is not None:
+        _need_cuda(cos, sin)
+        if cos.dtype != torch.float32 or cos.shape != sin.shape or cos.shape[1] != D // 2:
+            raise ValueError("rotary tables must be fp32 [rows, D/2]")
+    check(lib.msa_pool_chunks(ptr(k), ptr(v), ptr(kr), dtype_code(ref.dtype), T, H, D, ptr(table.chunk_start),
+                              ptr(table.chunk_len), ptr(table.chunk_doc), table.C, ptr(table.doc_start), ptr(cos),
+                              ptr(sin), 0 if cos is None else cos.shape[0], table.max_doc_len, int(normalize_kr),
+                              ptr(outs[0]), ptr(outs[1]), ptr(outs[2]), _stream()), "msa_pool_chunks")
+    return tuple(outs)
+
+
+# ------------------------------------------------------------------------------ bank + routing
+class Bank:
+    """Owner of an ``msa_bank`` handle plus the tensors it borrows."""
+
+    def __init__(self, n_layers: int, doc_chunk_off: Sequence[int], doc_global_id: Sequence[int], Hkv: int, D: int,
+                 dtype: torch.dtype):
+        lib = _lib.load()
+        self.off_host = torch.as_tensor(doc_chunk_off, dtype=torch.int32).contiguous()
+        self.gid_host = torch.as_tensor(doc_global_id, dtype=torch.int64).contiguous()
+        self.n_docs = self.gid_host.numel()
+        if self.off_host.numel() != self.n_docs + 1:
+            raise ValueError("doc_chunk_off must have n_docs + 1 entries")
+        self.C = int(self.off_host[-1])
+        self.n_layers, self.Hkv, self.D, self.dtype = n_layers, Hkv, D, dtype
+        self._keep = {}
+        self._ws: Optional[torch.Tensor] = None
+        h = C.c_void_p()
+        check(lib.msa_bank_create(C.byref(h), n_layers, self.C, Hkv, D, dtype_code(dtype), ptr(self.off_host),
+                                  ptr(self.gid_host), self.n_docs), "msa_bank_create")
+        self.handle = h
+
+    def set_layer(self, layer: int, kr: torch.Tensor, k_host: Optional[torch.Tensor] = None,
+                  v_host: Optional[torch.Tensor] = None):
+        want = (self.C, self.Hkv, self.D)
+        _need_cuda(kr)
+        for t in (kr, k_host, v_host):
+            if t is not None and (tuple(t.shape) != want or t.dtype != self.dtype or not t.is_contiguous()):
+                raise ValueError(f"bank tensors must be contiguous {want} {self.dtype}")
+        for t in (k_host, v_host):
+            if t is not None and (t.is_cuda or not t.is_pinned()):
+                raise ValueError("pooled K / V must live in pinned host memory")
+        check(_lib.load().msa_bank_set_layer(self.handle, layer, ptr(kr), ptr(k_host), ptr(v_host)),
+              "msa_bank_set_layer")
+        self._keep[layer] = (kr, k_host, v_host)
+
+    def workspace(self, B: int, S: int, Hq: int, topk: int, device) -> torch.Tensor:
+        need = _lib.load().msa_route_workspace_bytes(B, S, Hq, self.Hkv, self.D, self.C, self.n_docs, topk)
+        if self._ws is None or self._ws.numel() < need or self._ws.device != torch.device(device):
+            self._ws = torch.empty(need, dtype=torch.uint8, device=device)
+        return self._ws
+
+    def close(self):
+        if getattr(self, "handle", None):
+            _lib.load().msa_bank_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def _route_args(bank: Bank, q: torch.Tensor, qmask: Optional[torch.Tensor], mode: str):
+    _need_cuda(q, qmask)
+    if q.dim() != 4 or q.shape[3] != bank.D or q.dtype != bank.dtype:
+        raise ValueError(f"q must be [B, S, Hq, {bank.D}] {bank.dtype}")
+    B, S, Hq, _ = q.shape
+    if qmask is not None:
+        if tuple(qmask.shape) != (B, S):
+            raise ValueError("qmask must be [B, S]")
+        qmask = qmask.to(torch.uint8).contiguous()
+    if mode not in MODES:
+        raise NotImplementedError(f"unsupported scoring mode {mode!r}")
+    return B, S, Hq, qmask
+
+
+def chunk_scores(bank: Bank, layer: int, q: torch.Tensor, qmask: Optional[torch.Tensor] = None, mode: str = "cosine",
+                 scale: float = 1.0) -> torch.Tensor:
+    """fp32 ``[B, C]`` chunk scores (mean over heads, max over scored tokens)."""
+    B, S, Hq, qm = _route_args(bank, q, qmask, mode)
+    ws = bank.workspace(B, S, Hq, 16, q.device)
+    out = torch.empty((B, bank.C), dtype=torch.float32, device=q.device)
+    check(_lib.load().msa_chunk_scores(bank.handle, layer, ptr(q), ptr(qm), B, S, Hq, MODES[mode], scale, ptr(out),
+                                       ptr(ws), ws.numel(), _stream()), "msa_chunk_scores")
+    return out
+
+
+def route_topk(bank: Bank, layer: int, q: torch.Tensor, qmask: Optional[torch.Tensor] = None, mode: str = "cosine",
+               scale: float = 1.0, topk: int = 16):
+    """``(scores [B, k] fp32, doc [B, k] int32 0-based, doc_global [B, k] int64)``."""
+    B, S, Hq, qm = _route_args(bank, q, qmask, mode)
+    ws = bank.workspace(B, S, Hq, topk, q.device)
+    scores = torch.empty((B, topk), dtype=torch.float32, device=q.device)
+    doc = torch.empty((B, topk), dtype=torch.int32, device=q.device)
+    gid = torch.empty((B, topk), dtype=torch.int64, device=q.device)
+    check(_lib.load().msa_route_topk(bank.handle, layer, ptr(q), ptr(qm), B, S, Hq, MODES[mode], scale, topk,
+                                     ptr(scores), ptr(doc), ptr(gid), ptr(ws), ws.numel(), _stream()),
+          "msa_route_topk")
+    return scores, doc, gid
+
+
+# ------------------------------------------------------------------------------ gather
+def gather_kv(bank: Bank, layer: int, doc_sel_host: torch.Tensor, device, stream: Optional[torch.cuda.Stream] = None):
+    """Copies the selected documents' pooled K / V rows from pinned host memory on ``stream``.
+    Returns ``(K [sum, Hkv, D], V, cu_sel int64 [B + 1] (host))``; the copies are merely enqueued."""
+    lib = _lib.load()
+    sel = doc_sel_host.to(torch.int32).contiguous()
+    if sel.is_cuda or sel.dim() != 2:
+        raise ValueError("doc_sel_host must be a host tensor [B, k]")
+    B, k = sel.shape
+    cu = torch.empty(B + 1, dtype=torch.int64)
+    check(lib.msa_gather_plan(bank.handle, ptr(sel), B, k, ptr(cu)), "msa_gather_plan")
+    total = int(cu[-1])
+    with torch.cuda.stream(stream) if stream is not None else _null_ctx():
+        k_out = torch.empty((total, bank.Hkv, bank.D), dtype=bank.dtype, device=device)
+        v_out = torch.empty_like(k_out)
+    check(lib.msa_gather_kv(bank.handle, layer, ptr(sel), B, k, ptr(k_out), ptr(v_out), total, _stream(stream)),
+          "msa_gather_kv")
+    return k_out, v_out, cu
+
+
+class _null_ctx:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *a):
+        return False
+
+
+# ------------------------------------------------------------------------------ cache + attention
+def assemble_context(prefix_k, prefix_v, mem_k, mem_v, cu_sel, local_k, local_v, cu_local, B: int, Lcap: int):
+    """Builds ``kcache / vcache [B, Lcap, Hkv, D]`` and ``kv_len [B]`` from
+    ``[prefix | memory rows of b | local rows of b]``."""
+    ref = next(t for t in (prefix_k, mem_k, local_k) if t is not None)
+    Hkv, D = ref.shape[-2], ref.shape[-1]
+    _need_cuda(prefix_k, prefix_v, mem_k, mem_v, cu_sel, local_k, local_v, cu_local)
+    kc = torch.empty((B, Lcap, Hkv, D), dtype=ref.dtype, device=ref.device)
+    vc = torch.empty_like(kc)
+    kv_len = torch.empty(B, dtype=torch.int32, device=ref.device)
+    n_prefix = 0 if prefix_k is None else prefix_k.shape[0]
+    check(_lib.load().msa_assemble_context(ptr(prefix_k), ptr(prefix_v), n_prefix, ptr(mem_k), ptr(mem_v),
+                                           ptr(cu_sel), ptr(local_k), ptr(local_v), ptr(cu_local), B, Hkv, D,
+                                           dtype_code(ref.dtype), ptr(kc), ptr(vc), Lcap, ptr(kv_len), _stream()),
+          "msa_assemble_context")
+    return kc, vc, kv_len
+
+
+def cache_append(k_new, v_new, kcache, vcache, kv_len):
+    """Writes one ``[B, Hkv, D]`` row per sample at ``kv_len[b]`` and increments it, in place."""
+    _need_cuda(k_new, v_new, kcache, vcache, kv_len)
+    B, Lcap, Hkv, D = kcache.shape
+    check(_lib.load().msa_cache_append(ptr(k_new), ptr(v_new), B, Hkv, D, dtype_code(kcache.dtype), ptr(kcache),
+                                       ptr(vcache), Lcap, ptr(kv_len), _stream()), "msa_cache_append")
+
+
+_attn_ws = {}
+
+
+def sparse_attn(q, k, v, kv_off, kv_len, max_kv: int, cu_q=None, max_sq: int = 1, scale: Optional[float] = None,
+                causal: bool = True):
+    """GQA attention of ``q [total_q, Hq, D]`` over per-sample key ranges of ``k / v [rows, Hkv, D]``."""
+    _need_cuda(q, k, v, kv_off, kv_len, cu_q)
+    total_q, Hq, D = q.shape
+    Hkv = k.shape[-2]
+    B = kv_len.numel()
+    if kv_off.dtype != torch.int64 or kv_len.dtype != torch.int32 or (cu_q is not None and cu_q.dtype != torch.int32):
+        raise ValueError("kv_off int64, kv_len / cu_q int32")
+    lib = _lib.load()
+    need = lib.msa_attn_workspace_bytes(total_q, Hq, D, max_kv)
+    ws = _attn_ws.get(q.device)
+    if ws is None or ws.numel() < need:
+        ws = _attn_ws[q.device] = torch.empty(need, dtype=torch.uint8, device=q.device)
+    out = torch.empty_like(q)
+    check(lib.msa_sparse_attn(ptr(q), ptr(cu_q), ptr(k), ptr(v), ptr(kv_off), ptr(kv_len), B, total_q, max_sq, max_kv,
+                              Hq, Hkv, D, dtype_code(q.dtype), D ** -0.5 if scale is None else scale, int(causal),
+                              ptr(out), ptr(ws), ws.numel(), _stream()), "msa_sparse_attn")
+    return out

@@ -1,0 +1,74 @@
+"""CPU-only checks of the C-ABI library: it loads, exports every symbol the header declares, the
+ctypes table matches the header, and argument validation fails loudly without touching a GPU."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from msa_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "msa_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(msa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_exported_and_bound():
+    lib = _lib.load()
+    names = _declared()
+    assert len(names) >= 16
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in the header but not exported"
+    assert sorted(_lib.SIGNATURES) == names
+    assert lib.msa_abi_version() == 1
+
+
+def test_header_arity_matches_ctypes_table():
+    text = open(os.path.join(ROOT, "include", "msa_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    for name, (_, args) in _lib.SIGNATURES.items():
+        m = re.search(r"\b%s\s*\(([^;]*?)\)\s*;" % name, text, flags=re.S)
+        assert m, name
+        params = m.group(1).strip()
+        n = 0 if params in ("", "void") else len(params.split(","))
+        assert n == len(args), f"{name}: header has {n} parameters, ctypes table {len(args)}"
+
+
+def test_validation_errors_without_gpu():
+    lib = _lib.load()
+    # wrong head dim
+    rc = lib.msa_pool_chunks(None, None, None, 0, 10, 8, 64, None, None, None, 1, None, None, None, 0, 0, 0, None,
+                             None, None, None)
+    assert rc == -1 and b"head dim" in lib.msa_last_error()
+    # null bank
+    rc = lib.msa_route_topk(None, 0, None, None, 1, 1, 32, 0, 1.0, 16, C.c_void_p(8), C.c_void_p(8), None, None, 0,
+                            None)
+    assert rc == -1 and b"null bank" in lib.msa_last_error()
+    rc = lib.msa_route_topk(None, 0, None, None, 1, 1, 32, 0, 1.0, 65, C.c_void_p(8), C.c_void_p(8), None, None, 0,
+                            None)
+    assert rc == -1 and b"topk" in lib.msa_last_error()
+    # bank tables that do not add up are rejected before any device call
+    off = (C.c_int32 * 3)(0, 2, 5)
+    gid = (C.c_int64 * 2)(7, 9)
+    h = C.c_void_p()
+    rc = lib.msa_bank_create(C.byref(h), 1, 6, 8, 128, 0, C.addressof(off), C.addressof(gid), 2)
+    assert rc == -1 and b"doc_chunk_off" in lib.msa_last_error()
+    assert lib.msa_route_workspace_bytes(16, 128, 32, 8, 128, 1000, 50, 16) > 16 * 128 * 1024 * 2
+    assert lib.msa_attn_workspace_bytes(4, 32, 128, 1000) > 0
+    with pytest.raises(TypeError):
+        import torch
+        _lib.dtype_code(torch.float16)
+
+
+def test_product_does_not_import_oracle():
+    """Nothing under msa_amd/ may reach into oracle/."""
+    pkg = os.path.join(ROOT, "msa_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                src = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in src.replace("ORACLE", ""), f"{f} mentions the oracle"

@@ -1,0 +1,392 @@
+"""GPU parity: the HIP path (called through the C ABI) against the fp64 closed-form oracle on the
+same seeded inputs.  Tolerances are the contract's: 1e-2 (bf16) / 1e-5 (fp32) relative to the
+reference's max magnitude; integer and index work is bit-exact; top-k is exact wherever the
+boundary gap exceeds 1e-3."""
+import math
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import closed_form as cf
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.bfloat16: 1e-2, torch.float32: 1e-5}
+
+
+def say(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not torch.cuda.is_available():
+        pytest.fail("no GPU visible: the gpu-marked tests need an MI355X")
+    from msa_amd import ops as _ops
+    return _ops
+
+
+def _ragged(seed, n_docs, lo, hi):
+    g = np.random.default_rng(seed)
+    return [int(x) for x in g.integers(lo, hi + 1, size=n_docs)]
+
+
+def _randn(shape, seed, dtype):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(shape, generator=g).to(dtype)
+
+
+# ------------------------------------------------------------------ chunk table
+@pytest.mark.parametrize("P,first", [(64, 3), (4, 0)])
+def test_chunk_table(ops, P, first):
+    say(f"chunk_table P={P} first={first}")
+    lens = _ragged(2, 1500, 1, 40 * P // 8 + 5) + [1, P, P + 1, 2 * P]
+    t = ops.chunk_table(lens, P, first)
+    torch.cuda.synchronize()
+    ds, dco, cs, cl, cd = cf.chunk_table(lens, P, first)
+    assert int(t.n_chunks.item()) == len(cs) == t.C
+    assert t.doc_chunk_off.cpu().tolist() == dco.tolist()
+    assert t.chunk_start.cpu().tolist() == cs.tolist()
+    assert t.chunk_len.cpu().tolist() == cl.tolist()
+    assert t.chunk_doc.cpu().tolist() == cd.tolist()
+
+
+# ------------------------------------------------------------------ pooling
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("rope", [False, True])
+def test_pool_chunks(ops, dtype, rope):
+    say(f"pool dtype={dtype} rope={rope}")
+    P, H, D, first, theta = 64, 8, 128, 3, 1e6
+    lens = _ragged(3, 40, 1, 700) + [1, 64, 65, 128, 2048]
+    T = first + sum(lens)
+    k, v, kr = (_randn((T, H, D), s, dtype) for s in (10, 11, 12))
+    t = ops.chunk_table(lens, P, first)
+    tables = ops.rope_tables(2048, D, theta) if rope else None
+    pk, pv, pkr = ops.pool_chunks(k.cuda(), v.cuda(), kr.cuda(), t, rope=tables, normalize_kr=True)
+    torch.cuda.synchronize()
+    _, _, cs, cl, _ = cf.chunk_table(lens, P, first)
+    k_ref = k.double()
+    if rope:
+        k_ref = cf.apply_rope(k_ref, torch.as_tensor(cf.doc_positions(lens, first)), theta)
+    want_k = cf.pool_chunks(k_ref, cs, cl)
+    want_v = cf.pool_chunks(v, cs, cl)
+    want_kr = cf.l2_normalize(cf.pool_chunks(kr, cs, cl))
+    tol = TOL[dtype]
+    assert cf.rel_err(pk.cpu(), want_k) < tol
+    assert cf.rel_err(pv.cpu(), want_v) < tol
+    assert cf.rel_err(pkr.cpu(), want_kr) < tol
+    # identity on a length-1 document: its only chunk is the token itself (bit-exact without rope)
+    if not rope:
+        c1 = int(np.nonzero(cl == 1)[0][0])
+        assert torch.equal(pv[c1].cpu(), v[int(cs[c1])])
+
+
+def test_pool_subset_of_tensors_and_linearity(ops):
+    say("pool subset / linearity")
+    P, H, D = 64, 8, 128
+    lens = _ragged(4, 30, 10, 300)
+    T = sum(lens)
+    x, y = _randn((T, H, D), 1, torch.float32), _randn((T, H, D), 2, torch.float32)
+    t = ops.chunk_table(lens, P)
+    (_, px, _) = ops.pool_chunks(None, x.cuda(), None, t)
+    (_, _, py) = ops.pool_chunks(None, None, y.cuda(), t)
+    (pz, _, _) = ops.pool_chunks((2 * x - 0.5 * y).cuda(), None, None, t)
+    torch.cuda.synchronize()
+    assert cf.rel_err(pz.cpu(), 2 * px.cpu().double() - 0.5 * py.cpu().double()) < 1e-5
+    const = torch.full((T, H, D), 0.375)
+    (pc, _, _) = ops.pool_chunks(const.cuda(), None, None, t)
+    assert torch.allclose(pc.cpu(), torch.full_like(pc.cpu(), 0.375), rtol=1e-6)
+
+
+# ------------------------------------------------------------------ scoring + top-k
+def _make_bank(ops, doc_chunks, Hkv, D, dtype, seed, normalize=True, with_kv=False):
+    _, dco, _, _, _ = cf.chunk_table([n * 4 for n in doc_chunks], 4)
+    Ctot = int(dco[-1])
+    kr = _randn((Ctot, Hkv, D), seed, torch.float32)
+    if normalize:
+        kr = cf.l2_normalize(kr).float()
+    kr = kr.to(dtype)
+    gids = [1000 + 7 * d for d in range(len(doc_chunks))]
+    bank = ops.Bank(2, dco.tolist(), gids, Hkv, D, dtype)
+    kr_dev = kr.cuda()
+    kh = vh = None
+    if with_kv:
+        kh = _randn((Ctot, Hkv, D), seed + 1, dtype).pin_memory()
+        vh = _randn((Ctot, Hkv, D), seed + 2, dtype).pin_memory()
+    bank.set_layer(1, kr_dev, kh, vh)
+    return bank, kr, dco, gids, kh, vh
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("mode", ["cosine", "scaled_dot"])
+@pytest.mark.parametrize("B,S", [(1, 64), (3, 50), (5, 128)])
+def test_chunk_scores(ops, dtype, mode, B, S):
+    say(f"chunk_scores dtype={dtype} mode={mode} B={B} S={S}")
+    Hq, Hkv, D = 32, 8, 128
+    doc_chunks = _ragged(5, 150, 1, 9)                       # C not a multiple of the tile
+    bank, kr, dco, _, _, _ = _make_bank(ops, doc_chunks, Hkv, D, dtype, 21, normalize=(mode == "cosine"))
+    q = _randn((B, S, Hq, D), 22, dtype)
+    mask = torch.ones(B, S, dtype=torch.bool)
+    if B > 1:
+        mask[1, : S // 2] = False                            # left padding
+        mask[2, 5] = False
+    got = ops.chunk_scores(bank, 1, q.cuda(), mask.cuda(), mode, D ** -0.5)
+    torch.cuda.synchronize()
+    want = cf.chunk_scores(q, mask, kr, mode)
+    assert cf.rel_err(got.cpu(), want) < TOL[dtype]
+    # no mask == all-ones mask
+    got2 = ops.chunk_scores(bank, 1, q.cuda(), None, mode, D ** -0.5)
+    want2 = cf.chunk_scores(q, torch.ones(B, S, dtype=torch.bool), kr, mode)
+    assert cf.rel_err(got2.cpu(), want2) < TOL[dtype]
+
+
+def test_chunk_scores_fully_masked_query(ops):
+    say("chunk_scores fully masked")
+    bank, kr, *_ = _make_bank(ops, [3, 4, 5], 8, 128, torch.bfloat16, 31)
+    q = _randn((2, 40, 32, 128), 32, torch.bfloat16)
+    mask = torch.ones(2, 40, dtype=torch.bool); mask[0] = False
+    got = ops.chunk_scores(bank, 1, q.cuda(), mask.cuda()).cpu()
+    assert torch.isinf(got[0]).all() and (got[0] < 0).all() and torch.isfinite(got[1]).all()
+
+
+def _plant(q, kr, dco, b, t, doc, strength, dtype):
+    """Makes one chunk of `doc` point along query token (b, t): its cosine score becomes ~strength."""
+    Hq, D = q.shape[2], q.shape[3]
+    Hkv = kr.shape[1]
+    G = Hq // Hkv
+    qn = cf.l2_normalize(q[b, t].double()).view(Hkv, G, D).sum(1)              # [Hkv, D]
+    direction = cf.l2_normalize(qn)
+    c = int(dco[doc]) + (int(dco[doc + 1]) - int(dco[doc])) // 2
+    noise = cf.l2_normalize(kr[c].double())
+    mix = cf.l2_normalize(strength * direction + (1 - strength) * noise)
+    kr[c] = mix.to(dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_route_topk_needles_and_acceptance(ops, dtype):
+    say(f"route_topk dtype={dtype}")
+    B, S, Hq, Hkv, D, k = 4, 70, 32, 8, 128, 16
+    doc_chunks = _ragged(6, 9000, 1, 6)                      # > 4096 documents: several candidate blocks
+    _, dco, _, _, _ = cf.chunk_table([n * 4 for n in doc_chunks], 4)
+    kr = cf.l2_normalize(_randn((int(dco[-1]), Hkv, D), 41, torch.float32)).float().to(dtype)
+    q = _randn((B, S, Hq, D), 42, dtype)
+    g = np.random.default_rng(7)
+    planted = {}
+    for b in range(B):
+        docs = g.choice(len(doc_chunks), size=k, replace=False)
+        planted[b] = [int(d) for d in docs]
+        tok = int(g.integers(0, S))                          # one token per query: score is monotone in strength
+        for r, d in enumerate(docs):
+            _plant(q, kr, dco, b, tok, int(d), 0.9 - 0.04 * r, dtype)                     # separated by >> 1e-3
+    gids = [5 * d + 3 for d in range(len(doc_chunks))]
+    bank = ops.Bank(1, dco.tolist(), gids, Hkv, D, dtype)
+    kr_dev = kr.cuda()
+    bank.set_layer(0, kr_dev)
+    mask = torch.ones(B, S, dtype=torch.bool)
+    scores, doc, gid = ops.route_topk(bank, 0, q.cuda(), mask.cuda(), "cosine", 1.0, k)
+    torch.cuda.synchronize()
+    scores, doc, gid = scores.cpu(), doc.cpu().long(), gid.cpu()
+    ds = cf.doc_scores(cf.chunk_scores(q, mask, kr, "cosine"), dco)
+    want_s, want_i = cf.topk_docs(ds, k)
+    gaps = (want_s[:, :-1] - want_s[:, 1:]).min()
+    assert float(gaps) > 1e-3, "fixture must separate every rank by more than the contract's gap"
+    assert torch.equal(doc, want_i)                          # bit-exact ids, in order
+    for b in range(B):
+        assert sorted(doc[b].tolist()) == sorted(planted[b])
+    assert torch.equal(gid, torch.as_tensor(gids)[doc])
+    assert cf.rel_err(scores, want_s) < TOL[dtype]
+    assert (scores[:, :-1] >= scores[:, 1:]).all()
+
+
+def test_route_topk_random_bank_acceptance_and_small_bank(ops):
+    say("route_topk acceptance on an un-planted bank; fewer docs than k")
+    B, S, Hq, Hkv, D, k = 3, 33, 32, 8, 128, 16
+    doc_chunks = _ragged(8, 5000, 1, 5)
+    bank, kr, dco, gids, _, _ = _make_bank(ops, doc_chunks, Hkv, D, torch.bfloat16, 51)
+    q = _randn((B, S, Hq, D), 52, torch.bfloat16)
+    scores, doc, gid = ops.route_topk(bank, 1, q.cuda(), None, "cosine", 1.0, k)
+    ds = cf.doc_scores(cf.chunk_scores(q, torch.ones(B, S, dtype=torch.bool), kr, "cosine"), dco)
+    # bf16 scores carry ~1e-2 relative error, so the index contract is the gap rule
+    errs = cf.topk_acceptable(ds, doc.cpu().long(), k, gap=1e-3)
+    assert not errs, errs
+    # returned scores are the kernel's own doc scores, sorted, and match the oracle's for those docs
+    picked = torch.gather(ds, 1, doc.cpu().long())
+    assert cf.rel_err(scores.cpu(), picked) < 1e-2
+    # 5 documents, k = 16: tail is (-inf, -1)
+    bank2, kr2, dco2, gids2, _, _ = _make_bank(ops, [2, 1, 3, 1, 2], Hkv, D, torch.bfloat16, 53)
+    s2, d2, g2 = ops.route_topk(bank2, 1, q.cuda(), None, "cosine", 1.0, k)
+    d2 = d2.cpu()
+    assert (d2[:, 5:] == -1).all() and (g2.cpu()[:, 5:] == -1).all() and torch.isinf(s2.cpu()[:, 5:]).all()
+    for b in range(B):
+        assert sorted(d2[b, :5].tolist()) == [0, 1, 2, 3, 4]
+
+
+def test_route_topk_ties_are_broken_by_lower_doc(ops):
+    say("route_topk ties")
+    Hkv, D = 8, 128
+    doc_chunks = [1] * 40
+    _, dco, _, _, _ = cf.chunk_table([4] * 40, 4)
+    row = cf.l2_normalize(_randn((1, Hkv, D), 61, torch.float32)).float()
+    kr = row.expand(40, Hkv, D).contiguous().to(torch.bfloat16)          # every document scores the same
+    bank = ops.Bank(1, dco.tolist(), list(range(40)), Hkv, D, torch.bfloat16)
+    kr_dev = kr.cuda()
+    bank.set_layer(0, kr_dev)
+    q = _randn((2, 8, 32, D), 62, torch.bfloat16)
+    s, d, _ = ops.route_topk(bank, 0, q.cuda(), None, "cosine", 1.0, 16)
+    assert d.cpu().tolist() == [list(range(16))] * 2
+    assert float((s.cpu().max(1).values - s.cpu().min(1).values).max()) == 0.0
+
+
+# ------------------------------------------------------------------ gather
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_gather_kv_exact(ops, dtype):
+    say(f"gather dtype={dtype}")
+    doc_chunks = _ragged(9, 300, 1, 8)
+    bank, _, dco, _, kh, vh = _make_bank(ops, doc_chunks, 8, 128, dtype, 71, with_kv=True)
+    sel = torch.tensor([[5, 6, 7, 290, 0, 12, -1, 12], [299, 298, 1, 0, 2, 150, 151, 3], [-1] * 8, [42] * 8],
+                       dtype=torch.int32)
+    side = torch.cuda.Stream()
+    K, V, cu = ops.gather_kv(bank, 1, sel, "cuda", stream=side)
+    side.synchronize()
+    wk, wv, wcu, _ = cf.gather_selected(kh, vh, dco, sel)
+    assert cu.tolist() == wcu.tolist()
+    assert torch.equal(K.cpu(), wk) and torch.equal(V.cpu(), wv)
+    with pytest.raises(Exception, match="outside"):
+        ops.gather_kv(bank, 1, torch.tensor([[300]], dtype=torch.int32), "cuda")
+    with pytest.raises(Exception, match="no host K"):
+        ops.gather_kv(bank, 0, sel, "cuda")
+
+
+# ------------------------------------------------------------------ assembly, append, attention
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_assemble_append_attention(ops, dtype):
+    say(f"assemble/append/attention dtype={dtype}")
+    B, Hq, Hkv, D = 3, 32, 8, 128
+    n_sel = [37, 0, 300]
+    n_loc = [64, 5, 200]
+    prefix_k, prefix_v = _randn((3, Hkv, D), 80, dtype), _randn((3, Hkv, D), 81, dtype)
+    mem_k, mem_v = _randn((sum(n_sel), Hkv, D), 82, dtype), _randn((sum(n_sel), Hkv, D), 83, dtype)
+    loc_k, loc_v = _randn((sum(n_loc), Hkv, D), 84, dtype), _randn((sum(n_loc), Hkv, D), 85, dtype)
+    cu_sel = np.concatenate([[0], np.cumsum(n_sel)])
+    cu_loc = np.concatenate([[0], np.cumsum(n_loc)])
+    Lcap = 3 + max(a + b for a, b in zip(n_sel, n_loc)) + 4
+    dev = lambda t: t.cuda()
+    i32 = lambda a: torch.as_tensor(a, dtype=torch.int32).cuda()
+    kc, vc, kv_len = ops.assemble_context(dev(prefix_k), dev(prefix_v), dev(mem_k), dev(mem_v), i32(cu_sel),
+                                          dev(loc_k), dev(loc_v), i32(cu_loc), B, Lcap)
+    torch.cuda.synchronize()
+    wk, wcu = cf.assemble_context(prefix_k, mem_k, cu_sel, loc_k, cu_loc)
+    wv, _ = cf.assemble_context(prefix_v, mem_v, cu_sel, loc_v, cu_loc)
+    lens = np.diff(wcu)
+    assert kv_len.cpu().tolist() == lens.tolist()
+    for b in range(B):
+        assert torch.equal(kc[b, : lens[b]].cpu(), wk[wcu[b]: wcu[b + 1]])
+        assert torch.equal(vc[b, : lens[b]].cpu(), wv[wcu[b]: wcu[b + 1]])
+
+    # stage-2 style: the query's own S_b rows are the last S_b keys; causal, bottom-right aligned
+    q_rows = n_loc
+    q = _randn((sum(q_rows), Hq, D), 86, dtype)
+    kv_off = (torch.arange(B, dtype=torch.int64) * Lcap).cuda()
+    out = ops.sparse_attn(dev(q), kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), kv_off, kv_len, int(lens.max()),
+                          cu_q=i32(cu_loc), max_sq=max(q_rows), causal=True)
+    torch.cuda.synchronize()
+    want = cf.attention_ragged(q, cu_loc, wk, wv, wcu, causal=True)
+    assert cf.rel_err(out.cpu(), want) < TOL[dtype]
+
+    # decode: append one row per sample, one query row per sample over everything
+    k_new, v_new = _randn((B, Hkv, D), 87, dtype), _randn((B, Hkv, D), 88, dtype)
+    ops.cache_append(dev(k_new), dev(v_new), kc, vc, kv_len)
+    assert kv_len.cpu().tolist() == (lens + 1).tolist()
+    qd = _randn((B, Hq, D), 89, dtype)
+    outd = ops.sparse_attn(dev(qd), kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), kv_off, kv_len, int(lens.max()) + 1)
+    torch.cuda.synchronize()
+    for b in range(B):
+        kk = torch.cat([wk[wcu[b]: wcu[b + 1]], k_new[b: b + 1]])
+        vv = torch.cat([wv[wcu[b]: wcu[b + 1]], v_new[b: b + 1]])
+        assert cf.rel_err(outd[b: b + 1].cpu(), cf.attention(qd[b: b + 1], kk, vv)) < TOL[dtype]
+
+
+def test_attention_long_context_splits_and_special_cases(ops):
+    say("attention long / special cases")
+    Hq, Hkv, D = 32, 8, 128
+    L = [4500, 1, 777]
+    B = len(L)
+    Lcap = max(L)
+    k = _randn((B, Lcap, Hkv, D), 90, torch.bfloat16)
+    v = _randn((B, Lcap, Hkv, D), 91, torch.bfloat16)
+    q = _randn((B, Hq, D), 92, torch.bfloat16)
+    kv_off = (torch.arange(B, dtype=torch.int64) * Lcap).cuda()
+    kv_len = torch.tensor(L, dtype=torch.int32).cuda()
+    out = ops.sparse_attn(q.cuda(), k.cuda().view(-1, Hkv, D), v.cuda().view(-1, Hkv, D), kv_off, kv_len, Lcap).cpu()
+    for b in range(B):
+        want = cf.attention(q[b: b + 1], k[b, : L[b]], v[b, : L[b]])
+        assert cf.rel_err(out[b: b + 1], want) < 1e-2
+    # a single key returns its value exactly (bf16 in, bf16 out)
+    assert torch.equal(out[1].view(Hkv, 4, D), v[1, 0][:, None, :].expand(Hkv, 4, D))
+
+
+# ------------------------------------------------------------------ the CPU-runnable routing layer
+def test_config1_routing_layer_fp32(ops):
+    """1,000 documents of 512 tokens, 8 KV heads, head_dim 128, pooled at 64; 64 query tokens,
+    32 Q heads; cosine / mean heads / max tokens / max chunks; top-16; gather; one decode step over
+    [memory | 64 local tokens].  Pooling runs in blocks of 100 documents as stage 1 does."""
+    say("config 1 (fp32, seed 0)")
+    n_docs, doc_len, P, Hq, Hkv, D, k, S = 1000, 512, 64, 32, 8, 128, 16, 64
+    per_block = 100
+    g = torch.Generator().manual_seed(0)
+    pooled = {"k": [], "v": [], "kr": []}
+    oracle_pooled = {"k": [], "v": [], "kr": []}
+    for blk in range(n_docs // per_block):
+        lens = [doc_len] * per_block
+        T = sum(lens)
+        kk, vv, rr = (torch.randn((T, Hkv, D), generator=g) for _ in range(3))
+        t = ops.chunk_table(lens, P)
+        pk, pv, pkr = ops.pool_chunks(kk.cuda(), vv.cuda(), rr.cuda(), t, normalize_kr=True)
+        pooled["k"].append(pk.cpu()); pooled["v"].append(pv.cpu()); pooled["kr"].append(pkr)
+        if blk in (0, 9):                                   # whole chunks: the library routine pins the mean
+            for name, x in (("k", kk), ("v", vv)):
+                want = x.double().view(-1, P, Hkv, D).mean(1)
+                assert cf.rel_err(pooled[name][-1], want) < 1e-5
+            assert cf.rel_err(pkr.cpu(), cf.l2_normalize(rr.double().view(-1, P, Hkv, D).mean(1))) < 1e-5
+    k_bank = torch.cat(pooled["k"]).pin_memory()
+    v_bank = torch.cat(pooled["v"]).pin_memory()
+    kr_bank = torch.cat(pooled["kr"])
+    C = kr_bank.shape[0]
+    assert C == 8000
+    dco = (np.arange(n_docs + 1) * (doc_len // P)).astype(np.int64)
+    bank = ops.Bank(1, dco.tolist(), list(range(n_docs)), Hkv, D, torch.float32)
+    bank.set_layer(0, kr_bank, k_bank, v_bank)
+    q = torch.randn((1, S, Hq, D), generator=g)
+    mask = torch.ones(1, S, dtype=torch.bool)
+    scores, doc, gid = ops.route_topk(bank, 0, q.cuda(), mask.cuda(), "cosine", 1.0, k)
+    cs = ops.chunk_scores(bank, 0, q.cuda(), mask.cuda(), "cosine", 1.0)
+    torch.cuda.synchronize()
+    kr_cpu = kr_bank.cpu()
+    want_cs = cf.chunk_scores(q, mask, kr_cpu, "cosine")
+    assert cf.rel_err(cs.cpu(), want_cs) < 1e-5
+    ds = cf.doc_scores(want_cs, dco)
+    assert not cf.topk_acceptable(ds, doc.cpu().long(), k, gap=1e-3)
+    want_s, want_i = cf.topk_docs(ds, k)
+    assert cf.rel_err(scores.cpu(), want_s) < 1e-5
+    # fp32 error is ~1e-7, far below typical rank gaps: ids agree wherever ranks are separated by > 1e-5
+    sep = (want_s[0, :-1] - want_s[0, 1:]) > 1e-5
+    if bool(sep.all()):
+        assert torch.equal(doc.cpu().long(), want_i)
+    # gather + decode over [memory | 64 local tokens]
+    K, V, cu = ops.gather_kv(bank, 0, doc.cpu(), "cuda")
+    torch.cuda.synchronize()
+    wk, wv, wcu, _ = cf.gather_selected(k_bank, v_bank, dco, doc.cpu().long())
+    assert torch.equal(K.cpu(), wk) and torch.equal(V.cpu(), wv) and int(cu[-1]) == 16 * 8
+    loc_k, loc_v = torch.randn((64, Hkv, D), generator=g), torch.randn((64, Hkv, D), generator=g)
+    qd = torch.randn((1, Hq, D), generator=g)
+    i32 = lambda a: torch.as_tensor(a, dtype=torch.int32).cuda()
+    kc, vc, kv_len = ops.assemble_context(None, None, K, V, i32(cu.tolist()), loc_k.cuda(), loc_v.cuda(),
+                                          i32([0, 64]), 1, 256)
+    out = ops.sparse_attn(qd.cuda(), kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), torch.zeros(1, dtype=torch.int64).cuda(),
+                          kv_len, 192)
+    torch.cuda.synchronize()
+    want = cf.attention(qd, torch.cat([wk, loc_k]), torch.cat([wv, loc_v]))
+    assert cf.rel_err(out.cpu(), want) < 1e-5

@@ -1,0 +1,320 @@
+#!/usr/bin/env python3
+"""Benchmark of the MSA routing hot path on one MI355X.
+
+A step is one routed batch at the 100M-token bank: B = 16 queries of S = 128 tokens scored against
+the HBM-resident pooled K_r of each of 18 routed layers (cosine, mean over 32 heads, max over
+tokens, max over a document's chunks), top-16 documents per query and layer, and the selected
+documents' pooled K / V copied from pinned host memory on a side stream while the next layer is
+being scored.  Inputs are synthetic (seeded), resident in HBM / pinned memory before timing starts.
+
+Prints ONE JSON line: routed queries/s, plus the roofline of the dominant kernel (the scoring
+kernel, timed with HIP event pairs around each of its launches on its own stream) and the CPU
+baseline (the reference's torch op sequence on a bounded slice of the same bank, host cores).
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_BF16_PEAK_TFLOPS = 2500.0
+HQ, HKV, D, P, TOPK = 32, 8, 128, 64, 16
+
+
+def log(msg):
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def make_doc_lens(total_tokens: int, seed: int):
+    g = np.random.default_rng(seed)
+    lens, left = [], total_tokens
+    while left > 0:
+        n = int(g.integers(256, 2049))
+        n = min(n, left)
+        lens.append(n)
+        left -= n
+    return lens
+
+
+def build_kr_layer(C_total: int, seed: int, device) -> torch.Tensor:
+    """N(0,1) rows L2-normalised per (chunk, head), bf16, generated on the device slice by slice."""
+    g = torch.Generator(device=device).manual_seed(seed)
+    kr = torch.empty((C_total, HKV, D), dtype=torch.bfloat16, device=device)
+    step = 1 << 17
+    for s in range(0, C_total, step):
+        e = min(C_total, s + step)
+        x = torch.randn((e - s, HKV, D), generator=g, device=device)
+        kr[s:e] = (x / x.norm(dim=-1, keepdim=True)).to(torch.bfloat16)
+    return kr
+
+
+def plant_needles(kr, q, doc_chunk_off, n_docs, seed):
+    """For every query plants TOPK documents whose middle chunk has, per KV head, cosine 0.98, 0.955,
+    ... with the pre-summed heads of one query token (the remainder is the chunk's own noise made
+    orthogonal to it).  The planted scores are cos * mean_g |sum of the group's unit heads| / 4,
+    about 0.49 * cos, so ranks are separated by ~1e-2 (>> the 1e-3 contract gap) and far above the
+    ~0.06 of un-planted chunks.  Returns the expected [B, TOPK] document ids in rank order."""
+    B, S = q.shape[0], q.shape[1]
+    g = np.random.default_rng(seed)
+    want = np.zeros((B, TOPK), dtype=np.int64)
+    used = set()
+    for b in range(B):
+        tok = int(g.integers(0, S))
+        qt = q[b, tok].float()
+        qn = (qt / qt.norm(dim=-1, keepdim=True)).view(HKV, HQ // HKV, D).sum(1)
+        direction = qn / qn.norm(dim=-1, keepdim=True)
+        docs = []
+        while len(docs) < TOPK:
+            d = int(g.integers(0, n_docs))
+            if d not in used:
+                used.add(d)
+                docs.append(d)
+        for r, d in enumerate(docs):
+            c = (int(doc_chunk_off[d]) + int(doc_chunk_off[d + 1])) // 2
+            cos = 0.98 - 0.025 * r
+            noise = kr[c].float()
+            perp = noise - (noise * direction).sum(-1, keepdim=True) * direction
+            perp = perp / perp.norm(dim=-1, keepdim=True)
+            kr[c] = (cos * direction + (1 - cos * cos) ** 0.5 * perp).to(torch.bfloat16)
+            want[b, r] = d
+    return want
+
+
+def cpu_baseline(kr0, q0, doc_chunks, budget_s=25.0):
+    """Reference op sequence (oracle.reference_style) on the first ~200k chunks of the bank (about
+    10 s of work per dtype on 16 cores), on the host cores, extrapolated linearly in chunks and
+    layers to the whole routed batch."""
+    from oracle import reference_style as rs
+    C_total = int(sum(doc_chunks))
+    target = min(C_total, 200_000)
+    n, acc = 0, 0
+    while n < len(doc_chunks) and acc < target:
+        acc += doc_chunks[n]
+        n += 1
+    sub_chunks = doc_chunks[:n]
+    Cs = int(sum(sub_chunks))
+    pool_ids = torch.repeat_interleave(torch.arange(1, n + 1), torch.as_tensor(sub_chunks))
+    out = {}
+    for name, dt in (("fp32", torch.float32), ("bf16", torch.bfloat16)):
+        rk = kr0[:Cs].to("cpu").to(dt).transpose(0, 1).unsqueeze(0).contiguous()       # [1, Hkv, Cs, D]
+        qh = torch.nn.functional.normalize(q0.to("cpu").to(dt).permute(0, 2, 1, 3).contiguous(), p=2, dim=-1)
+        q5, m5 = rs.group_queries(qh, torch.ones(qh.shape[0], qh.shape[2], dtype=torch.bool), HQ // HKV, -1.0)
+        t0 = time.perf_counter()
+        rs.stage2_scores_topk(q5, m5, rk, pool_ids, sub_chunks, TOPK)
+        dt_s = time.perf_counter() - t0
+        out[name] = dt_s
+        if dt_s > budget_s:
+            break
+    return out, Cs
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=3)
+    ap.add_argument("--warmup", type=int, default=1)
+    ap.add_argument("--tokens", type=int, default=100_000_000, help="bank size in tokens")
+    ap.add_argument("--layers", type=int, default=18, help="routed layers resident in HBM")
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--seq", type=int, default=128)
+    ap.add_argument("--host-kv-layers", type=int, default=2,
+                    help="distinct pinned host K/V layer buffers (routed layers share them round-robin)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-sweep", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (no sharding, no collectives); use --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+
+    from msa_amd import _lib, ops
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    B, S, L = args.batch, args.seq, args.layers
+
+    t_setup = time.perf_counter()
+    doc_lens = make_doc_lens(args.tokens, 0)
+    doc_chunks = [(n + P - 1) // P for n in doc_lens]
+    doc_chunk_off = np.concatenate([[0], np.cumsum(doc_chunks)]).astype(np.int64)
+    n_docs, C_total = len(doc_lens), int(doc_chunk_off[-1])
+    log(f"bank: {args.tokens} tokens, {n_docs} docs, {C_total} chunks, {L} layers, "
+        f"{C_total * HKV * D * 2 * L / 1e9:.1f} GB of K_r")
+    bank = ops.Bank(L, doc_chunk_off.tolist(), list(range(n_docs)), HKV, D, torch.bfloat16)
+
+    # pinned host K / V: a few distinct layer buffers, filled from the device
+    n_host = max(1, min(args.host_kv_layers, L))
+    host_k, host_v = [], []
+    for i in range(n_host):
+        for dst, seed in ((host_k, 1000 + i), (host_v, 2000 + i)):
+            h = torch.empty((C_total, HKV, D), dtype=torch.bfloat16, pin_memory=True)
+            g = torch.Generator(device=dev).manual_seed(seed)
+            step = 1 << 18
+            for s in range(0, C_total, step):
+                e = min(C_total, s + step)
+                h[s:e].copy_(torch.randn((e - s, HKV, D), generator=g, device=dev).to(torch.bfloat16))
+            dst.append(h)
+    log(f"host K/V: {n_host} layer buffer(s), {2 * n_host * C_total * HKV * D * 2 / 1e9:.1f} GB pinned")
+
+    qs, wants, krs = [], [], []
+    gq = torch.Generator(device=dev).manual_seed(7)
+    for li in range(L):
+        kr = build_kr_layer(C_total, 100 + li, dev)
+        q = torch.randn((B, S, HQ, D), generator=gq, device=dev).to(torch.bfloat16)
+        wants.append(plant_needles(kr, q, doc_chunk_off, n_docs, 500 + li))
+        bank.set_layer(li, kr, host_k[li % n_host], host_v[li % n_host])
+        krs.append(kr)
+        qs.append(q)
+    torch.cuda.synchronize()
+    log(f"setup {time.perf_counter() - t_setup:.1f} s")
+
+    ws = bank.workspace(B, S, HQ, TOPK, dev)
+    scores = [torch.empty((B, TOPK), dtype=torch.float32, device=dev) for _ in range(L)]
+    docs = [torch.empty((B, TOPK), dtype=torch.int32, device=dev) for _ in range(L)]
+    gids = [torch.empty((B, TOPK), dtype=torch.int64, device=dev) for _ in range(L)]
+    docs_host = [torch.empty((B, TOPK), dtype=torch.int32, pin_memory=True) for _ in range(L)]
+    ready = [torch.cuda.Event() for _ in range(L)]
+    cap_chunks = B * TOPK * 32
+    gk = [torch.empty((cap_chunks, HKV, D), dtype=torch.bfloat16, device=dev) for _ in range(2)]
+    gv = [torch.empty((cap_chunks, HKV, D), dtype=torch.bfloat16, device=dev) for _ in range(2)]
+    side = torch.cuda.Stream()
+    main_stream = torch.cuda.current_stream()
+    sel_chunks = [0] * L
+
+    def route(li):
+        _lib.check(lib.msa_route_topk(bank.handle, li, qs[li].data_ptr(), None, B, S, HQ, _lib.MODE_COSINE, 1.0, TOPK,
+                                      scores[li].data_ptr(), docs[li].data_ptr(), gids[li].data_ptr(), ws.data_ptr(),
+                                      ws.numel(), main_stream.cuda_stream), "msa_route_topk")
+        docs_host[li].copy_(docs[li], non_blocking=True)
+        ready[li].record(main_stream)
+
+    def gather(li):
+        ready[li].synchronize()
+        cu = torch.empty(B + 1, dtype=torch.int64)
+        _lib.check(lib.msa_gather_plan(bank.handle, docs_host[li].data_ptr(), B, TOPK, cu.data_ptr()), "msa_gather_plan")
+        sel_chunks[li] = int(cu[-1])
+        _lib.check(lib.msa_gather_kv(bank.handle, li, docs_host[li].data_ptr(), B, TOPK, gk[li & 1].data_ptr(),
+                                     gv[li & 1].data_ptr(), cap_chunks, side.cuda_stream), "msa_gather_kv")
+
+    def step():
+        for li in range(L):
+            route(li)                      # layer li is being scored ...
+            if li > 0:
+                gather(li - 1)             # ... while layer li-1's K / V come over from the host
+        gather(L - 1)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    _lib.check(lib.msa_profile_enable(args.steps * L), "msa_profile_enable")
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_buf = (C.c_float * (args.steps * L))()
+    n_rec = C.c_int32(0)
+    _lib.check(lib.msa_profile_collect(ms_buf, args.steps * L, C.byref(n_rec)), "msa_profile_collect")
+    kern_ms = float(np.mean(list(ms_buf)[: n_rec.value]))
+    _lib.check(lib.msa_profile_enable(0), "msa_profile_enable")
+
+    # ---- parity at full size: planted needles must come back exactly, in rank order; gathered rows
+    # ---- of the last layer must equal the host rows
+    for li in range(L):
+        got = docs[li].cpu().numpy().astype(np.int64)
+        if not np.array_equal(got, wants[li]):
+            bad = np.nonzero((got != wants[li]).any(axis=1))[0]
+            log(f"layer {li}: rows {bad.tolist()} differ; got {got[bad[0]].tolist()} want {wants[li][bad[0]].tolist()} "
+                f"scores {scores[li][bad[0]].cpu().tolist()}")
+            sys.exit(f"bench.py: PARITY FAILURE at layer {li}: top-k ids differ from the planted documents")
+    last = L - 1
+    from oracle import closed_form as cf
+    wk, wv, wcu, _ = cf.gather_selected(host_k[last % n_host], host_v[last % n_host], doc_chunk_off,
+                                        torch.as_tensor(wants[last]))
+    n_sel = int(wcu[-1])
+    if n_sel != sel_chunks[last] or not torch.equal(gk[last & 1][:n_sel].cpu(), wk) or \
+            not torch.equal(gv[last & 1][:n_sel].cpu(), wv):
+        sys.exit("bench.py: PARITY FAILURE: gathered K / V rows differ from the host bank")
+
+    ms_per_step = elapsed / args.steps * 1e3
+    qps = B * args.steps / elapsed
+    flops = 2.0 * B * S * HKV * D * C_total                       # pre-summed GQA form, per launch
+    bytes_layer = C_total * HKV * D * 2 + B * S * HQ * D * 2 + C_total * 4 + B * TOPK * 16
+    tflops = flops / (kern_ms * 1e-3) / 1e12
+    intensity = flops / bytes_layer
+    bound = "mfma" if intensity > MFMA_BF16_PEAK_TFLOPS * 1e12 / (HBM_PEAK_GBS * 1e9) else "hbm"
+    if bound == "mfma":
+        roof = {"bound": "mfma", "achieved": round(tflops, 1), "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(tflops / MFMA_BF16_PEAK_TFLOPS, 4), "traffic": None}
+    else:
+        gbs = bytes_layer / (kern_ms * 1e-3) / 1e9
+        roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+    roof.update({"kernel": "score_gemm_kernel", "kernel_ms": round(kern_ms, 4), "launches_timed": n_rec.value,
+                 "flops_per_launch": flops, "algorithmic_bytes_per_launch": bytes_layer,
+                 "hbm_gbs_at_this_batch": round(bytes_layer / (kern_ms * 1e-3) / 1e9, 1)})
+
+    # ---- bandwidth-bound regime: one query (and fewer tokens) per scan of layer 0
+    sweep = []
+    if not args.no_sweep:
+        for b1, s1 in ((1, 16), (1, 64), (1, 128), (2, 128), (4, 128)):
+            q1 = qs[0][:b1, :s1].contiguous()
+            sc = torch.empty((b1, TOPK), dtype=torch.float32, device=dev)
+            dc = torch.empty((b1, TOPK), dtype=torch.int32, device=dev)
+            reps = 5
+            for r in range(reps + 1):
+                if r == 1:
+                    torch.cuda.synchronize()
+                    _lib.check(lib.msa_profile_enable(reps), "msa_profile_enable")
+                _lib.check(lib.msa_route_topk(bank.handle, 0, q1.data_ptr(), None, b1, s1, HQ, _lib.MODE_COSINE, 1.0,
+                                              TOPK, sc.data_ptr(), dc.data_ptr(), None, ws.data_ptr(), ws.numel(),
+                                              main_stream.cuda_stream), "msa_route_topk")
+            torch.cuda.synchronize()
+            buf = (C.c_float * reps)()
+            _lib.check(lib.msa_profile_collect(buf, reps, C.byref(n_rec)), "msa_profile_collect")
+            ms1 = float(np.mean(list(buf)[: n_rec.value]))
+            by = C_total * HKV * D * 2 + b1 * s1 * HKV * D * 2
+            sweep.append({"B": b1, "S": s1, "kernel_ms": round(ms1, 4), "GB/s": round(by / ms1 / 1e6, 1),
+                          "frac_hbm": round(by / ms1 / 1e6 / HBM_PEAK_GBS, 4)})
+        _lib.check(lib.msa_profile_enable(0), "msa_profile_enable")
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        times, Cs = cpu_baseline(krs[0], qs[0], doc_chunks)
+        best = min(times.values())
+        full = best * (C_total / Cs) * L
+        cpu = {"value": round(B / full, 5), "unit": "queries/s", "cores": torch.get_num_threads(), "kind": "port",
+               "sample": f"reference op sequence (matmul, masked_fill, mean, max, scatter_reduce amax, topk) on the "
+                         f"first {Cs} of {C_total} chunks of layer 0 for the same {B}x{S} queries; "
+                         f"{', '.join(f'{k} {v:.2f} s' for k, v in times.items())}; best extrapolated linearly "
+                         f"x{C_total / Cs:.1f} chunks x{L} layers",
+               "host_cpus": os.cpu_count()}
+
+    out = {
+        "metric": "routed queries/s at the 100M-token bank (router scoring + top-k + host gather, 18 layers)",
+        "value": round(qps, 2), "unit": "queries/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "configs[3]: 100M-token bank, K_r HBM-resident, K/V pinned host, B=16 x S=128, top-16",
+                   "bank_tokens": args.tokens, "chunks": C_total, "docs": n_docs, "routed_layers": L, "batch": B,
+                   "query_tokens": S, "top_k": TOPK, "kr_hbm_gb": round(C_total * HKV * D * 2 * L / 1e9, 1),
+                   "host_kv_layer_buffers": n_host, "selected_chunks_per_layer": int(np.mean(sel_chunks)),
+                   "mode": "cosine/mean-heads/max-tokens/max-chunks"},
+        "roofline": roof, "cpu_baseline": cpu, "hbm_regime_sweep": sweep, "parity": "needles exact on all layers",
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

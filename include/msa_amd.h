@@ -12,8 +12,8 @@
  *   - pointers are DEVICE pointers unless the name ends in `_host`;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); all work is
  *     enqueued on it and nothing synchronises unless stated;
- *   - no entry point allocates device memory: scratch comes in as `workspace`, sized by the
- *     matching *_workspace_bytes() function;
+ *   - only msa_bank_create allocates device memory (two small tables); every other entry point
+ *     takes its scratch as `workspace`, sized by the matching *_workspace_bytes() function;
  *   - activations are token-major [T, H, D]; pooled tensors and the bank are chunk-major
  *     [C, Hkv, D]; document indices are 0-based in bank order; D must be 128;
  *   - dtype: MSA_BF16 (storage bf16, fp32 accumulation) or MSA_F32.
@@ -107,6 +107,14 @@ int msa_route_topk(const msa_bank* bank, int32_t layer, const void* q, const uin
                    int32_t B, int32_t S, int32_t Hq, int32_t mode, float scale, int32_t topk,
                    float* scores_out, int32_t* doc_out, int64_t* doc_global_out, void* workspace,
                    size_t workspace_bytes, void* stream);
+
+/* Measurement hook (no counterpart in the reference): while enabled, every launch of the scoring
+ * kernel inside msa_chunk_scores / msa_route_topk is bracketed by a HIP event pair on its own
+ * stream, up to max_records launches (0 disables and frees the events).  msa_profile_collect waits
+ * for the recorded launches, writes their durations in milliseconds to ms_host[0..*n_out) and
+ * resets the record count.  Not thread-safe; meant for benchmarks. */
+int msa_profile_enable(int32_t max_records);
+int msa_profile_collect(float* ms_host, int32_t cap, int32_t* n_out);
 
 /* ---------------------------------------------------------------------------------------------
  * Gather of the selected documents' pooled K / V from pinned host memory.  Replaces the

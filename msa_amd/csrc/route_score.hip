@@ -241,6 +241,14 @@ __global__ void decode_scores_kernel(const uint32_t* __restrict__ key, int64_t n
   }
 }
 
+// Optional timing of the scoring kernel alone: event pairs recorded around its launch.
+struct KernelTimer {
+  hipEvent_t* start = nullptr;
+  hipEvent_t* stop = nullptr;
+  int cap = 0;
+  int n = 0;
+} g_timer;
+
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
 int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* chunk_key, int32_t M_rows,
                 int32_t C, int32_t K, int32_t blocks_per_query, hipStream_t st) {
@@ -255,9 +263,15 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
                                 (int)lds));
     attr_set = true;
   }
+  const bool timed = g_timer.n < g_timer.cap;
+  if (timed) MSA_HIP(hipEventRecord(g_timer.start[g_timer.n], st));
   kern<<<grid, WAVES_M * WAVES_N * 64, lds, st>>>(static_cast<const T*>(qs), static_cast<const T*>(kr), row_bits,
                                                   chunk_key, M_rows, C, K, blocks_per_query, tiles_m, tiles_n);
   MSA_LAUNCH_CHECK();
+  if (timed) {
+    MSA_HIP(hipEventRecord(g_timer.stop[g_timer.n], st));
+    ++g_timer.n;
+  }
   return MSA_OK;
 }
 
@@ -282,6 +296,38 @@ RouteWorkspace route_workspace_layout(int32_t B, int32_t S, int32_t Hkv, int32_t
   w.off_cand = off;     off = align_up(off + (size_t)B * w.topk_blocks * kTopkMax * sizeof(uint64_t), 256);
   w.bytes = off;
   return w;
+}
+
+extern "C" int msa_profile_enable(int32_t max_records) {
+  for (int i = 0; i < g_timer.cap; ++i) {
+    (void)hipEventDestroy(g_timer.start[i]);
+    (void)hipEventDestroy(g_timer.stop[i]);
+  }
+  delete[] g_timer.start;
+  delete[] g_timer.stop;
+  g_timer = KernelTimer{};
+  MSA_REQUIRE(max_records >= 0 && max_records <= 1 << 20, "msa_profile_enable: max_records=%d", max_records);
+  if (max_records == 0) return MSA_OK;
+  g_timer.start = new hipEvent_t[max_records];
+  g_timer.stop = new hipEvent_t[max_records];
+  for (int i = 0; i < max_records; ++i) {
+    MSA_HIP(hipEventCreate(&g_timer.start[i]));
+    MSA_HIP(hipEventCreate(&g_timer.stop[i]));
+    g_timer.cap = i + 1;
+  }
+  return MSA_OK;
+}
+
+extern "C" int msa_profile_collect(float* ms_host, int32_t cap, int32_t* n_out) {
+  MSA_REQUIRE(ms_host && n_out, "msa_profile_collect: null pointer");
+  const int n = std::min(g_timer.n, cap);
+  for (int i = 0; i < n; ++i) {
+    MSA_HIP(hipEventSynchronize(g_timer.stop[i]));
+    MSA_HIP(hipEventElapsedTime(&ms_host[i], g_timer.start[i], g_timer.stop[i]));
+  }
+  *n_out = n;
+  g_timer.n = 0;
+  return MSA_OK;
 }
 
 extern "C" size_t msa_route_workspace_bytes(int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D, int64_t C,

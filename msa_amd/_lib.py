@@ -9,7 +9,7 @@ import os
 from typing import Optional
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libmsa_amd.so")
+LIB_PATH = os.environ.get("MSA_AMD_LIB", os.path.join(HERE, "libmsa_amd.so"))   # override: an alternative build
 
 MSA_BF16, MSA_F32 = 0, 1
 MODE_COSINE, MODE_SCALED_DOT = 0, 1

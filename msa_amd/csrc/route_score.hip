@@ -6,7 +6,10 @@
 // an NT GEMM  [B*S_pad, Hkv*D] x [C, Hkv*D]^T  whose output is never written: each 32-row MFMA
 // block is reduced to a column max over its scored rows in registers and merged into
 // chunk_key[B, C] (order-preserving uint32 keys) with atomicMax.
+#include <stdlib.h>
+
 #include <algorithm>
+#include <type_traits>
 
 #include "common.h"
 
@@ -14,6 +17,7 @@ namespace {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 // ------------------------------------------------------------------------------------------
 // Prologue: normalise (cosine mode), sum the G heads of each KV group, cast, build row masks.
@@ -86,20 +90,24 @@ template <typename T>
 struct Mma;
 template <>
 struct Mma<bf16_t> {
+  typedef bf16x8_t Frag;
   static constexpr int kSub = 4;   // 32x32x16 steps per 64-element K tile
-  static __device__ __forceinline__ floatx16_t run(const char* a, const char* b, int sub, int half, floatx16_t c) {
-    const bf16x8_t fa = *reinterpret_cast<const bf16x8_t*>(a + sub * 32 + half * 16);
-    const bf16x8_t fb = *reinterpret_cast<const bf16x8_t*>(b + sub * 32 + half * 16);
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa, fb, c, 0, 0, 0);
+  static __device__ __forceinline__ Frag load(const char* row, int sub, int half) {
+    return *reinterpret_cast<const Frag*>(row + sub * 32 + half * 16);
+  }
+  static __device__ __forceinline__ floatx16_t mma(Frag a, Frag b, floatx16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
   }
 };
 template <>
 struct Mma<float> {
+  typedef float Frag;
   static constexpr int kSub = 16;  // 32x32x2 steps per 32-element K tile
-  static __device__ __forceinline__ floatx16_t run(const char* a, const char* b, int sub, int half, floatx16_t c) {
-    const float fa = *reinterpret_cast<const float*>(a + sub * 8 + half * 4);
-    const float fb = *reinterpret_cast<const float*>(b + sub * 8 + half * 4);
-    return __builtin_amdgcn_mfma_f32_32x32x2f32(fa, fb, c, 0, 0, 0);
+  static __device__ __forceinline__ Frag load(const char* row, int sub, int half) {
+    return *reinterpret_cast<const Frag*>(row + sub * 8 + half * 4);
+  }
+  static __device__ __forceinline__ floatx16_t mma(Frag a, Frag b, floatx16_t c) {
+    return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
   }
 };
 
@@ -138,33 +146,36 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   const char* ga = reinterpret_cast<const char*>(qs);
   const char* gb = reinterpret_cast<const char*>(kr);
 
-  uint4 ra[kVecA], rb[kVecB];
+  // Global -> register staging through buffer loads: one resource per operand tile whose extent is
+  // the valid part of the tile, so rows past M_rows / C read as zero in hardware (no branches, no
+  // clamps), one voffset register per thread, and the per-vector / per-K-tile displacement rides in
+  // the scalar offset.
+  const int rows_a = min(BM, M_rows - m0), rows_b = min(BN, C - n0);
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(ga) + (int64_t)m0 * row_bytes_g, 0, (int)(rows_a * row_bytes_g), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(gb) + (int64_t)n0 * row_bytes_g, 0, (int)(rows_b * row_bytes_g), 0x00020000);
+  const int voff = (tid >> 3) * (int)row_bytes_g + (tid & 7) * 16;
+  const int vec_stride = (kThreads / 8) * (int)row_bytes_g;     // rows between a thread's vectors
+  u32x4_t ra[kVecA], rb[kVecB];
   auto load_tile = [&](int kt) {
 #pragma unroll
-    for (int i = 0; i < kVecA; ++i) {
-      const int v = tid + i * kThreads, r = v >> 3, c = v & 7;
-      const int m = m0 + r;
-      ra[i] = m < M_rows ? *reinterpret_cast<const uint4*>(ga + m * row_bytes_g + (int64_t)kt * kRowBytes + c * 16)
-                         : make_uint4(0, 0, 0, 0);
-    }
+    for (int i = 0; i < kVecA; ++i)
+      ra[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, voff, i * vec_stride + kt * kRowBytes, 0);
 #pragma unroll
-    for (int i = 0; i < kVecB; ++i) {
-      const int v = tid + i * kThreads, r = v >> 3, c = v & 7;
-      const int n = n0 + r;
-      rb[i] = n < C ? *reinterpret_cast<const uint4*>(gb + n * row_bytes_g + (int64_t)kt * kRowBytes + c * 16)
-                    : make_uint4(0, 0, 0, 0);
-    }
+    for (int i = 0; i < kVecB; ++i)
+      rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, voff, i * vec_stride + kt * kRowBytes, 0);
   };
   auto store_tile = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < kVecA; ++i) {
       const int v = tid + i * kThreads, r = v >> 3, c = v & 7;
-      *reinterpret_cast<uint4*>(lds + buf * kBufBytes + r * kRowStride + c * 16) = ra[i];
+      *reinterpret_cast<u32x4_t*>(lds + buf * kBufBytes + r * kRowStride + c * 16) = ra[i];
     }
 #pragma unroll
     for (int i = 0; i < kVecB; ++i) {
       const int v = tid + i * kThreads, r = v >> 3, c = v & 7;
-      *reinterpret_cast<uint4*>(lds + buf * kBufBytes + (BM + r) * kRowStride + c * 16) = rb[i];
+      *reinterpret_cast<u32x4_t*>(lds + buf * kBufBytes + (BM + r) * kRowStride + c * 16) = rb[i];
     }
   };
 
@@ -176,28 +187,69 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
+  // Software pipeline over K tiles.  While tile kt is multiplied out of LDS buffer kt&1:
+  //   - tile kt+1 (already in registers) is written to the other buffer during sub-step 1, and the
+  //     global loads of tile kt+2 are issued right behind it (a whole iteration to land);
+  //   - operand fragments are double-buffered in registers, one sub-step ahead of the MFMAs;
+  //   - the single barrier per tile sits before the LAST sub-step's MFMAs, after that sub-step's
+  //     fragments were read, so the first fragments of tile kt+1 are fetched under those MFMAs.
+  // Hazards: buffer (kt+1)&1 held tile kt-1, whose last fragment reads were issued before the
+  // barrier of iteration kt-1; the writes of tile kt+1 are complete at the barrier of iteration kt.
+  typedef typename Mma<T>::Frag Frag;
+  constexpr int kSub = Mma<T>::kSub;
   const int k_tiles = (int)(row_bytes_g / kRowBytes);
-  load_tile(0);
-  store_tile(0);
-  __syncthreads();
-  for (int kt = 0; kt < k_tiles; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < k_tiles) load_tile(kt + 1);
-    const char* pa = lds + buf * kBufBytes + (wm * WM + l32) * kRowStride;
-    const char* pb = lds + buf * kBufBytes + (BM + wn * WN + l32) * kRowStride;
+  const int a_row = (wm * WM + l32) * kRowStride, b_row = (BM + wn * WN + l32) * kRowStride;
+  Frag fa[2][TM], fb[2][TN];
+  auto load_frags = [&](int buf, int sub, int slot) {
+    const char* pa = lds + buf * kBufBytes + a_row;
+    const char* pb = lds + buf * kBufBytes + b_row;
 #pragma unroll
-    for (int sub = 0; sub < Mma<T>::kSub; ++sub) {
+    for (int i = 0; i < TM; ++i) fa[slot][i] = Mma<T>::load(pa + i * 32 * kRowStride, sub, half);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) fb[slot][j] = Mma<T>::load(pb + j * 32 * kRowStride, sub, half);
+  };
+
+  // One K tile out of LDS buffer `buf`; kMore says a next tile exists (the steady-state loop is
+  // compiled without that condition so the wait counters around the barrier stay exact).
+  auto k_tile = [&](auto more_tag, int kt) {
+    constexpr bool kMore = decltype(more_tag)::value;
+    const int buf = kt & 1;
+#pragma unroll
+    for (int sub = 0; sub < kSub; ++sub) {
+#ifndef MSA_ABLATE
+#define MSA_ABLATE 0
+#endif
+      if (sub + 1 < kSub) {
+        if (MSA_ABLATE != 5) load_frags(buf, sub + 1, (sub + 1) & 1);
+      } else if (kMore) {
+        if (MSA_ABLATE != 3) __syncthreads();
+        if (MSA_ABLATE != 5) load_frags(buf ^ 1, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);   // keep the last sub-step's MFMAs behind these reads
+      }
+      if (sub == 1 && kMore) {
+        if (MSA_ABLATE != 4 && MSA_ABLATE != 6) store_tile(buf ^ 1);
+        if (kt + 2 < k_tiles && MSA_ABLATE != 4 && MSA_ABLATE != 7) load_tile(kt + 2);
+      }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = Mma<T>::run(pa + i * 32 * kRowStride, pb + j * 32 * kRowStride, sub, half, acc[i][j]);
+        for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::mma(fa[sub & 1][i], fb[sub & 1][j], acc[i][j]);
     }
-    if (kt + 1 < k_tiles) {
-      store_tile(buf ^ 1);   // the other buffer was last read one iteration ago, behind the barrier below
-      __syncthreads();
-    }
-  }
+  };
+
+  load_tile(0);
+  store_tile(0);
+  if (k_tiles > 1) load_tile(1);
+  __syncthreads();
+  load_frags(0, 0, 0);
+#if defined(MSA_ABLATE) && MSA_ABLATE == 9
+  for (int rep = 0; rep < 3; ++rep)
+#endif
+  for (int kt = 0; kt + 1 < k_tiles; ++kt) k_tile(std::true_type{}, kt);
+  k_tile(std::false_type{}, k_tiles - 1);
+#if defined(MSA_ABLATE) && MSA_ABLATE == 8
+  if (acc[0][0][0] != 123.456f) return;
+#endif
 
   // Epilogue.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of its 32x32 block.
 #pragma unroll
@@ -390,12 +442,23 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
   const int32_t bpq = w.S_pad / 32;
   int rc;
   if (bank->dtype == MSA_BF16) {
-    if (w.M_rows <= 128)
-      rc = launch_gemm<bf16_t, 128, 128, 2, 2>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C,
-                                              K, bpq, st);
-    else
-      rc = launch_gemm<bf16_t, 256, 128, 2, 2>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C,
-                                              K, bpq, st);
+    // Tile choice by query rows: small M is HBM-bound (narrow M tile, more workgroups in flight),
+    // large M is MFMA-bound (256 x 256 tile, 8 wavefronts).  MSA_SCORE_TILE overrides for tuning.
+    const char* ev = getenv("MSA_SCORE_TILE");
+    const int variant = ev ? atoi(ev) : (w.M_rows <= 64 ? 0 : w.M_rows <= 128 ? 1 : 2);
+#define MSA_GEMM(BM_, BN_, WM_, WN_)                                                                              \
+  launch_gemm<bf16_t, BM_, BN_, WM_, WN_>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C, \
+                                          K, bpq, st)
+    switch (variant) {
+      case 0: rc = MSA_GEMM(64, 128, 2, 2); break;
+      case 1: rc = MSA_GEMM(128, 256, 2, 4); break;
+      case 2: rc = MSA_GEMM(256, 256, 2, 4); break;
+      case 3: rc = MSA_GEMM(256, 256, 4, 2); break;
+      case 4: rc = MSA_GEMM(128, 128, 2, 2); break;
+      case 5: rc = MSA_GEMM(128, 128, 2, 4); break;
+      default: msa_set_error("MSA_SCORE_TILE=%d unknown", variant); return MSA_EINVAL;
+    }
+#undef MSA_GEMM
   } else {
     rc = launch_gemm<float, 128, 128, 2, 2>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C, K,
                                             bpq, st);

@@ -29,6 +29,10 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 HQ, HKV, D, P, TOPK = 32, 8, 128, 64, 16
+# Bytes past L2 per launch of the scoring kernel at the default workload, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a plain 1 GiB device copy
+# (FETCH_SIZE x2.0, WRITE_SIZE x1.0); see profiles/score_gemm_c4_100M_bank.txt.
+SCORE_TRAFFIC_DEFAULT_WORKLOAD = (2.0 * 4_904_568 + 1.0 * 122_269) * 1024
 
 
 def log(msg):
@@ -131,6 +135,8 @@ def main():
                     help="distinct pinned host K/V layer buffers (routed layers share them round-robin)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy (reference point for rocprof FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no sharding, no collectives); use --gpus 1")
@@ -261,6 +267,8 @@ def main():
         gbs = bytes_layer / (kern_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
+    if (args.tokens, B, S) == (100_000_000, 16, 128):
+        roof["traffic"] = SCORE_TRAFFIC_DEFAULT_WORKLOAD
     roof.update({"kernel": "score_gemm_kernel", "kernel_ms": round(kern_ms, 4), "launches_timed": n_rec.value,
                  "flops_per_launch": flops, "algorithmic_bytes_per_launch": bytes_layer,
                  "hbm_gbs_at_this_batch": round(bytes_layer / (kern_ms * 1e-3) / 1e9, 1)})
@@ -288,6 +296,14 @@ def main():
             sweep.append({"B": b1, "S": s1, "kernel_ms": round(ms1, 4), "GB/s": round(by / ms1 / 1e6, 1),
                           "frac_hbm": round(by / ms1 / 1e6 / HBM_PEAK_GBS, 4)})
         _lib.check(lib.msa_profile_enable(0), "msa_profile_enable")
+
+    if args.calibrate_copy:
+        src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).fill_(1.0)     # 1 GiB
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     cpu = None
     if not args.no_cpu_baseline:

@@ -1,0 +1,228 @@
+"""``MemorySparseAttention`` with the reference layer's interface
+(src/msa/memory_sparse_attention.py:20-405): same constructor arguments, parameter names,
+``set_memory_client``, ``forward`` signature and stage dispatch through
+``past_key_value.cache_kwargs[layer_idx]["stage"]``.
+
+The dense projections, RMSNorm and rotary are PyTorch-ROCm (the backbone is not part of the hot
+path); chunk pooling, routing, gather, context assembly and attention run in the HIP library.
+Inference only: the training branch of the reference (:407-465, 488-852) is not provided.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+from .config import MSAConfig
+
+
+class RMSNorm(nn.Module):
+    """Qwen3RMSNorm: fp32 statistics, weight applied in the input dtype."""
+
+    def __init__(self, dim: int, eps: float = 1e-6):
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim))
+        self.variance_epsilon = eps
+
+    def forward(self, x):
+        dt = x.dtype
+        xf = x.float()
+        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.variance_epsilon)
+        return self.weight * xf.to(dt)
+
+
+def rotate_half(x):
+    h = x.shape[-1] // 2
+    return torch.cat((-x[..., h:], x[..., :h]), dim=-1)
+
+
+def apply_rotary_bshd(x, cos, sin):
+    """Half-split rotary on ``x [B, S, H, D]`` with ``cos / sin [B, S, D]`` (transformers
+    ``apply_rotary_pos_emb`` with the head axis at 2)."""
+    return x * cos[:, :, None, :] + rotate_half(x) * sin[:, :, None, :]
+
+
+def rotary_embedding(position_ids: torch.Tensor, head_dim: int, theta: float, dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(cos, sin) [B, S, D]`` as Qwen3RotaryEmbedding computes them (fp32, then cast)."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2, dtype=torch.int64, device=position_ids.device).float() / head_dim))
+    freqs = position_ids[..., None].float() * inv_freq
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
+class MemorySparseAttention(nn.Module):
+    def __init__(self, config: MSAConfig, layer_idx: int):
+        super().__init__()
+        self.config = config
+        self.layer_idx = layer_idx
+        self.head_dim = config.head_dim
+        self.num_key_value_groups = config.num_attention_heads // config.num_key_value_heads
+        self.scaling = self.head_dim ** -0.5
+        self.attention_dropout = config.attention_dropout
+        hs, Hq, Hkv, D = config.hidden_size, config.num_attention_heads, config.num_key_value_heads, self.head_dim
+        self.q_proj = nn.Linear(hs, Hq * D, bias=config.attention_bias)
+        self.k_proj = nn.Linear(hs, Hkv * D, bias=config.attention_bias)
+        self.v_proj = nn.Linear(hs, Hkv * D, bias=config.attention_bias)
+        self.o_proj = nn.Linear(Hq * D, hs, bias=config.attention_bias)
+        self.q_norm = RMSNorm(D, eps=config.rms_norm_eps)
+        self.k_norm = RMSNorm(D, eps=config.rms_norm_eps)
+
+        mc = config.msa_config
+        self.top_k_docs = mc.top_k_docs
+        self.pooling_kernel_size = mc.pooling_kernel_size
+        ridx = mc.router_layer_idx
+        self.router_layer_idx = list(range(config.num_hidden_layers)) if ridx == "all" else [int(i) for i in ridx.split(",")]
+        self.is_router_layer = layer_idx in self.router_layer_idx
+        self.head_reduce_method, self.query_reduce_method = mc.head_reduce_method, mc.query_reduce_method
+        self.chunk_reduce_method, self.decouple_pooling_mode = mc.chunk_reduce_method, mc.decouple_pooling_mode
+        self.aux_loss_method, self.decouple_router = mc.aux_loss_method, mc.decouple_router
+        if self.is_router_layer and self.decouple_router:
+            self.router_k_proj = nn.Sequential(nn.Linear(hs, Hkv * D, bias=False))
+            self.router_q_proj = nn.Sequential(nn.Linear(hs, Hq * D, bias=False))
+        self.num_kv_heads = Hkv
+        self.template_prefix_kcache = None
+        self.template_prefix_vcache = None
+        self.memory_client = None
+        self.decode_reserve = 512      # rows kept free behind the stage-2 context for in-place decode appends
+
+    def set_memory_client(self, memory_client):
+        self.memory_client = memory_client
+
+    def forward(self, hidden_states: torch.Tensor, doc_ids: torch.LongTensor, attention_mask: Optional[torch.Tensor] = None,
+                position_embeddings: Optional[Tuple[torch.Tensor, torch.Tensor]] = None, past_key_value=None, **kwargs):
+        if self.training:
+            raise NotImplementedError("the training path of the reference layer is not part of this build")
+        if past_key_value is None:
+            raise Exception("error!")          # same failure as the reference without a cache (:97)
+        return self.forward_with_kvcache_for_batch_parrallel(hidden_states, doc_ids, attention_mask,
+                                                             position_embeddings, past_key_value, **kwargs)
+
+    # ------------------------------------------------------------------------------------------
+    def _project(self, hidden_states, position_embeddings):
+        B, S, _ = hidden_states.shape
+        D = self.head_dim
+        q = self.q_norm(self.q_proj(hidden_states).view(B, S, -1, D))
+        k = self.k_norm(self.k_proj(hidden_states).view(B, S, -1, D))
+        v = self.v_proj(hidden_states).view(B, S, -1, D)
+        cos, sin = position_embeddings
+        return apply_rotary_bshd(q, cos, sin).contiguous(), apply_rotary_bshd(k, cos, sin).contiguous(), v.contiguous()
+
+    def forward_with_kvcache_for_batch_parrallel(self, hidden_states, doc_ids, attention_mask=None,
+                                                 position_embeddings=None, past_key_value=None, **kwargs):
+        stage = past_key_value.cache_kwargs[self.layer_idx]["stage"]
+        q, k, v = self._project(hidden_states, position_embeddings)          # [B, S, H, D] token-major
+        if stage == "prefill_stage1":
+            return self._stage1(hidden_states, doc_ids, attention_mask, q, k, v, past_key_value)
+        if stage == "prefill_stage2":
+            return self._stage2(hidden_states, doc_ids, attention_mask, q, k, v, past_key_value)
+        return self._generate(hidden_states, q, k, v, past_key_value)
+
+    # ------------------------------------------------------------------------------------------ stage 1
+    def _stage1(self, hidden_states, doc_ids, attention_mask, q, k, v, cache):
+        """Encodes one packed block ``[template | doc 1 | doc 2 | ...]``: document-wise causal
+        attention, and on router layers chunk-mean pooling of K (rotated), V and K_r
+        (src/msa/memory_sparse_attention.py:137-243)."""
+        B, T, _ = hidden_states.shape
+        if B != 1:
+            raise ValueError("stage 1 takes one packed block at a time (batch size 1)")
+        Hq, Hkv, D, P = self.config.num_attention_heads, self.num_kv_heads, self.head_dim, self.pooling_kernel_size
+        ids = doc_ids[0]
+        n_template = int((ids == -2).sum())
+        vals, counts = torch.unique_consecutive(ids[n_template:], return_counts=True)
+        doc_lens = counts.tolist()
+        if (vals <= 0).any() or (attention_mask is not None and int(attention_mask.sum()) != T):
+            raise ValueError("stage 1 expects [template (-2) | documents (ids > 0)] with no padding")
+        kwargs = {"template_prefix_kcache": k[:, :n_template].transpose(1, 2),          # [1, Hkv, n, D] views
+                  "template_prefix_vcache": v[:, :n_template].transpose(1, 2)}
+        if self.is_router_layer:
+            table = ops.chunk_table(doc_lens, P, first_token=n_template, device=hidden_states.device)
+            rk = self.router_k_proj(hidden_states).view(T, Hkv, D).contiguous() if self.decouple_router else None
+            normalize = self.aux_loss_method == "INFONCE"
+            pk, pv, prk = ops.pool_chunks(k[0], v[0], rk if rk is not None else k[0], table, normalize_kr=normalize)
+            cache.update(pk.transpose(0, 1).unsqueeze(0), pv.transpose(0, 1).unsqueeze(0), self.layer_idx)
+            if rk is not None or normalize:
+                cache.update_router_kcache(prk.transpose(0, 1).unsqueeze(0), self.layer_idx)
+            kwargs.update({"doc_id_bias": T, "pooled_doc_ids": table.chunk_doc.long() + 1,
+                           "prefill_stage1_kvcache_size": cache.get_seq_length(self.layer_idx)})
+        cache.record_kwargs(self.layer_idx, kwargs)
+
+        # every document (and the template head) attends causally within itself
+        seg = ([n_template] if n_template else []) + doc_lens
+        cu = torch.tensor([0] + seg, dtype=torch.int64).cumsum(0)
+        dev = hidden_states.device
+        out = ops.sparse_attn(q[0], k[0], v[0], cu[:-1].to(dev), torch.tensor(seg, dtype=torch.int32, device=dev),
+                              max(seg), cu_q=cu.to(torch.int32).to(dev), max_sq=max(seg), scale=self.scaling, causal=True)
+        return self.o_proj(out.view(1, T, Hq * D)), None
+
+    # ------------------------------------------------------------------------------------------ stage 2
+    def _stage2(self, hidden_states, doc_ids, attention_mask, q, k, v, cache):
+        """Routes the query batch, pulls the winners' pooled K / V, lays out
+        ``[template prefix | selected chunks | query tokens]`` per sample and attends causally
+        (src/msa/memory_sparse_attention.py:245-359)."""
+        B, S, _ = hidden_states.shape
+        dev, dtype = hidden_states.device, hidden_states.dtype
+        Hq, Hkv, D = self.config.num_attention_heads, self.num_kv_heads, self.head_dim
+        ck = cache.cache_kwargs[self.layer_idx]
+        if self.memory_client is not None:
+            if self.template_prefix_kcache is None:
+                pk, pv = self.memory_client.get_template_prefix_kvcaches(self.layer_idx)
+                self.template_prefix_kcache, self.template_prefix_vcache = pk.to(dev), pv.to(dev)
+            pk, pv = self.template_prefix_kcache, self.template_prefix_vcache
+        else:
+            pk, pv = ck["template_prefix_kcache"].to(dev), ck["template_prefix_vcache"].to(dev)
+        prefix_k = pk[0].transpose(0, 1).contiguous()                     # [n_prefix, Hkv, D]
+        prefix_v = pv[0].transpose(0, 1).contiguous()
+        n_prefix = prefix_k.shape[0]
+
+        valid = attention_mask == 1
+        n_q = valid.sum(dim=1)
+        n_q_host = n_q.tolist()
+        mem_k = mem_v = cu_sel = None
+        n_sel_host = [0] * B
+        if self.is_router_layer:
+            rq = self.router_q_proj(hidden_states).view(B, S, Hq, D) if self.decouple_router else q
+            query_mask = (doc_ids == 0) & valid
+            mem_k, mem_v, scores, n_sel, gids = self.memory_client.doc_query(
+                rq.transpose(1, 2), query_mask, self.layer_idx, fused_normalize=(self.aux_loss_method == "INFONCE"),
+                native_layout=True)
+            n_sel_host = n_sel.tolist()
+            cu_sel = F.pad(n_sel.cumsum(0), (1, 0)).to(torch.int32)
+            if cache.meta.get("require_recall_topk", False):
+                ck["recall_topk"] = [{"topk_doc_ids": gids[i].tolist(), "score": scores[i].float().tolist()} for i in range(B)]
+        local_k, local_v, q_rows = k[valid], v[valid], q[valid]           # ragged [sum S_b, H, D]
+        cu_local = F.pad(n_q.cumsum(0), (1, 0)).to(torch.int32)
+        kv_host = [n_prefix + a + b for a, b in zip(n_sel_host, n_q_host)]
+        Lcap = max(kv_host) + self.decode_reserve
+        kc, vc, kv_len = ops.assemble_context(prefix_k, prefix_v, mem_k, mem_v, cu_sel, local_k, local_v, cu_local, B, Lcap)
+        kv_off = torch.arange(B, dtype=torch.int64, device=dev) * Lcap
+        out_rows = ops.sparse_attn(q_rows, kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), kv_off, kv_len, max(kv_host),
+                                   cu_q=cu_local, max_sq=max(n_q_host), scale=self.scaling, causal=True)
+        attn = torch.zeros((B, S, Hq * D), device=dev, dtype=dtype)
+        attn[valid] = out_rows.view(-1, Hq * D)
+        ck.update({"compacked_key_cache": kc, "compacked_value_cache": vc, "kv_lengths": kv_len, "kv_offsets": kv_off,
+                   "kv_capacity": Lcap})
+        cache.record_kwargs(self.layer_idx, ck)
+        return self.o_proj(attn), None
+
+    # ------------------------------------------------------------------------------------------ decode
+    def _generate(self, hidden_states, q, k, v, cache):
+        """One decode step over the compact cache, appended in place
+        (src/msa/memory_sparse_attention.py:361-405)."""
+        B, S, _ = hidden_states.shape
+        ck = cache.cache_kwargs[self.layer_idx]
+        if "compacked_key_cache" not in ck:
+            raise ValueError("compact KV cache not found: did prefill stage 2 run?")
+        if S != 1:
+            raise ValueError("the decode step takes one new token per sample")
+        kc, vc, kv_len = ck["compacked_key_cache"], ck["compacked_value_cache"], ck["kv_lengths"]
+        Hkv, D = self.num_kv_heads, self.head_dim
+        ck["decoded"] = ck.get("decoded", 0) + 1
+        if ck["decoded"] > self.decode_reserve:
+            raise RuntimeError("compact cache is full: raise decode_reserve before stage 2")
+        ops.cache_append(k[:, 0].contiguous(), v[:, 0].contiguous(), kc, vc, kv_len)
+        out = ops.sparse_attn(q[:, 0].contiguous(), kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), ck["kv_offsets"], kv_len,
+                              ck["kv_capacity"], scale=self.scaling, causal=True)
+        return self.o_proj(out.view(B, 1, -1)), None

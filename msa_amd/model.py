@@ -1,0 +1,117 @@
+"""Qwen3-shaped decoder hosting :class:`MemorySparseAttention` in every layer, with random-init
+weights, for the end-to-end sparse-generation workload (no checkpoint can be fetched here).  The
+dense parts (embedding, MLP, norms, LM head) are plain PyTorch-ROCm; they are the host model around
+the hot path, mirroring src/msa/model.py:51-255 without losses or training code."""
+from __future__ import annotations
+
+from typing import List, Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .cache import CustomDynamicCache, create_cache
+from .config import MSAConfig
+from .memory_sparse_attention import MemorySparseAttention, RMSNorm, rotary_embedding
+from .prefill import query_position_ids
+
+
+class MLP(nn.Module):
+    def __init__(self, config: MSAConfig):
+        super().__init__()
+        self.gate_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
+        self.up_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
+        self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=False)
+
+    def forward(self, x):
+        return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
+
+
+class MSADecoderLayer(nn.Module):
+    def __init__(self, config: MSAConfig, layer_idx: int):
+        super().__init__()
+        self.self_attn = MemorySparseAttention(config, layer_idx)
+        self.mlp = MLP(config)
+        self.input_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+        self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+
+    def forward(self, hidden_states, doc_ids, attention_mask, position_embeddings, past_key_value):
+        h, _ = self.self_attn(self.input_layernorm(hidden_states), doc_ids, attention_mask, position_embeddings,
+                              past_key_value)
+        hidden_states = hidden_states + h
+        return hidden_states + self.mlp(self.post_attention_layernorm(hidden_states))
+
+
+class MSAModel(nn.Module):
+    def __init__(self, config: MSAConfig):
+        super().__init__()
+        self.config = config
+        self.embed_tokens = nn.Embedding(config.vocab_size, config.hidden_size)
+        self.layers = nn.ModuleList(MSADecoderLayer(config, i) for i in range(config.num_hidden_layers))
+        self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+
+    def forward(self, input_ids, attention_mask, position_ids, past_key_values, doc_ids):
+        h = self.embed_tokens(input_ids)
+        pe = rotary_embedding(position_ids, self.config.head_dim, self.config.rope_theta, h.dtype)
+        for layer in self.layers:
+            h = layer(h, doc_ids, attention_mask, pe, past_key_values)
+        return self.norm(h)
+
+
+class MSAForCausalLM(nn.Module):
+    def __init__(self, config: MSAConfig):
+        super().__init__()
+        self.config = config
+        self.model = MSAModel(config)
+        self.lm_head = nn.Linear(config.hidden_size, config.vocab_size, bias=False)
+
+    @torch.no_grad()
+    def init_random(self, std: float = 0.02, seed: int = 0):
+        g = torch.Generator(device="cpu").manual_seed(seed)
+        for p in self.parameters():
+            if p.dim() > 1:
+                p.copy_(torch.randn(p.shape, generator=g).mul_(std).to(p.dtype))
+        return self
+
+    @torch.no_grad()
+    def generate_greedy(self, input_ids, attention_mask, doc_ids, max_new_tokens: int, top_k_docs: Optional[int] = None,
+                        require_recall_topk: bool = False, past_key_values: Optional[CustomDynamicCache] = None):
+        """Stage 2 on the (left-padded) query batch, then ``max_new_tokens`` greedy decode steps.
+        Positions follow the reference: queries start at ``3 + top_k`` (src/msa_service.py:1823-1836),
+        padding repeats the first position, each decode step advances by one
+        (src/msa/generate.py:102-105).  Returns ``(tokens [B, max_new_tokens], cache)``."""
+        B, S = input_ids.shape
+        cfg = self.config
+        k = cfg.msa_config.top_k_docs if top_k_docs is None else top_k_docs
+        cache = past_key_values or create_cache()
+        cache.meta["require_recall_topk"] = require_recall_topk
+        for i in range(cfg.num_hidden_layers):
+            cache.record_kwargs(i, {"stage": "prefill_stage2"})
+        n_valid = attention_mask.sum(dim=1).tolist()
+        pos = torch.tensor([query_position_ids(n, k, 3, S - n) for n in n_valid], dtype=torch.long, device=input_ids.device)
+        h = self.model(input_ids, attention_mask, pos, cache, doc_ids)
+        tok = self.lm_head(h[:, -1:]).argmax(-1)
+        out = [tok]
+        for i in range(cfg.num_hidden_layers):
+            cache.cache_kwargs[i]["stage"] = "generate"
+        next_pos = pos[:, -1:] + 1
+        ones = torch.ones((B, 1), dtype=attention_mask.dtype, device=input_ids.device)
+        gen_ids = torch.full((B, 1), -1, dtype=doc_ids.dtype, device=input_ids.device)
+        for _ in range(max_new_tokens - 1):
+            h = self.model(tok, ones, next_pos, cache, gen_ids)
+            tok = self.lm_head(h).argmax(-1)
+            out.append(tok)
+            next_pos = next_pos + 1
+        return torch.cat(out, dim=1), cache
+
+
+def encode_block(model: MSAForCausalLM, block_input, device) -> CustomDynamicCache:
+    """Runs stage 1 over one packed block and returns the cache holding its pooled K / V / K_r
+    (the inference half of src/prefill.py:248-305)."""
+    cache = create_cache()
+    for i in range(model.config.num_hidden_layers):
+        cache.record_kwargs(i, {"stage": "prefill_stage1"})
+    with torch.no_grad():
+        model.model(block_input.doc_input_ids.to(device), block_input.doc_attention_mask.to(device),
+                    block_input.position_ids.to(device), cache, block_input.doc_ids.to(device))
+    return cache

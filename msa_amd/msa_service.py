@@ -1,0 +1,268 @@
+"""Memory bank and query service with the reference's call surface
+(src/msa_service.py: ``BlockDesc`` :191-231, ``Memory`` :269-828, ``MSAService.doc_query`` :1133-1314),
+single GPU, every tensor operation done by the HIP library.
+
+Bank layout (differs from the reference on purpose): pooled tensors are chunk-major ``[C, Hkv, D]``
+— K_r resident in HBM, K / V in pinned host memory — so a chunk's routing key is one contiguous
+2 KB row for the scoring kernel and a document's K / V is one contiguous range for the gather.
+Reference-shaped views (``[1, Hkv, C, D]``, ``[Hkv, n, D]``) are handed out where its API says so.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from . import ops
+from .cache import CustomDynamicCache
+from .config import GenerateConfig, MemoryConfig, ModelConfig, MSAConfig
+from .prefill import Document
+
+
+def cumulative_concat(tensors: Sequence[torch.Tensor]) -> torch.Tensor:
+    """Concatenates per-block 1-based pool ids into bank-wide ids: each block is shifted by the last
+    id of everything before it (src/utils/tools.py:34-55)."""
+    out, shift = [], 0
+    for t in tensors:
+        out.append(t + shift)
+        shift += int(t[-1])
+    return torch.cat(out)
+
+
+@dataclass
+class BlockDesc:
+    """Bank description (src/msa_service.py:191-231): tables carry a dummy slot 0."""
+    docs: List[Document] = None
+    tmp_doc_ids: List[torch.Tensor] = None
+    pool_ids: torch.Tensor = None
+    pool_ids_cpu: torch.Tensor = None
+    doc_ids: torch.Tensor = None
+    doc_ids_cpu: torch.Tensor = None
+    doc_offsets_cpu: torch.Tensor = None
+    doc_lens_cpu: torch.Tensor = None
+
+    def init_docs(self, docs: List[Document], device):
+        self.docs = docs
+        self.doc_ids_cpu = torch.tensor([0] + [d.doc_id for d in docs], dtype=torch.long)
+        self.doc_ids = self.doc_ids_cpu.to(device)
+        self.tmp_doc_ids = []
+        lens = [0] + [d.num_chunks for d in docs]
+        self.doc_lens_cpu = torch.tensor(lens, dtype=torch.long)
+        self.doc_offsets_cpu = torch.cumsum(torch.tensor([0] + lens[:-1], dtype=torch.long), dim=0)
+
+    def create_global_doc_ids(self, local_doc_ids):
+        return self.doc_ids[local_doc_ids]
+
+    def merge_poolig_doc_id(self, device):
+        self.pool_ids_cpu = cumulative_concat([t.cpu() for t in self.tmp_doc_ids])
+        self.pool_ids = self.pool_ids_cpu.to(device)
+        self.tmp_doc_ids.clear()
+
+    def chunks(self) -> int:
+        return sum(d.num_chunks for d in self.docs)
+
+    @property
+    def nr_docs(self) -> int:
+        return len(self.docs)
+
+
+class MemoryClientBase:
+    """What the layer calls (src/msa_service.py:259-264)."""
+
+    def get_template_prefix_kvcaches(self, layer_idx: int):
+        raise NotImplementedError
+
+    def doc_query(self, query_states: torch.Tensor, attention_mask: torch.Tensor, layer_idx: int):
+        raise NotImplementedError
+
+
+def _chunk_major(t: torch.Tensor) -> torch.Tensor:
+    """``[1, Hkv, C, D]`` (reference) or ``[C, Hkv, D]`` (native) -> ``[C, Hkv, D]`` view."""
+    return t[0].transpose(0, 1) if t.dim() == 4 else t
+
+
+class Memory:
+    """Tiered bank + scorer.  Fill it with :meth:`begin`, one :meth:`add_block` per stage-1 block and
+    :meth:`finish`; then :meth:`prefill_stage2` scores queries against it."""
+
+    def __init__(self, gpu_id: int, generate_config: GenerateConfig, model_config: ModelConfig,
+                 memory_config: MemoryConfig, msa_model_config: Optional[MSAConfig] = None):
+        self.gpu_id = gpu_id
+        self.device = torch.device(f"cuda:{gpu_id}")
+        self.generate_config, self.model_config, self.memory_config = generate_config, model_config, memory_config
+        self.msa_model_config = msa_model_config or MSAConfig()
+        cfg = self.msa_model_config
+        n_layers = cfg.num_hidden_layers
+        self.router_layer_ids = sorted(range(n_layers) if model_config.router_layer_idx == "all"
+                                       else (int(x) for x in model_config.router_layer_idx.split(",")))
+        self.num_key_value_groups = cfg.num_attention_heads // cfg.num_key_value_heads
+        mc = cfg.msa_config
+        self.head_reduce_method, self.query_reduce_method = mc.head_reduce_method, mc.query_reduce_method
+        self.chunk_reduce_method, self.aux_loss_method = mc.chunk_reduce_method, mc.aux_loss_method
+        self.decouple_router = mc.decouple_router
+        # the kernels implement the shipped reductions only (src/msa_service.py:742-813 has others)
+        for name, got, want in (("head_reduce_method", self.head_reduce_method, "mean"),
+                                ("query_reduce_method", self.query_reduce_method, "max")):
+            if got != want:
+                raise NotImplementedError(f"Unsupported {name.split('_')[0]} reduce method: {got}")
+        if self.chunk_reduce_method != "max":
+            raise ValueError(f"Invalid chunk reduction method: {self.chunk_reduce_method}")
+        # -1 marks "already cosine, do not scale" exactly as the reference does (:318-321)
+        self.scaling = -1.0 if (self.aux_loss_method == "INFONCE" and self.decouple_router) else cfg.head_dim ** -0.5
+        self.block_desc = BlockDesc()
+        self.template_prefix_kvcache: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = {}
+        self.bank: Optional[ops.Bank] = None
+        self._rk: Dict[int, torch.Tensor] = {}
+        self._k: Dict[int, torch.Tensor] = {}
+        self._v: Dict[int, torch.Tensor] = {}
+        self._kv_offset = 0
+        self._layer_slot = {layer: i for i, layer in enumerate(self.router_layer_ids)}
+
+    def num_model_layers(self) -> int:
+        return self.msa_model_config.num_hidden_layers
+
+    # ---------------------------------------------------------------- bank fill (:497-582)
+    def begin(self, docs: List[Document]) -> None:
+        self.block_desc.init_docs(docs, self.device)
+        self._kv_offset = 0
+
+    def _init_block_data(self, Hkv: int, D: int, dtype: torch.dtype) -> None:
+        C = self.block_desc.chunks()
+        for layer in self.router_layer_ids:
+            self._rk[layer] = torch.empty((C, Hkv, D), dtype=dtype, device=self.device)
+            self._k[layer] = torch.empty((C, Hkv, D), dtype=dtype, pin_memory=True)
+            self._v[layer] = torch.empty((C, Hkv, D), dtype=dtype, pin_memory=True)
+
+    def add_block(self, past_key_values: CustomDynamicCache) -> None:
+        """Copies one stage-1 block's pooled K / V / K_r into the bank at the running chunk offset
+        and records its pooled document ids (:541-569)."""
+        if not self.template_prefix_kvcache:
+            kw = past_key_values.cache_kwargs
+            self.template_prefix_kvcache = {
+                layer: (kw[layer]["template_prefix_kcache"].to(self.device), kw[layer]["template_prefix_vcache"].to(self.device))
+                for layer in range(self.num_model_layers()) if "template_prefix_kcache" in kw.get(layer, {})}
+        meta_chunks = None
+        for layer in self.router_layer_ids:
+            k, v = past_key_values.get_kvcache(layer)
+            rk = past_key_values.get_router_kcache(layer)
+            if rk is None:
+                raise ValueError("this bank needs decoupled routing keys (router_k_proj) for every router layer")
+            k, v, rk = _chunk_major(k), _chunk_major(v), _chunk_major(rk)
+            if not self._rk:
+                self._init_block_data(k.shape[1], k.shape[2], k.dtype)
+            if layer == self.router_layer_ids[0]:
+                self.block_desc.tmp_doc_ids.append(past_key_values.cache_kwargs[layer]["pooled_doc_ids"])
+            n = k.shape[0]
+            if meta_chunks is None:
+                meta_chunks = n
+            assert meta_chunks == n, f"expect meta_chunks {meta_chunks} but got {n}"
+            total = self.block_desc.chunks()
+            assert self._kv_offset + n <= total, f"overflow: offset {self._kv_offset}, meta_chunks {n}, total_chunks {total}"
+            s = slice(self._kv_offset, self._kv_offset + n)
+            self._k[layer][s].copy_(k)
+            self._v[layer][s].copy_(v)
+            self._rk[layer][s].copy_(rk)
+        self._kv_offset += meta_chunks or 0
+
+    def finish(self) -> None:
+        """Merges the pooled ids, checks them against the documents' chunk counts and creates the
+        native bank handle (replaces ``_generate_slice``: no slices, no transposed views)."""
+        desc = self.block_desc
+        desc.merge_poolig_doc_id(self.device)
+        counts = torch.bincount(desc.pool_ids_cpu, minlength=desc.nr_docs + 1)
+        if not torch.equal(counts, desc.doc_lens_cpu):
+            raise AssertionError("pooled document ids do not match the documents' chunk counts")
+        if self._kv_offset != desc.chunks():
+            raise AssertionError(f"bank holds {self._kv_offset} chunks, documents need {desc.chunks()}")
+        off = torch.cat([desc.doc_offsets_cpu[1:], torch.tensor([desc.chunks()])])      # [n_docs + 1], 0-based docs
+        ref = self._rk[self.router_layer_ids[0]]
+        self.bank = ops.Bank(len(self.router_layer_ids), off.tolist(), desc.doc_ids_cpu[1:].tolist(), ref.shape[1],
+                             ref.shape[2], ref.dtype)
+        for layer, slot in self._layer_slot.items():
+            self.bank.set_layer(slot, self._rk[layer], self._k[layer], self._v[layer])
+
+    def get_max_local_pool_doc_id(self) -> int:
+        return int(self.block_desc.pool_ids_cpu[-1])
+
+    def get_template_prefix_kvcaches(self, layer_idx: int):
+        return self.template_prefix_kvcache[layer_idx]
+
+    # ---------------------------------------------------------------- scorer (:703-828)
+    def _route(self, layer_idx: int, q_bshd: torch.Tensor, mask_bs: Optional[torch.Tensor], mode: str, scale: float):
+        top_k = self.model_config.doc_top_k
+        scores, doc, gid = ops.route_topk(self.bank, self._layer_slot[layer_idx], q_bshd, mask_bs, mode, scale, top_k)
+        return scores, doc, gid
+
+    def prefill_stage2(self, layer_idx: int, query_states: torch.Tensor, query_mask: torch.Tensor):
+        """``query_states [B, Hkv, G, S, D]`` already scaled / normalised by the caller, ``query_mask
+        [B, 1, 1, S, 1]`` -> ``(scores [B, k], local_ids [B, k] 1-based, global_ids [B, k])`` with
+        ``k = min(doc_top_k, nr_docs + 1)``; when the bank has fewer than ``doc_top_k`` documents
+        the dummy slot 0 fills the tail with the dtype's lowest value, as ``torch.topk`` over the
+        reference's score table does."""
+        B, Hkv, G, S, D = query_states.shape
+        q = query_states.permute(0, 3, 1, 2, 4).reshape(B, S, Hkv * G, D).contiguous()
+        mask = query_mask.reshape(B, S)
+        scores, doc, gid = self._route(layer_idx, q, mask, "scaled_dot", 1.0)
+        dtype = query_states.dtype
+        k = min(self.model_config.doc_top_k, self.block_desc.nr_docs + 1)
+        lowest = torch.finfo(dtype).min
+        scores = scores[:, :k].clamp_min(lowest).to(dtype)
+        local = (doc[:, :k].long() + 1)                      # -1 (no document) becomes the dummy slot 0
+        scores = torch.where(local == 0, torch.full_like(scores, lowest), scores)
+        return scores, local, self.block_desc.create_global_doc_ids(local)
+
+
+class MSAService(Memory, MemoryClientBase):
+    """Single-GPU service: the reference's collectives (src/msa_service.py:1098-1131, 1163-1198,
+    1267-1283) are the identity at world size 1 and are not present."""
+
+    def __init__(self, gpu_id: int, generate_config: GenerateConfig, model_config: ModelConfig,
+                 memory_config: MemoryConfig, msa_model_config: Optional[MSAConfig] = None):
+        super().__init__(gpu_id, generate_config, model_config, memory_config, msa_model_config)
+        self.copy_stream = torch.cuda.Stream(device=self.device)
+        self._ids_host: Optional[torch.Tensor] = None
+
+    def setup_memory_client(self, model) -> None:
+        for _, module in model.named_modules():
+            if callable(getattr(module, "set_memory_client", None)):
+                module.set_memory_client(self)
+
+    def doc_query(self, query_states: torch.Tensor, query_mask: torch.Tensor, layer_idx: int,
+                  fused_normalize: bool = False, native_layout: bool = False):
+        """``query_states [B, Hq, S, D]`` (the layer's ``.transpose(1, 2)`` view, normalised by the
+        caller in cosine mode unless ``fused_normalize``), ``query_mask [B, S]`` bool.
+
+        Returns ``(K [Hkv, n, D], V [Hkv, n, D], scores [B, k], n_sel [B] int64, global_ids [B, k])``
+        as src/msa_service.py:1314 does — K / V are views of chunk-major ``[n, Hkv, D]`` buffers
+        (pass ``native_layout=True`` to get those).  Within a sample the selected documents'
+        chunks come in ascending bank order, each document once; picks whose score is <= -1e9 are
+        dropped (:1190-1191).  The host copies run on a side stream; the current stream waits for
+        them before returning."""
+        B, Hq, S, D = query_states.shape
+        q = query_states.transpose(1, 2)
+        if not q.is_contiguous():
+            q = q.contiguous()
+        if fused_normalize:
+            mode, scale = "cosine", 1.0
+        else:
+            mode, scale = "scaled_dot", (1.0 if self.scaling < 0 else self.scaling)
+        scores, doc, gid = self._route(layer_idx, q, query_mask, mode, scale)
+        valid = scores > -1e9
+        doc = torch.where(valid, doc, torch.full_like(doc, -1))
+        if self._ids_host is None or self._ids_host.shape != doc.shape:
+            self._ids_host = torch.empty(doc.shape, dtype=torch.int32, pin_memory=True)
+        self._ids_host.copy_(doc, non_blocking=True)
+        torch.cuda.current_stream().synchronize()            # the ids must be on the host to address pinned K / V
+        k_sel, v_sel, cu = ops.gather_kv(self.bank, self._layer_slot[layer_idx], self._ids_host, self.device,
+                                         stream=self.copy_stream)
+        torch.cuda.current_stream().wait_stream(self.copy_stream)
+        k_sel.record_stream(torch.cuda.current_stream())
+        v_sel.record_stream(torch.cuda.current_stream())
+        n_sel = (cu[1:] - cu[:-1]).to(self.device)
+        dtype = query_states.dtype
+        scores = scores.clamp_min(torch.finfo(dtype).min).to(dtype)
+        gid = torch.where(doc >= 0, gid, torch.zeros_like(gid))
+        if native_layout:
+            return k_sel, v_sel, scores, n_sel, gid
+        return k_sel.permute(1, 0, 2), v_sel.permute(1, 0, 2), scores, n_sel, gid

@@ -1,0 +1,239 @@
+"""GPU tests of the reference-shaped host interface: ``MemorySparseAttention`` (stage 1, stage 2,
+decode), ``Memory.prefill_stage2`` / ``MSAService.doc_query`` and the greedy loop.  Dense
+projections are re-done in fp64 torch on the CPU with the layer's own weights; everything the HIP
+library computes is checked against the closed-form oracle."""
+import copy
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import closed_form as cf
+
+pytestmark = pytest.mark.gpu
+
+P, HID, HQ, HKV, D, TOPK = 8, 256, 4, 2, 128, 3
+HEAD_IDS = [7, 8, 9]
+TOL = 3e-5
+
+
+def say(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def env():
+    if not torch.cuda.is_available():
+        pytest.fail("no GPU visible")
+    from msa_amd import config, memory_sparse_attention as msa, model, msa_service, prefill
+    cfg = config.MSAConfig(hidden_size=HID, num_hidden_layers=2, num_attention_heads=HQ, num_key_value_heads=HKV,
+                           head_dim=D, intermediate_size=512, vocab_size=500,
+                           msa_config=dict(config.default_msa_config(), top_k_docs=TOPK, pooling_kernel_size=P,
+                                           router_layer_idx="1"))
+    return dict(cfg=cfg, config=config, msa=msa, model=model, svc=msa_service, prefill=prefill)
+
+
+def _layer(env, seed=0):
+    torch.manual_seed(seed)
+    layer = env["msa"].MemorySparseAttention(env["cfg"], 1).float()
+    with torch.no_grad():
+        for p in layer.parameters():
+            if p.dim() > 1:
+                p.copy_(torch.randn(p.shape) * 0.08)
+            else:
+                p.copy_(1.0 + 0.1 * torch.randn(p.shape))
+    return layer.eval()
+
+
+def _tables(env, position_ids):
+    cos, sin = env["msa"].rotary_embedding(position_ids, D, env["cfg"].rope_theta, torch.float32)
+    return cos, sin
+
+
+def _docs(env, lens, first_id=100):
+    pf = env["prefill"]
+    g = np.random.default_rng(5)
+    return [pf.Document(doc=f"d{i}", doc_id=first_id + i, num_chunks=pf.num_chunks(n, P),
+                        input_ids=[int(x) for x in g.integers(10, 400, size=n)]) for i, n in enumerate(lens)]
+
+
+def test_layer_stage1_stage2_decode_against_oracle(env):
+    say("layer: stage 1 -> bank -> stage 2 -> decode")
+    pf, svc_mod = env["prefill"], env["svc"]
+    layer = _layer(env)
+    layer64 = copy.deepcopy(layer).double()
+    layer = layer.cuda()
+    lens = [5, 8, 17, 1, 30, 9, 16, 23, 12]
+    docs = _docs(env, lens)
+    blocks = pf.split_docs(docs, 8)
+    assert len(blocks) >= 2
+    service = svc_mod.MSAService(0, env["config"].GenerateConfig(devices=[0]),
+                                 env["config"].ModelConfig(doc_top_k=TOPK, pooling_kernel_size=P, router_layer_idx="1"),
+                                 env["config"].MemoryConfig(pooling_kernel_size=P), env["cfg"])
+    service.begin(docs)
+    g = torch.Generator().manual_seed(3)
+    bank_k, bank_v, bank_rk, prefix = [], [], [], None
+    for blk in blocks:
+        inp = pf.prepare_block_inputs(blk, HEAD_IDS, P)
+        T = inp.doc_ids.shape[1]
+        hs = torch.randn((1, T, HID), generator=g)
+        cos, sin = _tables(env, inp.position_ids)
+        cache = env["model"].create_cache()
+        cache.record_kwargs(1, {"stage": "prefill_stage1"})
+        with torch.no_grad():
+            out, _ = layer(hs.cuda(), inp.doc_ids.cuda(), inp.doc_attention_mask.cuda(), (cos.cuda(), sin.cuda()), cache)
+            q64, k64, v64 = layer64._project(hs.double(), (cos.double(), sin.double()))
+            rk64 = layer64.router_k_proj(hs.double()).view(T, HKV, D)
+        _, _, cs, cl, cd = cf.chunk_table(inp.doc_lens, P, 3)
+        want_k, want_v = cf.pool_chunks(k64[0], cs, cl), cf.pool_chunks(v64[0], cs, cl)
+        want_rk = cf.l2_normalize(cf.pool_chunks(rk64, cs, cl))
+        pk, pv = cache.get_kvcache(1)
+        assert pk.shape == (1, HKV, len(cs), D)                              # the reference's [1, Hkv, C, D] view
+        assert cf.rel_err(pk[0].transpose(0, 1).cpu(), want_k) < TOL
+        assert cf.rel_err(pv[0].transpose(0, 1).cpu(), want_v) < TOL
+        assert cf.rel_err(cache.get_router_kcache(1)[0].transpose(0, 1).cpu(), want_rk) < TOL
+        kw = cache.cache_kwargs[1]
+        assert kw["pooled_doc_ids"].cpu().tolist() == (cd + 1).tolist()      # 1-based within the block
+        assert kw["template_prefix_kcache"].shape == (1, HKV, 3, D)
+        assert cf.rel_err(kw["template_prefix_kcache"][0].transpose(0, 1).cpu(), k64[0, :3]) < TOL
+        # document-wise causal attention, template head as its own segment
+        seg = [3] + inp.doc_lens
+        edges = np.concatenate([[0], np.cumsum(seg)])
+        want_attn = cf.attention_ragged(q64[0], edges, k64[0], v64[0], edges, causal=True)
+        with torch.no_grad():
+            want_out = layer64.o_proj(want_attn.reshape(1, T, HQ * D))
+        assert cf.rel_err(out.cpu(), want_out) < TOL
+        bank_k.append(want_k); bank_v.append(want_v); bank_rk.append(want_rk)
+        if prefix is None:
+            prefix = (k64[0, :3], v64[0, :3])
+        service.add_block(cache)
+    service.finish()
+    bank_k, bank_v, bank_rk = torch.cat(bank_k), torch.cat(bank_v), torch.cat(bank_rk)
+    _, dco, _, _, _ = cf.chunk_table(lens, P)
+    assert service.block_desc.pool_ids_cpu.tolist() == (np.repeat(np.arange(len(lens)), np.diff(dco)) + 1).tolist()
+    layer.set_memory_client(service)
+
+    # ---- stage 2: two left-padded queries
+    n_q = [7, 4]
+    B, S = 2, max(n_q)
+    hs2 = torch.randn((B, S, HID), generator=g)
+    mask = torch.tensor([[1] * 7, [0] * 3 + [1] * 4])
+    pos = torch.tensor([pf.query_position_ids(n, TOPK, 3, S - n) for n in n_q])
+    cos, sin = _tables(env, pos)
+    cache2 = env["model"].create_cache()
+    cache2.meta["require_recall_topk"] = True
+    cache2.record_kwargs(1, {"stage": "prefill_stage2"})
+    dz = torch.zeros((B, S), dtype=torch.long)
+    with torch.no_grad():
+        out2, _ = layer(hs2.cuda(), dz.cuda(), mask.cuda(), (cos.cuda(), sin.cuda()), cache2)
+        q64, k64, v64 = layer64._project(hs2.double(), (cos.double(), sin.double()))
+        rq64 = layer64.router_q_proj(hs2.double()).view(B, S, HQ, D)
+    ds = cf.doc_scores(cf.chunk_scores(rq64, mask.bool(), bank_rk, "cosine"), dco)
+    want_s, want_i = cf.topk_docs(ds, TOPK)
+    recall = cache2.cache_kwargs[1]["recall_topk"]
+    got_i = torch.tensor([[d - 100 for d in r["topk_doc_ids"]] for r in recall])
+    assert not cf.topk_acceptable(ds, got_i, TOPK, gap=1e-4)
+    if float((want_s[:, :-1] - want_s[:, 1:]).min()) > 1e-4:
+        assert torch.equal(got_i, want_i)
+    assert cf.rel_err(torch.tensor([r["score"] for r in recall]), torch.gather(ds, 1, got_i)) < TOL
+    mk, mv, cu_sel, _ = cf.gather_selected(bank_k, bank_v, dco, got_i)
+    want_rows = []
+    for b in range(B):
+        lo = S - n_q[b]
+        kk = torch.cat([prefix[0], mk[cu_sel[b]:cu_sel[b + 1]], k64[b, lo:]])
+        vv = torch.cat([prefix[1], mv[cu_sel[b]:cu_sel[b + 1]], v64[b, lo:]])
+        want_rows.append((cf.attention(q64[b, lo:], kk, vv, causal=True), kk, vv))
+    with torch.no_grad():
+        for b in range(B):
+            lo = S - n_q[b]
+            want_out = layer64.o_proj(want_rows[b][0].reshape(1, n_q[b], HQ * D))
+            assert cf.rel_err(out2[b:b + 1, lo:].cpu(), want_out) < TOL
+            assert float(out2[b, :lo].abs().max()) == 0.0 if lo else True
+    kw2 = cache2.cache_kwargs[1]
+    assert kw2["kv_lengths"].cpu().tolist() == [3 + int(cu_sel[b + 1] - cu_sel[b]) + n_q[b] for b in range(B)]
+
+    # ---- two decode steps
+    for i in range(cache2.get_layer_length()):
+        cache2.cache_kwargs[1]["stage"] = "generate"
+    ctx = [(r[1], r[2]) for r in want_rows]
+    for step in range(2):
+        hs3 = torch.randn((B, 1, HID), generator=g)
+        pos3 = pos[:, -1:] + 1 + step
+        cos, sin = _tables(env, pos3)
+        with torch.no_grad():
+            out3, _ = layer(hs3.cuda(), torch.full((B, 1), -1).cuda(), torch.ones(B, 1, dtype=torch.long).cuda(),
+                            (cos.cuda(), sin.cuda()), cache2)
+            q64, k64, v64 = layer64._project(hs3.double(), (cos.double(), sin.double()))
+            for b in range(B):
+                ctx[b] = (torch.cat([ctx[b][0], k64[b]]), torch.cat([ctx[b][1], v64[b]]))
+                want = layer64.o_proj(cf.attention(q64[b], ctx[b][0], ctx[b][1]).reshape(1, 1, HQ * D))
+                assert cf.rel_err(out3[b:b + 1].cpu(), want) < TOL
+
+    # ---- the scorer / client surface with the reference's argument conventions
+    with torch.no_grad():
+        rq = torch.nn.functional.normalize(layer.router_q_proj(hs2.cuda()).view(B, S, HQ, D).transpose(1, 2), p=2, dim=-1)
+    q5 = rq.reshape(B, HKV, HQ // HKV, S, D)                                 # [B, Hkv, G, S, D], cosine: not scaled
+    m5 = mask.bool().cuda().view(B, 1, 1, S, 1)
+    s, local, gids = service.prefill_stage2(1, q5, m5)
+    assert s.shape == (B, TOPK) and local.dtype == torch.int64
+    assert not cf.topk_acceptable(ds, local.cpu() - 1, TOPK, gap=1e-4)       # local ids are 1-based
+    assert torch.equal(gids.cpu(), local.cpu() + 99)
+    K, V, s2, n_sel, g2 = service.doc_query(rq, mask.bool().cuda(), 1)
+    assert K.shape == (HKV, int(cu_sel[-1]), D) and V.shape == K.shape        # the reference's [Hkv, n, D]
+    assert n_sel.cpu().tolist() == np.diff(cu_sel).tolist() and n_sel.dtype == torch.int64
+    assert cf.rel_err(K.permute(1, 0, 2).cpu(), mk) < TOL and cf.rel_err(V.permute(1, 0, 2).cpu(), mv) < TOL
+    assert torch.equal(g2.cpu(), got_i + 100)
+
+    # fewer documents than top-k: the dummy slot 0 pads the tail with the dtype's lowest value
+    small = svc_mod.MSAService(0, env["config"].GenerateConfig(devices=[0]),
+                               env["config"].ModelConfig(doc_top_k=16, pooling_kernel_size=P, router_layer_idx="1"),
+                               env["config"].MemoryConfig(pooling_kernel_size=P), env["cfg"])
+    small.block_desc = service.block_desc
+    small.bank, small._layer_slot = service.bank, service._layer_slot
+    s, local, gids = small.prefill_stage2(1, q5, m5)
+    assert s.shape == (B, len(lens) + 1) and (local[:, -1] == 0).all() and (gids[:, -1] == 0).all()
+    assert float(s[0, -1]) == torch.finfo(torch.float32).min
+    assert sorted(local[0, :-1].cpu().tolist()) == list(range(1, len(lens) + 1))
+
+
+def test_unsupported_reductions_raise(env):
+    say("unsupported reduce methods")
+    cfgm = env["config"]
+    bad = cfgm.MSAConfig(msa_config=dict(cfgm.default_msa_config(), head_reduce_method="max"))
+    with pytest.raises(NotImplementedError, match="Unsupported head reduce method"):
+        env["svc"].Memory(0, cfgm.GenerateConfig(devices=[0]), cfgm.ModelConfig(), cfgm.MemoryConfig(), bad)
+    bad = cfgm.MSAConfig(msa_config=dict(cfgm.default_msa_config(), chunk_reduce_method="mean"))
+    with pytest.raises(ValueError, match="Invalid chunk reduction method"):
+        env["svc"].Memory(0, cfgm.GenerateConfig(devices=[0]), cfgm.ModelConfig(), cfgm.MemoryConfig(), bad)
+    layer = _layer(env).cuda()
+    with pytest.raises(Exception, match="error!"):
+        layer(torch.zeros(1, 1, HID).cuda(), torch.zeros(1, 1).long().cuda())
+
+
+def test_model_greedy_generation_runs_and_is_deterministic(env):
+    say("model: encode -> bank -> greedy generation (bf16)")
+    pf, svc_mod, M = env["prefill"], env["svc"], env["model"]
+    model = M.MSAForCausalLM(env["cfg"]).init_random(0.05, seed=1).to(torch.bfloat16).cuda().eval()
+    lens = [20, 33, 9, 41, 16, 27]
+    docs = _docs(env, lens, first_id=0)
+    service = svc_mod.MSAService(0, env["config"].GenerateConfig(devices=[0]),
+                                 env["config"].ModelConfig(doc_top_k=TOPK, pooling_kernel_size=P, router_layer_idx="1"),
+                                 env["config"].MemoryConfig(pooling_kernel_size=P), env["cfg"])
+    service.begin(docs)
+    for blk in pf.split_docs(docs, 12):
+        service.add_block(M.encode_block(model, pf.prepare_block_inputs(blk, HEAD_IDS, P), "cuda"))
+    service.finish()
+    assert set(service.template_prefix_kvcache) == {0, 1}                    # every layer keeps its template prefix
+    service.setup_memory_client(model)
+    ids = torch.tensor([[5, 6, 7, 8, 9, 10], [0, 0, 11, 12, 13, 14]]).cuda()
+    mask = torch.tensor([[1] * 6, [0, 0, 1, 1, 1, 1]]).cuda()
+    dz = torch.zeros_like(ids)
+    t1, c1 = model.generate_greedy(ids, mask, dz, 5, require_recall_topk=True)
+    t2, _ = model.generate_greedy(ids, mask, dz, 5)
+    assert t1.shape == (2, 5) and torch.equal(t1, t2)
+    rec = c1.cache_kwargs[1]["recall_topk"]
+    assert len(rec) == 2 and all(len(set(r["topk_doc_ids"])) == TOPK for r in rec)
+    assert "recall_topk" not in c1.cache_kwargs[0]                           # layer 0 is not a router layer
+    assert c1.cache_kwargs[1]["kv_lengths"].cpu().tolist()[0] > c1.cache_kwargs[0]["kv_lengths"].cpu().tolist()[0]

@@ -1,0 +1,93 @@
+"""CPU tests of the host-side mirror of the reference interface: block input construction, bank
+metadata helpers, the cache container and configuration (no GPU, no HIP calls)."""
+import pytest
+import torch
+
+from msa_amd import cache as mcache
+from msa_amd import config as mconfig
+from msa_amd import prefill
+from oracle import closed_form as cf
+
+
+def _docs(lens, P):
+    return [prefill.Document(doc=f"d{i}", doc_id=100 + i, num_chunks=prefill.num_chunks(n, P), input_ids=list(range(n)))
+            for i, n in enumerate(lens)]
+
+
+def test_prepare_block_inputs_matches_oracle_layout():
+    P, lens, head = 8, [5, 8, 17, 1], [11, 12, 13]
+    inp = prefill.prepare_block_inputs(_docs(lens, P), head, P)
+    assert inp.doc_ids[0].tolist() == [-2] * 3 + [1] * 5 + [2] * 8 + [3] * 17 + [4]
+    assert inp.position_ids[0].tolist() == cf.doc_positions(lens, 3).tolist()      # restart at 0 per document
+    assert inp.chunk_sizes == [1, 1, 3, 1] and inp.num_chunks == 6
+    assert inp.doc_attention_mask.sum() == 3 + sum(lens)
+    assert inp.doc_input_ids[0, :3].tolist() == head
+    _, dco, _, _, _ = cf.chunk_table(lens, P, 3)
+    assert dco[-1] == inp.num_chunks
+    bad = _docs(lens, P)
+    bad[2].num_chunks = 2
+    with pytest.raises(AssertionError, match="pre calculated chunk"):
+        prefill.prepare_block_inputs(bad, head, P)
+    with pytest.raises(ValueError):
+        prefill.prepare_block_inputs([prefill.Document(doc_id=1)], head, P)
+
+
+def test_split_docs_budget_and_order():
+    docs = _docs([64, 64, 200, 8, 8, 8], 8)           # chunks 8, 8, 25, 1, 1, 1
+    blocks = prefill.split_docs(docs, 16)
+    assert [[d.doc_id for d in b] for b in blocks] == [[100, 101], [102], [103, 104, 105]]
+    assert prefill.split_docs(docs, 1000) == [docs]
+    assert prefill.split_docs([], 16) == []
+
+
+def test_query_positions_rule():
+    assert prefill.query_position_ids(3, 16) == [19, 20, 21]
+    assert prefill.query_position_ids(2, 16, left_pad=3) == [19, 19, 19, 19, 20]
+    assert prefill.query_position_ids(4, 16, 3, 1) == cf.query_positions(4, 16, 3, 1).tolist()
+
+
+def test_cumulative_concat_and_block_desc():
+    from msa_amd.msa_service import BlockDesc, cumulative_concat
+    a, b, c = torch.tensor([1, 1, 2, 3, 3]), torch.tensor([1, 2, 2]), torch.tensor([1])
+    assert cumulative_concat([a, b, c]).tolist() == [1, 1, 2, 3, 3, 4, 5, 5, 6]
+    desc = BlockDesc()
+    desc.init_docs(_docs([5, 8, 17], 8), "cpu")
+    assert desc.doc_ids_cpu.tolist() == [0, 100, 101, 102]
+    assert desc.doc_lens_cpu.tolist() == [0, 1, 1, 3]
+    assert desc.doc_offsets_cpu.tolist() == [0, 0, 1, 2]
+    assert desc.chunks() == 5 and desc.nr_docs == 3
+    assert desc.create_global_doc_ids(torch.tensor([[3, 1]])).tolist() == [[102, 100]]
+
+
+def test_cache_container():
+    c = mcache.create_cache()
+    c.record_kwargs(2, {"stage": "prefill_stage1"})
+    c.record_kwargs(2, {"x": 1})
+    assert c.cache_kwargs[2] == {"stage": "prefill_stage1", "x": 1} and c.get_layer_length() == 1
+    k1, v1 = torch.ones(1, 2, 3, 4), torch.zeros(1, 2, 3, 4)
+    c.update(k1, v1, 2)
+    c.update(2 * k1, v1, 2)
+    k, v = c.get_kvcache(2)
+    assert k.shape == (1, 2, 6, 4) and k[0, 0, 3, 0] == 2 and c.get_seq_length(2) == 6 and c.get_seq_length(0) == 0
+    assert c.get_router_kcache(2) is None
+    c.update_router_kcache(k1, 2)
+    assert c.get_router_kcache(2).shape == (1, 2, 3, 4) and c.get_router_kcache(0) is None
+    c.record_kwargs(2, {"compacked_key_cache": 1, "compacked_value_cache": 2, "recall_topk": 3})
+    c.clear_query()
+    assert "compacked_key_cache" not in c.cache_kwargs[2] and "recall_topk" not in c.cache_kwargs[2]
+    c.clear_kvcache()
+    assert c.key_cache == [] and c.get_seq_length(2) == 0
+
+
+def test_configs():
+    g = mconfig.GenerateConfig(devices=[0], template="QWEN3_INSTRUCT_TEMPLATE")
+    assert g.world == 1 and "{prompt}" in g.template["prompt"]
+    with pytest.raises(ValueError):
+        mconfig.GenerateConfig(template="NOPE")
+    m = mconfig.ModelConfig()
+    assert (m.doc_top_k, m.pooling_kernel_size, m.template_token_id, m.template_id_num) == (16, 64, -2, 3)
+    assert mconfig.MemoryConfig().slice_chunk_size == 16384
+    cfg = mconfig.MSAConfig(msa_config={"top_k_docs": 4})
+    assert cfg.msa_config.top_k_docs == 4 and cfg.msa_config.missing is None
+    d = mconfig.MSAConfig()
+    assert d.msa_config.router_layer_idx.split(",")[0] == "18" and d.num_key_value_heads == 8

@@ -122,6 +122,61 @@ def cpu_baseline(kr0, q0, doc_chunks, budget_s=25.0):
     return out, Cs
 
 
+def time_cuda(fn, reps, warm=2):
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / reps
+
+
+def extra_pooling(dev):
+    """configs[1]: chunk-mean pooling of K (rotated in the kernel), V and K_r (normalised) over 1M tokens of
+    ragged documents, bf16, 8 KV heads x 128, chunk 64; one layer per launch."""
+    from msa_amd import ops
+    lens = make_doc_lens(1_000_000, 1)
+    T = sum(lens)
+    g = torch.Generator(device=dev).manual_seed(11)
+    k, v, kr = (torch.randn((T, HKV, D), generator=g, device=dev).to(torch.bfloat16) for _ in range(3))
+    table = ops.chunk_table(lens, P, device=dev)
+    rope = ops.rope_tables(2048, D, 1e6, device=dev)
+    ms = time_cuda(lambda: ops.pool_chunks(k, v, kr, table, rope=rope, normalize_kr=True), 10)
+    by = 3 * T * HKV * D * 2 + 3 * table.C * HKV * D * 2
+    return {"workload": "configs[1]: 1M tokens, docs U[256,2048], K (RoPE fused) + V + K_r (normalised), bf16",
+            "tokens": T, "chunks": table.C, "ms_per_layer": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
+            "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4), "tokens_per_s": round(T / ms * 1e3)}
+
+
+def extra_decode(dev):
+    """configs[4] attention share: one decode step of one layer, B=16, 32 Q / 8 KV heads, context
+    3 + 16 docs x 18 chunks + 4096 local tokens, bf16, cache appended in place."""
+    from msa_amd import ops
+    B, L = 16, 3 + 288 + 4096
+    Lcap = L + 64
+    g = torch.Generator(device=dev).manual_seed(12)
+    kc = torch.randn((B, Lcap, HKV, D), generator=g, device=dev).to(torch.bfloat16)
+    vc = torch.randn((B, Lcap, HKV, D), generator=g, device=dev).to(torch.bfloat16)
+    q = torch.randn((B, HQ, D), generator=g, device=dev).to(torch.bfloat16)
+    kn, vn = q[:, :HKV].contiguous(), q[:, HKV:2 * HKV].contiguous()
+    kv_off = torch.arange(B, dtype=torch.int64, device=dev) * Lcap
+    kv_len = torch.full((B,), L, dtype=torch.int32, device=dev)
+
+    def step():                       # the context grows by one row per step, as in a real decode
+        ops.cache_append(kn, vn, kc, vc, kv_len)
+        ops.sparse_attn(q, kc.view(-1, HKV, D), vc.view(-1, HKV, D), kv_off, kv_len, Lcap)
+    ms = time_cuda(step, 20)
+    by = 2 * B * (L + 12) * HKV * D * 2        # mean context over the 22 steps run
+    return {"workload": "configs[4] attention share: 1 layer-step, B=16, L=4388, GQA 32/8, bf16",
+            "ms_per_layer_step": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
+            "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
+            "attention_only_tok_per_s_36_layers": round(B / (36 * ms) * 1e3)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -135,6 +190,7 @@ def main():
                     help="distinct pinned host K/V layer buffers (routed layers share them round-robin)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the pooling and decode-attention side measurements")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for rocprof FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -305,6 +361,10 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    extras = None
+    if not args.no_extras:
+        extras = {"pooling": extra_pooling(dev), "decode_attention": extra_decode(dev)}
+
     cpu = None
     if not args.no_cpu_baseline:
         times, Cs = cpu_baseline(krs[0], qs[0], doc_chunks)
@@ -327,7 +387,7 @@ def main():
                    "query_tokens": S, "top_k": TOPK, "kr_hbm_gb": round(C_total * HKV * D * 2 * L / 1e9, 1),
                    "host_kv_layer_buffers": n_host, "selected_chunks_per_layer": int(np.mean(sel_chunks)),
                    "mode": "cosine/mean-heads/max-tokens/max-chunks"},
-        "roofline": roof, "cpu_baseline": cpu, "hbm_regime_sweep": sweep, "parity": "needles exact on all layers",
+        "roofline": roof, "cpu_baseline": cpu, "hbm_regime_sweep": sweep, "other_kernels": extras, "parity": "needles exact on all layers",
     }
     print(json.dumps(out), flush=True)
 

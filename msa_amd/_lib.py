@@ -37,7 +37,7 @@ SIGNATURES = {
     "msa_assemble_context": (C.c_int, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp,
                                        _vp, _i32, _vp, _vp]),
     "msa_cache_append": (C.c_int, [_vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp]),
-    "msa_attn_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32]),
+    "msa_attn_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32, _i32]),
     "msa_sparse_attn": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32,
                                   _i32, _vp, _vp, _sz, _vp]),
 }

@@ -12,7 +12,7 @@
 namespace {
 
 constexpr int kAttnWaves = 4;
-constexpr int kSplitKeys = 256;   // keys per workgroup
+constexpr int kMinSplitKeys = 256;   // fewest keys worth a workgroup of its own
 constexpr int kMaxG = 8;
 
 template <typename T>
@@ -39,7 +39,8 @@ template <typename T, int G>
 __global__ __launch_bounds__(kAttnWaves * 64) void attn_partial_kernel(
     const T* __restrict__ q, const int32_t* __restrict__ cu_q, const T* __restrict__ k, const T* __restrict__ v,
     const int64_t* __restrict__ kv_off, const int32_t* __restrict__ kv_len, int32_t B, int32_t Hq, int32_t Hkv,
-    float scale_log2e, int32_t causal, int32_t n_split, float* __restrict__ part_ml, float* __restrict__ part_acc) {
+    float scale_log2e, int32_t causal, int32_t n_split, int32_t split_keys, float* __restrict__ part_ml,
+    float* __restrict__ part_acc) {
   __shared__ float sm_m[kAttnWaves][G], sm_l[kAttnWaves][G];
   __shared__ float sm_acc[kAttnWaves][G][kHeadDim];
 
@@ -49,8 +50,8 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_partial_kernel(
   const int sq = cu_q ? cu_q[b + 1] - q_first : 1;
   const int L = kv_len[b];
   const int visible = causal ? max(0, L - sq + (row - q_first) + 1) : L;
-  const int key0 = split * kSplitKeys;
-  const int key1 = min(visible, key0 + kSplitKeys);
+  const int key0 = split * split_keys;
+  const int key1 = min(visible, key0 + split_keys);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int slot = lane >> 4, j = lane & 15;
@@ -73,24 +74,52 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_partial_kernel(
     for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
   }
 
-  for (int kk = key0 + wave * 4 + slot; kk < key1; kk += kAttnWaves * 4) {
-    const int64_t off = (base + kk) * row_elems + g * kHeadDim + 8 * j;
-    float kx[8], vx[8];
-    ld8<T>(k + off, kx);
-    ld8<T>(v + off, vx);
+  // Keys in batches of kBatch steps: all K / V loads of a batch are issued before any arithmetic
+  // (bytes in flight), scores are reduced over the 16 lanes of a key with DPP row rotations, and
+  // the running softmax is rescaled once per batch.
+  constexpr int kBatch = 4;
+  constexpr int kStride = kAttnWaves * 4;          // keys between a lane's consecutive steps
+  for (int kb = key0 + wave * 4 + slot; kb < key1; kb += kStride * kBatch) {
+    float kx[kBatch][8], vx[kBatch][8];
+    bool ok[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int kk = kb + u * kStride;
+      ok[u] = kk < key1;
+      const int64_t off = (base + (ok[u] ? kk : kb)) * row_elems + g * kHeadDim + 8 * j;   // clamp: always in range
+      ld8<T>(k + off, kx[u]);
+      ld8<T>(v + off, vx[u]);
+    }
 #pragma unroll
     for (int h = 0; h < G; ++h) {
-      float s = 0.f;
+      float s[kBatch];
+      float mb = m[h];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) s += qv[h][i] * kx[i];
-      s += __shfl_xor(s, 1); s += __shfl_xor(s, 2); s += __shfl_xor(s, 4); s += __shfl_xor(s, 8);
-      const float mn = fmaxf(m[h], s);
-      const float alpha = exp2f(m[h] - mn);     // first key: exp2f(-inf) = 0
-      const float p = exp2f(s - mn);
-      m[h] = mn;
-      l[h] = l[h] * alpha + p;
+      for (int u = 0; u < kBatch; ++u) {
+        float d = 0.f;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[h][i] = acc[h][i] * alpha + p * vx[i];
+        for (int i = 0; i < 8; ++i) d += qv[h][i] * kx[u][i];
+        d += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, d), 0x128, 0xf, 0xf, false));
+        d += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, d), 0x124, 0xf, 0xf, false));
+        d += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, d), 0x122, 0xf, 0xf, false));
+        d += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, d), 0x121, 0xf, 0xf, false));
+        s[u] = ok[u] ? d : -INFINITY;
+        mb = fmaxf(mb, s[u]);
+      }
+      // mb is finite here: the batch's first key is always valid
+      const float alpha = exp2f(m[h] - mb);
+      float psum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[h][i] *= alpha;
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const float pu = exp2f(s[u] - mb);
+        psum += pu;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[h][i] += pu * vx[u][i];
+      }
+      l[h] = l[h] * alpha + psum;
+      m[h] = mb;
     }
   }
 
@@ -158,12 +187,26 @@ __global__ __launch_bounds__(kHeadDim) void attn_combine_kernel(const float* __r
   else out[rh * kHeadDim + d] = o;
 }
 
-inline int splits_for(int32_t max_kv) { return std::max(1, (max_kv + kSplitKeys - 1) / kSplitKeys); }
+// Splits of the key range: enough workgroups to fill the chip (about 2048) when there are few
+// (query row, KV head) pairs, a single pass over the keys when there are many.
+struct SplitPlan {
+  int n_split;
+  int split_keys;
+};
+inline SplitPlan plan_splits(int64_t total_q, int32_t Hkv, int32_t max_kv) {
+  const int64_t pairs = std::max<int64_t>(1, total_q * Hkv);
+  const int by_fill = (int)std::max<int64_t>(1, (2048 + pairs - 1) / pairs);
+  const int by_size = std::max(1, (max_kv + kMinSplitKeys - 1) / kMinSplitKeys);
+  const int n = std::min(by_fill, by_size);
+  const int keys = ((max_kv + n - 1) / n + 63) / 64 * 64;
+  return {(max_kv + keys - 1) / keys, keys};
+}
 
 template <typename T>
 int launch_attn(const void* q, const int32_t* cu_q, const void* k, const void* v, const int64_t* kv_off,
                 const int32_t* kv_len, int32_t B, int32_t total_q, int32_t Hq, int32_t Hkv, float scale,
-                int32_t causal, int32_t n_split, void* out, float* part_ml, float* part_acc, hipStream_t st) {
+                int32_t causal, SplitPlan plan, void* out, float* part_ml, float* part_acc, hipStream_t st) {
+  const int n_split = plan.n_split;
   const int G = Hq / Hkv;
   dim3 grid((unsigned)total_q, (unsigned)Hkv, (unsigned)n_split);
   const float sl2 = scale * 1.4426950408889634f;
@@ -171,7 +214,7 @@ int launch_attn(const void* q, const int32_t* cu_q, const void* k, const void* v
   case GG:                                                                                                         \
     attn_partial_kernel<T, GG><<<grid, kAttnWaves * 64, 0, st>>>(                                                  \
         static_cast<const T*>(q), cu_q, static_cast<const T*>(k), static_cast<const T*>(v), kv_off, kv_len, B, Hq, \
-        Hkv, sl2, causal, n_split, part_ml, part_acc);                                                             \
+        Hkv, sl2, causal, n_split, plan.split_keys, part_ml, part_acc);                                                             \
     break;
   switch (G) {
     MSA_ATTN_CASE(1)
@@ -192,9 +235,9 @@ int launch_attn(const void* q, const int32_t* cu_q, const void* k, const void* v
 
 }  // namespace
 
-extern "C" size_t msa_attn_workspace_bytes(int32_t total_q, int32_t Hq, int32_t D, int32_t max_kv) {
-  if (total_q <= 0 || Hq <= 0 || D <= 0 || max_kv <= 0) return 0;
-  const size_t n = (size_t)total_q * Hq * splits_for(max_kv);
+extern "C" size_t msa_attn_workspace_bytes(int32_t total_q, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_kv) {
+  if (total_q <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || max_kv <= 0) return 0;
+  const size_t n = (size_t)total_q * Hq * plan_splits(total_q, Hkv, max_kv).n_split;
   return align_up(n * 2 * sizeof(float), 256) + align_up(n * D * sizeof(float), 256);
 }
 
@@ -211,9 +254,10 @@ extern "C" int msa_sparse_attn(const void* q, const int32_t* cu_q, const void* k
   MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "msa_sparse_attn: bad dtype %d", dtype);
   MSA_REQUIRE(scale > 0.f, "msa_sparse_attn: scale must be positive");
   MSA_REQUIRE((int64_t)total_q * Hq < (int64_t)1 << 31 && total_q < 65536 * 32, "msa_sparse_attn: too many rows");
-  const int n_split = splits_for(max_kv);
+  const SplitPlan plan = plan_splits(total_q, Hkv, max_kv);
+  const int n_split = plan.n_split;
   MSA_REQUIRE(n_split <= 65535, "msa_sparse_attn: max_kv=%d too large", max_kv);
-  const size_t need = msa_attn_workspace_bytes(total_q, Hq, D, max_kv);
+  const size_t need = msa_attn_workspace_bytes(total_q, Hq, Hkv, D, max_kv);
   if (need > workspace_bytes) {
     msa_set_error("msa_sparse_attn: workspace of %zu bytes, need %zu", workspace_bytes, need);
     return MSA_ESIZE;
@@ -223,8 +267,8 @@ extern "C" int msa_sparse_attn(const void* q, const int32_t* cu_q, const void* k
   float* part_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + align_up(n * 2 * sizeof(float), 256));
   hipStream_t st = as_stream(stream);
   if (dtype == MSA_BF16)
-    return launch_attn<bf16_t>(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, n_split, out,
+    return launch_attn<bf16_t>(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, plan, out,
                                part_ml, part_acc, st);
-  return launch_attn<float>(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, n_split, out, part_ml,
+  return launch_attn<float>(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, plan, out, part_ml,
                             part_acc, st);
 }

@@ -216,19 +216,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     const int buf = kt & 1;
 #pragma unroll
     for (int sub = 0; sub < kSub; ++sub) {
-#ifndef MSA_ABLATE
-#define MSA_ABLATE 0
-#endif
       if (sub + 1 < kSub) {
-        if (MSA_ABLATE != 5) load_frags(buf, sub + 1, (sub + 1) & 1);
+        load_frags(buf, sub + 1, (sub + 1) & 1);
       } else if (kMore) {
-        if (MSA_ABLATE != 3) __syncthreads();
-        if (MSA_ABLATE != 5) load_frags(buf ^ 1, 0, 0);
+        __syncthreads();
+        load_frags(buf ^ 1, 0, 0);
         __builtin_amdgcn_sched_barrier(0);   // keep the last sub-step's MFMAs behind these reads
       }
       if (sub == 1 && kMore) {
-        if (MSA_ABLATE != 4 && MSA_ABLATE != 6) store_tile(buf ^ 1);
-        if (kt + 2 < k_tiles && MSA_ABLATE != 4 && MSA_ABLATE != 7) load_tile(kt + 2);
+        store_tile(buf ^ 1);
+        if (kt + 2 < k_tiles) load_tile(kt + 2);
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -242,14 +239,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   if (k_tiles > 1) load_tile(1);
   __syncthreads();
   load_frags(0, 0, 0);
-#if defined(MSA_ABLATE) && MSA_ABLATE == 9
-  for (int rep = 0; rep < 3; ++rep)
-#endif
   for (int kt = 0; kt + 1 < k_tiles; ++kt) k_tile(std::true_type{}, kt);
   k_tile(std::false_type{}, k_tiles - 1);
-#if defined(MSA_ABLATE) && MSA_ABLATE == 8
-  if (acc[0][0][0] != 123.456f) return;
-#endif
 
   // Epilogue.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of its 32x32 block.
 #pragma unroll

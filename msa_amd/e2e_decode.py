@@ -1,0 +1,107 @@
+"""End-to-end sparse generation at Qwen3-4B shape (BASELINE configs[4]): random-init bf16 weights,
+36 layers, routing on the upper 18, a synthetic pooled memory bank, top-16 documents, a 4K-token
+local context per query, batch 16, greedy decoding.
+
+    python -m msa_amd.e2e_decode [--bank-tokens 10000000] [--batch 16] [--context 4096] [--steps 256]
+
+Prints one JSON line with prefill time and decode tokens/s.  The bank is synthetic at the pooled
+level (N(0,1) rows, K_r L2-normalised): encoding 10M tokens through a 4B-parameter model is not part
+of what this measures.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+
+import numpy as np
+import torch
+
+from .config import GenerateConfig, MemoryConfig, ModelConfig, MSAConfig
+from .model import MSAForCausalLM
+from .msa_service import MSAService
+from .prefill import Document, num_chunks
+
+
+def build_service(cfg: MSAConfig, bank_tokens: int, seed: int = 0) -> MSAService:
+    dev = torch.device("cuda:0")
+    P = cfg.msa_config.pooling_kernel_size
+    g = np.random.default_rng(seed)
+    lens, left = [], bank_tokens
+    while left > 0:
+        n = min(int(g.integers(256, 2049)), left)
+        lens.append(n)
+        left -= n
+    docs = [Document(doc_id=i, num_chunks=num_chunks(n, P)) for i, n in enumerate(lens)]
+    C = sum(d.num_chunks for d in docs)
+    Hkv, D = cfg.num_key_value_heads, cfg.head_dim
+    svc = MSAService(0, GenerateConfig(devices=[0]),
+                     ModelConfig(doc_top_k=cfg.msa_config.top_k_docs, pooling_kernel_size=P,
+                                 router_layer_idx=cfg.msa_config.router_layer_idx),
+                     MemoryConfig(pooling_kernel_size=P), cfg)
+    tg = torch.Generator(device=dev).manual_seed(seed)
+    rk, k, v = {}, {}, {}
+    for layer in svc.router_layer_ids:
+        x = torch.randn((C, Hkv, D), generator=tg, device=dev)
+        rk[layer] = (x / x.norm(dim=-1, keepdim=True)).to(torch.bfloat16)
+        for store in (k, v):
+            h = torch.empty((C, Hkv, D), dtype=torch.bfloat16, pin_memory=True)
+            h.copy_(torch.randn((C, Hkv, D), generator=tg, device=dev).to(torch.bfloat16))
+            store[layer] = h
+    prefix = {l: (torch.randn((1, Hkv, 3, D), generator=tg, device=dev).to(torch.bfloat16),
+                  torch.randn((1, Hkv, 3, D), generator=tg, device=dev).to(torch.bfloat16))
+              for l in range(cfg.num_hidden_layers)}
+    svc.load_pooled(docs, rk, k, v, prefix)
+    return svc
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--bank-tokens", type=int, default=10_000_000)
+    ap.add_argument("--batch", type=int, default=16)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--layers", type=int, default=36)
+    args = ap.parse_args(argv)
+    if not torch.cuda.is_available():
+        sys.exit("e2e_decode: no GPU visible; the HIP path has no CPU fallback")
+    dev = torch.device("cuda:0")
+    cfg = MSAConfig(num_hidden_layers=args.layers)
+    if args.layers != 36:
+        half = args.layers // 2
+        cfg.msa_config.router_layer_idx = ",".join(str(i) for i in range(half, args.layers))
+    t0 = time.perf_counter()
+    with torch.device(dev):
+        model = MSAForCausalLM(cfg).to(torch.bfloat16)
+    model.init_random_(0.02, seed=0).eval()
+    svc = build_service(cfg, args.bank_tokens)
+    svc.setup_memory_client(model)
+    for layer in model.model.layers:
+        layer.self_attn.decode_reserve = args.steps + 8
+    torch.cuda.synchronize()
+    setup_s = time.perf_counter() - t0
+    g = torch.Generator(device=dev).manual_seed(3)
+    B, S = args.batch, args.context
+    ids = torch.randint(0, cfg.vocab_size, (B, S), generator=g, device=dev)
+    mask = torch.ones((B, S), dtype=torch.long, device=dev)
+    doc_ids = torch.zeros((B, S), dtype=torch.long, device=dev)
+    model.generate_greedy(ids[:, :64].contiguous(), mask[:, :64].contiguous(), doc_ids[:, :64].contiguous(), 4)   # warm-up
+    timings = {}
+    toks, cache = model.generate_greedy(ids, mask, doc_ids, args.steps, require_recall_topk=True, timings=timings)
+    last_router = svc.router_layer_ids[-1]
+    kv = cache.cache_kwargs[last_router]["kv_lengths"].cpu().tolist()
+    out = {"metric": "sparse decode tok/s (end to end, greedy)", "value": round(B * timings["decode_steps"] / timings["decode_s"], 1),
+           "unit": "tokens/s", "ms_per_decode_step": round(timings["decode_s"] / timings["decode_steps"] * 1e3, 3),
+           "prefill_s": round(timings["prefill_s"], 3), "setup_s": round(setup_s, 1), "dtype": "bf16", "data": "synthetic",
+           "config": {"workload": "configs[4]: Qwen3-4B shape, random init, routing on the upper half of the layers",
+                      "layers": args.layers, "bank_tokens": args.bank_tokens, "batch": B, "context_tokens": S,
+                      "decode_steps": args.steps, "top_k": cfg.msa_config.top_k_docs,
+                      "kv_rows_last_router_layer": kv[:4]},
+           "generated_shape": list(toks.shape)}
+    print(json.dumps(out), flush=True)
+    return out
+
+
+if __name__ == "__main__":
+    main()

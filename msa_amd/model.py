@@ -74,8 +74,19 @@ class MSAForCausalLM(nn.Module):
         return self
 
     @torch.no_grad()
+    def init_random_(self, std: float = 0.02, seed: int = 0):
+        """In-place normal init on whatever device the parameters live on (fast for 4B parameters on
+        the GPU); norm weights stay at one."""
+        g = torch.Generator(device=next(self.parameters()).device).manual_seed(seed)
+        for p in self.parameters():
+            if p.dim() > 1:
+                p.normal_(0.0, std, generator=g)
+        return self
+
+    @torch.no_grad()
     def generate_greedy(self, input_ids, attention_mask, doc_ids, max_new_tokens: int, top_k_docs: Optional[int] = None,
-                        require_recall_topk: bool = False, past_key_values: Optional[CustomDynamicCache] = None):
+                        require_recall_topk: bool = False, past_key_values: Optional[CustomDynamicCache] = None,
+                        timings: Optional[dict] = None):
         """Stage 2 on the (left-padded) query batch, then ``max_new_tokens`` greedy decode steps.
         Positions follow the reference: queries start at ``3 + top_k`` (src/msa_service.py:1823-1836),
         padding repeats the first position, each decode step advances by one
@@ -89,9 +100,17 @@ class MSAForCausalLM(nn.Module):
             cache.record_kwargs(i, {"stage": "prefill_stage2"})
         n_valid = attention_mask.sum(dim=1).tolist()
         pos = torch.tensor([query_position_ids(n, k, 3, S - n) for n in n_valid], dtype=torch.long, device=input_ids.device)
+        if timings is not None:
+            import time
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
         h = self.model(input_ids, attention_mask, pos, cache, doc_ids)
         tok = self.lm_head(h[:, -1:]).argmax(-1)
         out = [tok]
+        if timings is not None:
+            torch.cuda.synchronize()
+            timings["prefill_s"] = time.perf_counter() - t0
+            t0 = time.perf_counter()
         for i in range(cfg.num_hidden_layers):
             cache.cache_kwargs[i]["stage"] = "generate"
         next_pos = pos[:, -1:] + 1
@@ -102,6 +121,10 @@ class MSAForCausalLM(nn.Module):
             tok = self.lm_head(h).argmax(-1)
             out.append(tok)
             next_pos = next_pos + 1
+        if timings is not None:
+            torch.cuda.synchronize()
+            timings["decode_s"] = time.perf_counter() - t0
+            timings["decode_steps"] = max_new_tokens - 1
         return torch.cat(out, dim=1), cache
 
 

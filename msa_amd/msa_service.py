@@ -168,8 +168,11 @@ class Memory:
     def finish(self) -> None:
         """Merges the pooled ids, checks them against the documents' chunk counts and creates the
         native bank handle (replaces ``_generate_slice``: no slices, no transposed views)."""
+        self.block_desc.merge_poolig_doc_id(self.device)
+        self._finish_bank()
+
+    def _finish_bank(self) -> None:
         desc = self.block_desc
-        desc.merge_poolig_doc_id(self.device)
         counts = torch.bincount(desc.pool_ids_cpu, minlength=desc.nr_docs + 1)
         if not torch.equal(counts, desc.doc_lens_cpu):
             raise AssertionError("pooled document ids do not match the documents' chunk counts")
@@ -181,6 +184,24 @@ class Memory:
                              ref.shape[2], ref.dtype)
         for layer, slot in self._layer_slot.items():
             self.bank.set_layer(slot, self._rk[layer], self._k[layer], self._v[layer])
+
+    def load_pooled(self, docs: List[Document], rk: Dict[int, torch.Tensor], k: Dict[int, torch.Tensor],
+                    v: Dict[int, torch.Tensor], template_prefix: Dict[int, Tuple[torch.Tensor, torch.Tensor]]) -> None:
+        """Adopts an already pooled bank: per router layer ``rk`` on the device and ``k`` / ``v`` in
+        pinned host memory, all chunk-major ``[C, Hkv, D]`` in document order, plus the template
+        prefix K / V ``[1, Hkv, n, D]`` of every layer.  (Entry point for synthetic banks and for a
+        bank read back from storage; :meth:`add_block` is the path that follows stage 1.)"""
+        self.block_desc.init_docs(docs, self.device)
+        lens = self.block_desc.doc_lens_cpu
+        self.block_desc.pool_ids_cpu = torch.repeat_interleave(torch.arange(lens.numel()), lens)
+        self.block_desc.pool_ids = self.block_desc.pool_ids_cpu.to(self.device)
+        missing = [l for l in self.router_layer_ids if l not in rk or l not in k or l not in v]
+        if missing:
+            raise ValueError(f"router layers {missing} have no pooled tensors")
+        self._rk, self._k, self._v = dict(rk), dict(k), dict(v)
+        self._kv_offset = self.block_desc.chunks()
+        self.template_prefix_kvcache = {l: (a.to(self.device), b.to(self.device)) for l, (a, b) in template_prefix.items()}
+        self._finish_bank()
 
     def get_max_local_pool_doc_id(self) -> int:
         return int(self.block_desc.pool_ids_cpu[-1])

@@ -260,7 +260,7 @@ def sparse_attn(q, k, v, kv_off, kv_len, max_kv: int, cu_q=None, max_sq: int = 1
     if kv_off.dtype != torch.int64 or kv_len.dtype != torch.int32 or (cu_q is not None and cu_q.dtype != torch.int32):
         raise ValueError("kv_off int64, kv_len / cu_q int32")
     lib = _lib.load()
-    need = lib.msa_attn_workspace_bytes(total_q, Hq, D, max_kv)
+    need = lib.msa_attn_workspace_bytes(total_q, Hq, Hkv, D, max_kv)
     ws = _attn_ws.get(q.device)
     if ws is None or ws.numel() < need:
         ws = _attn_ws[q.device] = torch.empty(need, dtype=torch.uint8, device=q.device)

@@ -58,7 +58,9 @@ def test_validation_errors_without_gpu():
     rc = lib.msa_bank_create(C.byref(h), 1, 6, 8, 128, 0, C.addressof(off), C.addressof(gid), 2)
     assert rc == -1 and b"doc_chunk_off" in lib.msa_last_error()
     assert lib.msa_route_workspace_bytes(16, 128, 32, 8, 128, 1000, 50, 16) > 16 * 128 * 1024 * 2
-    assert lib.msa_attn_workspace_bytes(4, 32, 128, 1000) > 0
+    assert lib.msa_attn_workspace_bytes(4, 32, 8, 128, 1000) > 0
+    # many query rows: one pass over the keys, so the workspace stays linear in the rows
+    assert lib.msa_attn_workspace_bytes(65536, 32, 8, 128, 4400) < 2 * 65536 * 32 * 130 * 4
     with pytest.raises(TypeError):
         import torch
         _lib.dtype_code(torch.float16)

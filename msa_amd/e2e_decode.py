@@ -63,6 +63,9 @@ def main(argv=None):
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--layers", type=int, default=36)
+    ap.add_argument("--eager", action="store_true", help="do not capture the decode step as a HIP graph")
+    ap.add_argument("--verify-graph", type=int, default=0, metavar="N",
+                    help="also decode N steps eagerly and require identical tokens from the graph replays")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
         sys.exit("e2e_decode: no GPU visible; the HIP path has no CPU fallback")
@@ -88,7 +91,14 @@ def main(argv=None):
     doc_ids = torch.zeros((B, S), dtype=torch.long, device=dev)
     model.generate_greedy(ids[:, :64].contiguous(), mask[:, :64].contiguous(), doc_ids[:, :64].contiguous(), 4)   # warm-up
     timings = {}
-    toks, cache = model.generate_greedy(ids, mask, doc_ids, args.steps, require_recall_topk=True, timings=timings)
+    toks, cache = model.generate_greedy(ids, mask, doc_ids, args.steps, require_recall_topk=True, timings=timings,
+                                        use_graph=not args.eager)
+    verified = None
+    if args.verify_graph:
+        ref, _ = model.generate_greedy(ids, mask, doc_ids, args.verify_graph, use_graph=False)
+        verified = bool(torch.equal(ref, toks[:, :args.verify_graph]))
+        if not verified:
+            sys.exit("e2e_decode: graph replays and eager decoding produced different tokens")
     last_router = svc.router_layer_ids[-1]
     kv = cache.cache_kwargs[last_router]["kv_lengths"].cpu().tolist()
     out = {"metric": "sparse decode tok/s (end to end, greedy)", "value": round(B * timings["decode_steps"] / timings["decode_s"], 1),
@@ -98,6 +108,7 @@ def main(argv=None):
                       "layers": args.layers, "bank_tokens": args.bank_tokens, "batch": B, "context_tokens": S,
                       "decode_steps": args.steps, "top_k": cfg.msa_config.top_k_docs,
                       "kv_rows_last_router_layer": kv[:4]},
+           "decode_mode": "eager" if args.eager else "hip graph replay", "graph_equals_eager": verified,
            "generated_shape": list(toks.shape)}
     print(json.dumps(out), flush=True)
     return out

@@ -219,9 +219,8 @@ class MemorySparseAttention(nn.Module):
             raise ValueError("the decode step takes one new token per sample")
         kc, vc, kv_len = ck["compacked_key_cache"], ck["compacked_value_cache"], ck["kv_lengths"]
         Hkv, D = self.num_kv_heads, self.head_dim
-        ck["decoded"] = ck.get("decoded", 0) + 1
-        if ck["decoded"] > self.decode_reserve:
-            raise RuntimeError("compact cache is full: raise decode_reserve before stage 2")
+        # capacity is the caller's job (rows behind the context: decode_reserve); a full cache drops the
+        # new row inside the kernel instead of writing out of bounds
         ops.cache_append(k[:, 0].contiguous(), v[:, 0].contiguous(), kc, vc, kv_len)
         out = ops.sparse_attn(q[:, 0].contiguous(), kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), ck["kv_offsets"], kv_len,
                               ck["kv_capacity"], scale=self.scaling, causal=True)

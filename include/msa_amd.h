@@ -164,6 +164,24 @@ int msa_sparse_attn(const void* q, const int32_t* cu_q, const void* k, const voi
                     int32_t dtype, float scale, int32_t causal, void* out, void* workspace,
                     size_t workspace_bytes, void* stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * Fused helpers around the attention call.  msa_qk_norm_rope replaces q_norm / k_norm + apply_rotary_pos_emb
+ * (src/msa/memory_sparse_attention.py:129-133; transformers Qwen3RMSNorm, rotate_half): per head RMSNorm over the
+ * 128 dims in fp32 times the norm weight, then half-split rotary at positions[n] from fp32 tables
+ * [rope_rows, D/2] (positions are clamped to the table).  q / k / v are rows of a (possibly fused) projection
+ * output with the given row strides in elements; outputs are dense [N, H, D].  v may be NULL (no copy).
+ * msa_rmsnorm: out = rmsnorm(x) * weight over rows of H elements; with `residual` it first does
+ * residual += x in place and normalises the sum (the residual add + norm of a decoder layer).
+ * msa_silu_mul: out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i] for a fused gate/up projection. */
+int msa_qk_norm_rope(const void* q, const void* k, const void* v, int64_t q_row_stride,
+                     int64_t k_row_stride, int64_t v_row_stride, const int64_t* positions,
+                     const void* q_norm_w, const void* k_norm_w, float eps, const float* rope_cos,
+                     const float* rope_sin, int32_t rope_rows, int32_t dtype, int64_t N, int32_t Hq,
+                     int32_t Hkv, int32_t D, void* q_out, void* k_out, void* v_out, void* stream);
+int msa_rmsnorm(const void* x, void* residual, const void* weight, int32_t dtype, int64_t N,
+                int32_t H, float eps, void* out, void* stream);
+int msa_silu_mul(const void* gate_up, int32_t dtype, int64_t N, int32_t I, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,201 @@
+// Small fused kernels around the attention call of a decoder layer: per-head q/k RMSNorm + rotary
+// in one pass, row RMSNorm with the residual add folded in, and SiLU(gate) * up.  All are a few
+// bytes per FLOP: one read of the input, one write of the output.
+#include <algorithm>
+
+#include "common.h"
+
+namespace {
+
+__device__ __forceinline__ float row16_sum(float v) {   // all-reduce over the 16 lanes of a DPP row
+  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));
+  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));
+  return v;
+}
+__device__ __forceinline__ float row16_ror8(float v) {  // value of the lane 8 places away in the row
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
+}
+
+template <typename T>
+__device__ __forceinline__ void load8g(const T* p, float (&x)[8]) {
+  if constexpr (sizeof(T) == 2) {
+    const uint4 w = *reinterpret_cast<const uint4*>(p);
+    x[0] = bf16lo(w.x); x[1] = bf16hi(w.x); x[2] = bf16lo(w.y); x[3] = bf16hi(w.y);
+    x[4] = bf16lo(w.z); x[5] = bf16hi(w.z); x[6] = bf16lo(w.w); x[7] = bf16hi(w.w);
+  } else {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    const float4 b = *reinterpret_cast<const float4*>(p + 4);
+    x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
+  }
+}
+template <typename T>
+__device__ __forceinline__ void store8g(T* p, const float (&x)[8]) {
+  if constexpr (sizeof(T) == 2) {
+    uint4 w;
+    w.x = pack_bf16x2(x[0], x[1]); w.y = pack_bf16x2(x[2], x[3]);
+    w.z = pack_bf16x2(x[4], x[5]); w.w = pack_bf16x2(x[6], x[7]);
+    *reinterpret_cast<uint4*>(p) = w;
+  } else {
+    *reinterpret_cast<float4*>(p) = make_float4(x[0], x[1], x[2], x[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(x[4], x[5], x[6], x[7]);
+  }
+}
+
+// One workgroup per token; 16 lanes per head (8 dims each): heads 0..Hq-1 are q, the rest k.
+// RMSNorm over the head's 128 dims (fp32), times the norm weight, then half-split rotary at the
+// token's position: lane j pairs with lane j^8 of its row (dims d and d +- 64).
+template <typename T>
+__global__ void qk_norm_rope_kernel(const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v,
+                                    int64_t q_stride, int64_t k_stride, int64_t v_stride,
+                                    const int64_t* __restrict__ pos, const T* __restrict__ qw,
+                                    const T* __restrict__ kw, float eps, const float* __restrict__ cos_t,
+                                    const float* __restrict__ sin_t, int32_t rope_rows, int32_t Hq, int32_t Hkv,
+                                    T* __restrict__ q_out, T* __restrict__ k_out, T* __restrict__ v_out) {
+  const int64_t n = blockIdx.x;
+  const int head = threadIdx.x >> 4, j = threadIdx.x & 15;
+  if (head >= Hq + Hkv) {                       // optional V heads: a straight copy into a dense row
+    const int hv = head - Hq - Hkv;
+    if (v != nullptr && hv < Hkv) {
+      float t[8];
+      load8g<T>(v + n * v_stride + hv * kHeadDim + 8 * j, t);
+      store8g<T>(v_out + (n * Hkv + hv) * kHeadDim + 8 * j, t);
+    }
+    return;
+  }
+  const bool is_q = head < Hq;
+  const int h = is_q ? head : head - Hq;
+  const T* src = is_q ? q + n * q_stride + h * kHeadDim : k + n * k_stride + h * kHeadDim;
+  T* dst = is_q ? q_out + (n * Hq + h) * kHeadDim : k_out + (n * Hkv + h) * kHeadDim;
+  float x[8], w[8];
+  load8g<T>(src + 8 * j, x);
+  load8g<T>((is_q ? qw : kw) + 8 * j, w);
+  float ssq = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ssq += x[i] * x[i];
+  const float inv = rsqrtf(row16_sum(ssq) * (1.0f / kHeadDim) + eps);
+  const int64_t p = min((int64_t)max((int64_t)0, pos[n]), (int64_t)rope_rows - 1);
+  const int f = 8 * (j & 7);                    // frequency index of this lane's first element
+  float out[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float y = x[i] * inv * w[i];
+    const float other = row16_ror8(y);          // the paired dim (d + 64 for j < 8, d - 64 for j >= 8)
+    const float c = cos_t[p * 64 + f + i], s = sin_t[p * 64 + f + i];
+    out[i] = j < 8 ? y * c - other * s : y * c + other * s;
+  }
+  store8g<T>(dst + 8 * j, out);
+}
+
+// One workgroup per row.  With `residual`: residual <- residual + x (stored in T), then normalised.
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, T* __restrict__ residual,
+                                                      const T* __restrict__ w, int32_t H, float eps,
+                                                      T* __restrict__ out) {
+  __shared__ float part[4];
+  const int64_t row = blockIdx.x;
+  const T* xr = x + row * H;
+  T* rr = residual ? residual + row * H : nullptr;
+  float ssq = 0.f;
+  for (int i = threadIdx.x; i < H; i += 256) {
+    float v;
+    if constexpr (sizeof(T) == 2) v = bf16_to_f32(xr[i]); else v = xr[i];
+    if (rr) {
+      float r;
+      if constexpr (sizeof(T) == 2) { r = bf16_to_f32(rr[i]); v = bf16_to_f32(f32_to_bf16(v + r)); rr[i] = f32_to_bf16(v); }
+      else { r = rr[i]; v = v + r; rr[i] = v; }
+    }
+    ssq += v * v;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) ssq += __shfl_xor(ssq, o);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ssq;
+  __syncthreads();
+  const float inv = rsqrtf((part[0] + part[1] + part[2] + part[3]) / (float)H + eps);
+  const T* src = rr ? rr : xr;      // rr was written by this same thread for the same indices
+  for (int i = threadIdx.x; i < H; i += 256) {
+    float v, g;
+    if constexpr (sizeof(T) == 2) { v = bf16_to_f32(src[i]); g = bf16_to_f32(w[i]); out[row * H + i] = f32_to_bf16(v * inv * g); }
+    else { v = src[i]; g = w[i]; out[row * H + i] = v * inv * g; }
+  }
+}
+
+// out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gate_up, int64_t N, int32_t I, T* __restrict__ out) {
+  const int64_t total = N * I;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+    const int64_t n = idx / I, i = idx % I;
+    float g, u;
+    if constexpr (sizeof(T) == 2) { g = bf16_to_f32(gate_up[n * 2 * I + i]); u = bf16_to_f32(gate_up[n * 2 * I + I + i]); }
+    else { g = gate_up[n * 2 * I + i]; u = gate_up[n * 2 * I + I + i]; }
+    const float y = g / (1.0f + __expf(-g)) * u;
+    if constexpr (sizeof(T) == 2) out[idx] = f32_to_bf16(y); else out[idx] = y;
+  }
+}
+
+}  // namespace
+
+extern "C" int msa_qk_norm_rope(const void* q, const void* k, const void* v, int64_t q_row_stride,
+                                int64_t k_row_stride, int64_t v_row_stride, const int64_t* positions, const void* q_norm_w, const void* k_norm_w, float eps,
+                                const float* rope_cos, const float* rope_sin, int32_t rope_rows, int32_t dtype,
+                                int64_t N, int32_t Hq, int32_t Hkv, int32_t D, void* q_out, void* k_out,
+                                void* v_out, void* stream) {
+  MSA_REQUIRE(q && k && positions && q_norm_w && k_norm_w && rope_cos && rope_sin && q_out && k_out,
+              "msa_qk_norm_rope: null pointer");
+  MSA_REQUIRE(D == kHeadDim, "msa_qk_norm_rope: head dim %d unsupported (need %d)", D, kHeadDim);
+  MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "msa_qk_norm_rope: bad dtype %d", dtype);
+  MSA_REQUIRE(N > 0 && N < (int64_t)1 << 31, "msa_qk_norm_rope: N=%lld out of range", (long long)N);
+  MSA_REQUIRE((v == nullptr) == (v_out == nullptr), "msa_qk_norm_rope: v and v_out go together");
+  const int heads = Hq + Hkv + (v ? Hkv : 0);
+  MSA_REQUIRE(Hq > 0 && Hkv > 0 && heads * 16 <= 1024, "msa_qk_norm_rope: Hq=%d Hkv=%d unsupported", Hq, Hkv);
+  MSA_REQUIRE(v == nullptr || (v_row_stride >= (int64_t)Hkv * D && v_row_stride % 8 == 0),
+              "msa_qk_norm_rope: bad V row stride");
+  MSA_REQUIRE(rope_rows > 0, "msa_qk_norm_rope: empty rotary table");
+  MSA_REQUIRE(q_row_stride >= (int64_t)Hq * D && k_row_stride >= (int64_t)Hkv * D && q_row_stride % 8 == 0 &&
+                  k_row_stride % 8 == 0, "msa_qk_norm_rope: bad row strides");
+  const int threads = (heads * 16 + 63) / 64 * 64;
+  if (dtype == MSA_BF16)
+    qk_norm_rope_kernel<bf16_t><<<(unsigned)N, threads, 0, as_stream(stream)>>>(
+        (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, q_row_stride, k_row_stride, v_row_stride, positions,
+        (const bf16_t*)q_norm_w, (const bf16_t*)k_norm_w, eps, rope_cos, rope_sin, rope_rows, Hq, Hkv,
+        (bf16_t*)q_out, (bf16_t*)k_out, (bf16_t*)v_out);
+  else
+    qk_norm_rope_kernel<float><<<(unsigned)N, threads, 0, as_stream(stream)>>>(
+        (const float*)q, (const float*)k, (const float*)v, q_row_stride, k_row_stride, v_row_stride, positions,
+        (const float*)q_norm_w, (const float*)k_norm_w, eps, rope_cos, rope_sin, rope_rows, Hq, Hkv, (float*)q_out,
+        (float*)k_out, (float*)v_out);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
+
+extern "C" int msa_rmsnorm(const void* x, void* residual, const void* weight, int32_t dtype, int64_t N, int32_t H,
+                           float eps, void* out, void* stream) {
+  MSA_REQUIRE(x && weight && out, "msa_rmsnorm: null pointer");
+  MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "msa_rmsnorm: bad dtype %d", dtype);
+  MSA_REQUIRE(N > 0 && N < (int64_t)1 << 31 && H > 0, "msa_rmsnorm: bad shape");
+  if (dtype == MSA_BF16)
+    rmsnorm_kernel<bf16_t><<<(unsigned)N, 256, 0, as_stream(stream)>>>((const bf16_t*)x, (bf16_t*)residual,
+                                                                       (const bf16_t*)weight, H, eps, (bf16_t*)out);
+  else
+    rmsnorm_kernel<float><<<(unsigned)N, 256, 0, as_stream(stream)>>>((const float*)x, (float*)residual,
+                                                                      (const float*)weight, H, eps, (float*)out);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
+
+extern "C" int msa_silu_mul(const void* gate_up, int32_t dtype, int64_t N, int32_t I, void* out, void* stream) {
+  MSA_REQUIRE(gate_up && out, "msa_silu_mul: null pointer");
+  MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "msa_silu_mul: bad dtype %d", dtype);
+  MSA_REQUIRE(N > 0 && I > 0, "msa_silu_mul: bad shape");
+  const int64_t total = N * I;
+  const int grid = (int)std::min<int64_t>((total + 255) / 256, 16384);
+  if (dtype == MSA_BF16)
+    silu_mul_kernel<bf16_t><<<grid, 256, 0, as_stream(stream)>>>((const bf16_t*)gate_up, N, I, (bf16_t*)out);
+  else
+    silu_mul_kernel<float><<<grid, 256, 0, as_stream(stream)>>>((const float*)gate_up, N, I, (float*)out);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}

@@ -53,6 +53,9 @@ def rotary_embedding(position_ids: torch.Tensor, head_dim: int, theta: float, dt
     return emb.cos().to(dtype), emb.sin().to(dtype)
 
 
+_ROPE_TABLES = {}
+
+
 class MemorySparseAttention(nn.Module):
     def __init__(self, config: MSAConfig, layer_idx: int):
         super().__init__()
@@ -87,6 +90,7 @@ class MemorySparseAttention(nn.Module):
         self.template_prefix_vcache = None
         self.memory_client = None
         self.decode_reserve = 512      # rows kept free behind the stage-2 context for in-place decode appends
+        self._qkv_weight = None        # q / k / v weights concatenated on first use of the fused projection
 
     def set_memory_client(self, memory_client):
         self.memory_client = memory_client
@@ -110,10 +114,31 @@ class MemorySparseAttention(nn.Module):
         cos, sin = position_embeddings
         return apply_rotary_bshd(q, cos, sin).contiguous(), apply_rotary_bshd(k, cos, sin).contiguous(), v.contiguous()
 
+    def _project_fused(self, hidden_states, position_ids):
+        """Same result as :meth:`_project` from integer positions: one GEMM over the concatenated q / k / v
+        weights, then per-head RMSNorm + rotary (+ the dense copy of V) in one HIP kernel."""
+        B, S, _ = hidden_states.shape
+        Hq, Hkv, D = self.config.num_attention_heads, self.num_kv_heads, self.head_dim
+        if self._qkv_weight is None or self._qkv_weight.device != hidden_states.device:
+            self._qkv_weight = torch.cat([self.q_proj.weight, self.k_proj.weight, self.v_proj.weight], dim=0).contiguous()
+        dev = hidden_states.device
+        rows = min(self.config.max_position_embeddings, 32768)
+        key = (dev, rows, float(self.config.rope_theta))
+        if key not in _ROPE_TABLES:
+            _ROPE_TABLES[key] = ops.rope_tables(rows, D, self.config.rope_theta, device=dev)
+        qkv = F.linear(hidden_states.reshape(B * S, -1), self._qkv_weight)
+        q, k, v = ops.qk_norm_rope(qkv, Hq, Hkv, D, position_ids.reshape(-1).contiguous(), self.q_norm.weight,
+                                   self.k_norm.weight, self.q_norm.variance_epsilon, _ROPE_TABLES[key])
+        return q.view(B, S, Hq, D), k.view(B, S, Hkv, D), v.view(B, S, Hkv, D)
+
     def forward_with_kvcache_for_batch_parrallel(self, hidden_states, doc_ids, attention_mask=None,
-                                                 position_embeddings=None, past_key_value=None, **kwargs):
+                                                 position_embeddings=None, past_key_value=None, position_ids=None,
+                                                 **kwargs):
         stage = past_key_value.cache_kwargs[self.layer_idx]["stage"]
-        q, k, v = self._project(hidden_states, position_embeddings)          # [B, S, H, D] token-major
+        if position_ids is not None and hidden_states.is_cuda and self.q_proj.bias is None:
+            q, k, v = self._project_fused(hidden_states, position_ids)       # [B, S, H, D] token-major
+        else:
+            q, k, v = self._project(hidden_states, position_embeddings)
         if stage == "prefill_stage1":
             return self._stage1(hidden_states, doc_ids, attention_mask, q, k, v, past_key_value)
         if stage == "prefill_stage2":

@@ -10,6 +10,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
+from . import ops
 from .cache import CustomDynamicCache, create_cache
 from .config import MSAConfig
 from .memory_sparse_attention import MemorySparseAttention, RMSNorm, rotary_embedding
@@ -23,7 +24,13 @@ class MLP(nn.Module):
         self.up_proj = nn.Linear(config.hidden_size, config.intermediate_size, bias=False)
         self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=False)
 
+        self._gate_up_weight = None
+
     def forward(self, x):
+        if x.is_cuda and x.dtype in (torch.bfloat16, torch.float32):
+            if self._gate_up_weight is None or self._gate_up_weight.device != x.device:
+                self._gate_up_weight = torch.cat([self.gate_proj.weight, self.up_proj.weight], dim=0).contiguous()
+            return self.down_proj(ops.silu_mul(F.linear(x, self._gate_up_weight)))
         return self.down_proj(F.silu(self.gate_proj(x)) * self.up_proj(x))
 
 
@@ -35,7 +42,14 @@ class MSADecoderLayer(nn.Module):
         self.input_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
         self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
 
-    def forward(self, hidden_states, doc_ids, attention_mask, position_embeddings, past_key_value):
+    def forward(self, hidden_states, doc_ids, attention_mask, position_embeddings, past_key_value, position_ids=None):
+        if hidden_states.is_cuda and hidden_states.dtype in (torch.bfloat16, torch.float32):
+            # HIP glue: norm kernels with the residual add folded in; hidden_states is updated in place
+            n1, n2 = self.input_layernorm, self.post_attention_layernorm
+            h, _ = self.self_attn(ops.rmsnorm(hidden_states, n1.weight, n1.variance_epsilon), doc_ids, attention_mask,
+                                  position_embeddings, past_key_value, position_ids=position_ids)
+            x = ops.rmsnorm(h.contiguous(), n2.weight, n2.variance_epsilon, residual=hidden_states)
+            return hidden_states.add_(self.mlp(x))
         h, _ = self.self_attn(self.input_layernorm(hidden_states), doc_ids, attention_mask, position_embeddings,
                               past_key_value)
         hidden_states = hidden_states + h
@@ -52,6 +66,10 @@ class MSAModel(nn.Module):
 
     def forward(self, input_ids, attention_mask, position_ids, past_key_values, doc_ids):
         h = self.embed_tokens(input_ids)
+        if h.is_cuda:
+            for layer in self.layers:
+                h = layer(h, doc_ids, attention_mask, None, past_key_values, position_ids=position_ids)
+            return ops.rmsnorm(h, self.norm.weight, self.norm.variance_epsilon)
         pe = rotary_embedding(position_ids, self.config.head_dim, self.config.rope_theta, h.dtype)
         for layer in self.layers:
             h = layer(h, doc_ids, attention_mask, pe, past_key_values)

@@ -269,3 +269,45 @@ def sparse_attn(q, k, v, kv_off, kv_len, max_kv: int, cu_q=None, max_sq: int = 1
                               Hq, Hkv, D, dtype_code(q.dtype), D ** -0.5 if scale is None else scale, int(causal),
                               ptr(out), ptr(ws), ws.numel(), _stream()), "msa_sparse_attn")
     return out
+
+
+# ------------------------------------------------------------------------------ fused layer helpers
+def qk_norm_rope(qkv: torch.Tensor, Hq: int, Hkv: int, D: int, positions: torch.Tensor, q_norm_w, k_norm_w, eps: float,
+                 rope: Tuple[torch.Tensor, torch.Tensor]):
+    """``qkv [N, (Hq + 2 Hkv) * D]`` (fused projection output) -> ``q [N, Hq, D]`` and ``k [N, Hkv, D]``
+    normalised per head and rotated at ``positions [N]``, plus ``v [N, Hkv, D]`` copied dense."""
+    _need_cuda(qkv, positions, q_norm_w, k_norm_w, rope[0], rope[1])
+    N, W = qkv.shape
+    if W != (Hq + 2 * Hkv) * D or positions.dtype != torch.int64 or positions.numel() != N:
+        raise ValueError("qkv must be [N, (Hq + 2 Hkv) D] and positions int64 [N]")
+    q = torch.empty((N, Hq, D), dtype=qkv.dtype, device=qkv.device)
+    k = torch.empty((N, Hkv, D), dtype=qkv.dtype, device=qkv.device)
+    v = torch.empty((N, Hkv, D), dtype=qkv.dtype, device=qkv.device)
+    es = qkv.element_size()
+    base = qkv.data_ptr()
+    check(_lib.load().msa_qk_norm_rope(base, base + Hq * D * es, base + (Hq + Hkv) * D * es, W, W, W, ptr(positions),
+                                       ptr(q_norm_w), ptr(k_norm_w), eps, ptr(rope[0]), ptr(rope[1]), rope[0].shape[0],
+                                       dtype_code(qkv.dtype), N, Hq, Hkv, D, ptr(q), ptr(k), ptr(v), _stream()),
+          "msa_qk_norm_rope")
+    return q, k, v
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Row RMSNorm of ``x [..., H]``; with ``residual`` (same shape) does ``residual += x`` in place first
+    and normalises the sum."""
+    _need_cuda(x, weight, residual)
+    H = x.shape[-1]
+    out = torch.empty_like(x)
+    check(_lib.load().msa_rmsnorm(ptr(x), ptr(residual), ptr(weight), dtype_code(x.dtype), x.numel() // H, H, eps,
+                                  ptr(out), _stream()), "msa_rmsnorm")
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    """``silu(gate) * up`` for a fused ``[..., 2 I]`` projection output (gate first)."""
+    _need_cuda(gate_up)
+    I = gate_up.shape[-1] // 2
+    out = torch.empty(gate_up.shape[:-1] + (I,), dtype=gate_up.dtype, device=gate_up.device)
+    check(_lib.load().msa_silu_mul(ptr(gate_up), dtype_code(gate_up.dtype), gate_up.numel() // (2 * I), I, ptr(out),
+                                   _stream()), "msa_silu_mul")
+    return out

@@ -390,3 +390,48 @@ def test_config1_routing_layer_fp32(ops):
     torch.cuda.synchronize()
     want = cf.attention(qd, torch.cat([wk, loc_k]), torch.cat([wv, loc_v]))
     assert cf.rel_err(out.cpu(), want) < 1e-5
+
+
+# ------------------------------------------------------------------ fused layer helpers
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_qk_norm_rope_rmsnorm_silu(ops, dtype):
+    say(f"qk_norm_rope / rmsnorm / silu_mul dtype={dtype}")
+    N, Hq, Hkv, D, theta, eps = 37, 32, 8, 128, 1e6, 1e-6
+    qkv = _randn((N, (Hq + 2 * Hkv) * D), 100, dtype)
+    qw, kw = (1 + 0.1 * _randn((D,), 101, torch.float32)).to(dtype), (1 + 0.1 * _randn((D,), 102, torch.float32)).to(dtype)
+    pos = torch.tensor([0, 1, 5, 19, 4387, 2047] + list(range(100, 131)), dtype=torch.int64)
+    rope = ops.rope_tables(8192, D, theta)
+    q, k, v = ops.qk_norm_rope(qkv.cuda(), Hq, Hkv, D, pos.cuda(), qw.cuda(), kw.cuda(), eps, rope)
+    x = qkv.double().view(N, Hq + 2 * Hkv, D)
+
+    def norm(t, w):
+        return t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps) * w.double()
+    nq, nk = norm(x[:, :Hq], qw), norm(x[:, Hq:Hq + Hkv], kw)
+    # (a) small positions against the fp64 rotary (pins pairing and signs; fp32 angle error is negligible there)
+    small = pos < 64
+    assert cf.rel_err(q.cpu()[small], cf.apply_rope(nq[small], pos[small], theta)) < TOL[dtype]
+    assert cf.rel_err(k.cpu()[small], cf.apply_rope(nk[small], pos[small], theta)) < TOL[dtype]
+    # (b) every position against a rotation by the SAME fp32 table entries the kernel reads: the tables carry the
+    # fp32 angle rounding of Qwen3's rotary embedding (about 4387 * 2^-24 rad at the largest position here)
+    c, s_ = rope[0].cpu().double()[pos][:, None, :], rope[1].cpu().double()[pos][:, None, :]
+
+    def rot(t):
+        a, b = t[..., :64], t[..., 64:]
+        return torch.cat([a * c - b * s_, b * c + a * s_], dim=-1)
+    assert cf.rel_err(q.cpu(), rot(nq)) < TOL[dtype] and cf.rel_err(k.cpu(), rot(nk)) < TOL[dtype]
+    assert torch.equal(v.cpu(), qkv.view(N, Hq + 2 * Hkv, D)[:, Hq + Hkv:])
+
+    H = 2560
+    xs, res, w = _randn((N, H), 103, dtype), _randn((N, H), 104, dtype), (1 + 0.1 * _randn((H,), 105, torch.float32)).to(dtype)
+    out = ops.rmsnorm(xs.cuda(), w.cuda(), eps)
+    assert cf.rel_err(out.cpu(), norm(xs.double(), w)) < TOL[dtype]
+    res_dev = res.cuda()
+    out2 = ops.rmsnorm(xs.cuda(), w.cuda(), eps, residual=res_dev)
+    summed = (xs.double() + res.double()).to(dtype)                       # the sum is stored in the model dtype
+    assert torch.equal(res_dev.cpu(), summed)
+    assert cf.rel_err(out2.cpu(), norm(summed.double(), w)) < TOL[dtype]
+
+    gu = _randn((N, 2 * 1024), 106, dtype)
+    got = ops.silu_mul(gu.cuda())
+    g64, u64 = gu.double()[:, :1024], gu.double()[:, 1024:]
+    assert cf.rel_err(got.cpu(), g64 * torch.sigmoid(g64) * u64) < TOL[dtype]

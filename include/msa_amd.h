@@ -164,6 +164,14 @@ int msa_sparse_attn(const void* q, const int32_t* cu_q, const void* k, const voi
                     int32_t dtype, float scale, int32_t causal, void* out, void* workspace,
                     size_t workspace_bytes, void* stream);
 
+/* Same contract as msa_sparse_attn for bf16, built for blocks of query rows (stage-1 document-wise attention,
+ * src/msa/memory_sparse_attention.py:216-241, and the stage-2 query prefill, :334-339): an MFMA flash kernel, one
+ * pass over the keys, no workspace.  Use msa_sparse_attn for decode (one row per sample) and for fp32. */
+int msa_flash_attn(const void* q, const int32_t* cu_q, const void* k, const void* v,
+                   const int64_t* kv_off, const int32_t* kv_len, int32_t B, int32_t total_q,
+                   int32_t Hq, int32_t Hkv, int32_t D, float scale, int32_t causal, void* out,
+                   void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Fused helpers around the attention call.  msa_qk_norm_rope replaces q_norm / k_norm + apply_rotary_pos_emb
  * (src/msa/memory_sparse_attention.py:129-133; transformers Qwen3RMSNorm, rotate_half): per head RMSNorm over the

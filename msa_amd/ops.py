@@ -248,6 +248,7 @@ def cache_append(k_new, v_new, kcache, vcache, kv_len):
 
 
 _attn_ws = {}
+FLASH_MIN_ROWS = 16     # bf16 query blocks at least this long go to the MFMA flash kernel
 
 
 def sparse_attn(q, k, v, kv_off, kv_len, max_kv: int, cu_q=None, max_sq: int = 1, scale: Optional[float] = None,
@@ -260,6 +261,12 @@ def sparse_attn(q, k, v, kv_off, kv_len, max_kv: int, cu_q=None, max_sq: int = 1
     if kv_off.dtype != torch.int64 or kv_len.dtype != torch.int32 or (cu_q is not None and cu_q.dtype != torch.int32):
         raise ValueError("kv_off int64, kv_len / cu_q int32")
     lib = _lib.load()
+    sc = D ** -0.5 if scale is None else scale
+    if q.dtype == torch.bfloat16 and max_sq >= FLASH_MIN_ROWS:
+        out = torch.empty_like(q)
+        check(lib.msa_flash_attn(ptr(q), ptr(cu_q), ptr(k), ptr(v), ptr(kv_off), ptr(kv_len), B, total_q, Hq, Hkv, D, sc,
+                                 int(causal), ptr(out), _stream()), "msa_flash_attn")
+        return out
     need = lib.msa_attn_workspace_bytes(total_q, Hq, Hkv, D, max_kv)
     ws = _attn_ws.get(q.device)
     if ws is None or ws.numel() < need:

@@ -435,3 +435,34 @@ def test_qk_norm_rope_rmsnorm_silu(ops, dtype):
     got = ops.silu_mul(gu.cuda())
     g64, u64 = gu.double()[:, :1024], gu.double()[:, 1024:]
     assert cf.rel_err(got.cpu(), g64 * torch.sigmoid(g64) * u64) < TOL[dtype]
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 8), (16, 2)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_flash_attention_blocks(ops, Hq, Hkv, causal):
+    say(f"flash attention Hq={Hkv} Hkv={Hkv} causal={causal}")
+    D = 128
+    sq = [130, 1, 33, 64, 17]                 # ragged query blocks, including a single row and non-multiples of the tile
+    L = [400, 70, 33, 1000, 90]               # keys per sample (>= sq for the causal alignment)
+    B = len(sq)
+    cu_q = np.concatenate([[0], np.cumsum(sq)])
+    cu_kv = np.concatenate([[0], np.cumsum(L)])
+    q = _randn((int(cu_q[-1]), Hq, D), 200, torch.bfloat16)
+    k = _randn((int(cu_kv[-1]), Hkv, D), 201, torch.bfloat16)
+    v = _randn((int(cu_kv[-1]), Hkv, D), 202, torch.bfloat16)
+    kv_off = torch.as_tensor(cu_kv[:-1], dtype=torch.int64).cuda()
+    kv_len = torch.as_tensor(L, dtype=torch.int32).cuda()
+    out = ops.sparse_attn(q.cuda(), k.cuda(), v.cuda(), kv_off, kv_len, max(L),
+                          cu_q=torch.as_tensor(cu_q, dtype=torch.int32).cuda(), max_sq=max(sq), causal=causal)
+    torch.cuda.synchronize()
+    want = cf.attention_ragged(q, cu_q, k, v, cu_kv, causal=causal)
+    assert cf.rel_err(out.cpu(), want) < 1e-2
+    # the split-KV kernel (forced by a high threshold) must agree with the flash kernel
+    old = ops.FLASH_MIN_ROWS
+    try:
+        ops.FLASH_MIN_ROWS = 1 << 30
+        out2 = ops.sparse_attn(q.cuda(), k.cuda(), v.cuda(), kv_off, kv_len, max(L),
+                               cu_q=torch.as_tensor(cu_q, dtype=torch.int32).cuda(), max_sq=max(sq), causal=causal)
+    finally:
+        ops.FLASH_MIN_ROWS = old
+    assert cf.rel_err(out2.cpu(), want) < 1e-2

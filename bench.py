@@ -177,6 +177,27 @@ def extra_decode(dev):
             "attention_only_tok_per_s_36_layers": round(B / (36 * ms) * 1e3)}
 
 
+def extra_prefill_attention(dev):
+    """Stage-2 prefill attention of the end-to-end shape: B=16 queries of 4096 tokens over
+    [3 + 288 memory rows | the 4096 query tokens], causal, GQA 32/8, bf16 (MFMA flash kernel)."""
+    from msa_amd import ops
+    B, S, M = 16, 4096, 3 + 288
+    L = M + S
+    g = torch.Generator(device=dev).manual_seed(13)
+    q = torch.randn((B * S, HQ, D), generator=g, device=dev).to(torch.bfloat16)
+    kc = torch.randn((B * L, HKV, D), generator=g, device=dev).to(torch.bfloat16)
+    vc = torch.randn((B * L, HKV, D), generator=g, device=dev).to(torch.bfloat16)
+    kv_off = torch.arange(B, dtype=torch.int64, device=dev) * L
+    kv_len = torch.full((B,), L, dtype=torch.int32, device=dev)
+    cu_q = (torch.arange(B + 1, dtype=torch.int32, device=dev) * S)
+    ms = time_cuda(lambda: ops.sparse_attn(q, kc, vc, kv_off, kv_len, L, cu_q=cu_q, max_sq=S, causal=True), 5)
+    pairs = B * (S * M + S * (S + 1) // 2)
+    fl = 4.0 * pairs * HQ * D
+    return {"workload": "stage-2 prefill attention: B=16 x 4096 query tokens over 4387 keys, causal, GQA 32/8, bf16",
+            "ms_per_layer": round(ms, 3), "TFLOP/s": round(fl / ms / 1e9, 1),
+            "frac_mfma_peak": round(fl / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -363,7 +384,8 @@ def main():
 
     extras = None
     if not args.no_extras:
-        extras = {"pooling": extra_pooling(dev), "decode_attention": extra_decode(dev)}
+        extras = {"pooling": extra_pooling(dev), "decode_attention": extra_decode(dev),
+                  "prefill_attention": extra_prefill_attention(dev)}
 
     cpu = None
     if not args.no_cpu_baseline:

@@ -8,9 +8,10 @@
 // keeps the online softmax per column in registers (a column lives in one lane pair), and
 //   O^T[128 dims x 32 cols] += V^T . P^T      (contraction over keys).
 // S^T's accumulator layout IS the B-operand layout of the second product (same lane, same
-// column), up to the order of keys inside a group of 16, which the V^T operand simply mirrors, so
-// P never leaves registers; V^T operands are gathered from the row-major V tile with 16-bit LDS
-// reads.
+// column), up to the order of keys inside a group of 16, which the V^T operand mirrors, so P never
+// leaves registers.  V is transposed on its way into LDS (16-bit stores into [dim][key] rows with
+// that key order, XOR-swizzled so the stores of a wavefront spread over all banks) and read back
+// as 16-byte operands.
 #include <algorithm>
 
 #include "common.h"
@@ -22,17 +23,25 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
 
 constexpr int kKeysPerTile = 64;
 constexpr int kTileStride = 2 * kHeadDim + 16;   // bytes per key row in LDS: 256 + 16 pad (conflict-free b128 reads)
+constexpr int kVtStride = 2 * kKeysPerTile + 16;  // bytes per dim row of the transposed V tile
 constexpr int kFlashWaves = 4;
 
+// Position of key (0..63) inside a V^T row: bits 2 and 3 swapped (the accumulator layout holds keys
+// {0-3, 8-11} in one half-wave and {4-7, 12-15} in the other), then XOR with a per-dim-group value.
+__device__ __forceinline__ int vt_pos(int key, int dim) {
+  const int p = (key & ~12) | ((key & 4) << 1) | ((key & 8) >> 1);
+  return p ^ ((dim >> 4) << 3);
+}
+
 template <int G>
-__global__ __launch_bounds__(kFlashWaves * 64) void flash_attn_kernel(
+__global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
     const bf16_t* __restrict__ q, const int32_t* __restrict__ cu_q, const bf16_t* __restrict__ k,
     const bf16_t* __restrict__ v, const int64_t* __restrict__ kv_off, const int32_t* __restrict__ kv_len, int32_t B,
     int32_t Hq, int32_t Hkv, float scale_log2e, int32_t causal, bf16_t* __restrict__ out) {
   constexpr int kTokPerWave = 32 / G;
   constexpr int kTokPerBlock = kFlashWaves * kTokPerWave;
   __shared__ __align__(16) char lds_k[kKeysPerTile * kTileStride];
-  __shared__ __align__(16) char lds_v[kKeysPerTile * kTileStride];
+  __shared__ __align__(16) char lds_v[kHeadDim * kVtStride];
 
   // which (sample, token block) is this workgroup?  B is small; the scan is uniform.
   int blk = blockIdx.x, b = 0;
@@ -80,6 +89,9 @@ __global__ __launch_bounds__(kFlashWaves * 64) void flash_attn_kernel(
 #pragma unroll
     for (int e = 0; e < 16; ++e) o[d][e] = 0.f;
   float m = -INFINITY, l = 0.f;
+  int wave_min_limit = limit;               // tiles that end below it need no masking in this wavefront
+#pragma unroll
+  for (int x = 32; x > 0; x >>= 1) wave_min_limit = min(wave_min_limit, __shfl_xor(wave_min_limit, x));
 
   uint4 rk[4], rv[4];
   auto gload = [&](int t) {
@@ -103,7 +115,12 @@ __global__ __launch_bounds__(kFlashWaves * 64) void flash_attn_kernel(
       const int vv = tid + i * kFlashWaves * 64;
       const int at = (vv >> 4) * kTileStride + (vv & 15) * 16;
       *reinterpret_cast<uint4*>(lds_k + at) = rk[i];
-      *reinterpret_cast<uint4*>(lds_v + at) = rv[i];
+      const int key = vv >> 4, d0 = (vv & 15) * 8;
+      const uint32_t w[4] = {rv[i].x, rv[i].y, rv[i].z, rv[i].w};
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        *reinterpret_cast<bf16_t*>(lds_v + (d0 + e) * kVtStride + vt_pos(key, d0 + e) * 2) =
+            (bf16_t)(w[e >> 1] >> (16 * (e & 1)));
     }
   };
 
@@ -131,48 +148,64 @@ __global__ __launch_bounds__(kFlashWaves * 64) void flash_attn_kernel(
     // online softmax of this lane's column; element e of block rb is key 64 t + 32 rb + 8 (e / 4) + 4 half + e % 4
     const int key_base = t * kKeysPerTile + 4 * half;
     float mx = m;
+    if ((t + 1) * kKeysPerTile <= wave_min_limit) {    // interior tile: every key visible to every column
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+      for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const int key = key_base + 32 * rb + 8 * (e >> 2) + (e & 3);
-        const float x = key < limit ? s[rb][e] * scale_log2e : -INFINITY;
-        s[rb][e] = x;
-        mx = fmaxf(mx, x);
-      }
+        for (int e = 0; e < 16; ++e) {
+          s[rb][e] *= scale_log2e;
+          mx = fmaxf(mx, s[rb][e]);
+        }
+    } else {
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const int key = key_base + 32 * rb + 8 * (e >> 2) + (e & 3);
+          const float x = key < limit ? s[rb][e] * scale_log2e : -INFINITY;
+          s[rb][e] = x;
+          mx = fmaxf(mx, x);
+        }
+    }
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const bool none = mx == -INFINITY;                 // nothing visible to this column so far
-    const float alpha = none ? 1.f : exp2f(m - mx);
+    // Lazy rescaling: keep the old reference maximum while the new one is at most 2^6 above it; the
+    // probabilities are then at most 64 (exact in bf16's range) and the accumulators are untouched.
+    // The decision is wave-uniform so the 64 accumulator multiplies are skipped as a block.
+    const bool grow = !none && mx > m + 6.0f;
+    if (__any(grow)) {
+      const float mref = none ? m : mx;
+      const float alpha = (none || m == -INFINITY) ? (m == -INFINITY ? 0.f : 1.f) : exp2f(m - mref);
+      l *= alpha;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) o[d][e] *= alpha;
+      m = mref;
+    }
     float psum = 0.f;
     bf16x8_t pf[2][2];
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const float p = none ? 0.f : exp2f(s[rb][e] - mx);
+        const float p = none ? 0.f : exp2f(s[rb][e] - m);
         psum += p;
         pf[rb][e >> 3][e & 7] = (__bf16)p;
       }
     psum += __shfl_xor(psum, 32);
-    l = l * alpha + psum;
-    m = mx;
-#pragma unroll
-    for (int d = 0; d < 4; ++d)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) o[d][e] *= alpha;
+    l += psum;
 
     // O^T += V^T . P^T: the k slots of step (rb, j) are the keys this lane's P values belong to
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
-        const char* vbase = lds_v + (32 * rb + 16 * j + 4 * half) * kTileStride + col * 2;
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          bf16x8_t a;
-#pragma unroll
-          for (int i = 0; i < 8; ++i)
-            a[i] = *reinterpret_cast<const __bf16*>(vbase + (8 * (i >> 2) + (i & 3)) * kTileStride + d * 64);
+          const int dim = 32 * d + col;
+          const int pos = (32 * rb + 16 * j + 8 * half) ^ ((dim >> 4) << 3);      // 8 keys of this half, in slot order
+          const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(lds_v + dim * kVtStride + pos * 2);
           o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[rb][j], o[d], 0, 0, 0);
         }
       }

@@ -5,14 +5,11 @@
 // per key, 8 head-dim elements per lane); every (key slot, dim slice) lane keeps an independent
 // online-softmax state (m, l, acc[G][8]) that is merged across slots, wavefronts and finally
 // splits (second kernel).  K / V rows are [Hkv, 128].
-#include <algorithm>
-
-#include "common.h"
+#include "attn_internal.h"
 
 namespace {
 
 constexpr int kAttnWaves = 4;
-constexpr int kMinSplitKeys = 256;   // fewest keys worth a workgroup of its own
 constexpr int kMaxG = 8;
 
 template <typename T>
@@ -187,21 +184,6 @@ __global__ __launch_bounds__(kHeadDim) void attn_combine_kernel(const float* __r
   else out[rh * kHeadDim + d] = o;
 }
 
-// Splits of the key range: enough workgroups to fill the chip (about 2048) when there are few
-// (query row, KV head) pairs, a single pass over the keys when there are many.
-struct SplitPlan {
-  int n_split;
-  int split_keys;
-};
-inline SplitPlan plan_splits(int64_t total_q, int32_t Hkv, int32_t max_kv) {
-  const int64_t pairs = std::max<int64_t>(1, total_q * Hkv);
-  const int by_fill = (int)std::max<int64_t>(1, (2048 + pairs - 1) / pairs);
-  const int by_size = std::max(1, (max_kv + kMinSplitKeys - 1) / kMinSplitKeys);
-  const int n = std::min(by_fill, by_size);
-  const int keys = ((max_kv + n - 1) / n + 63) / 64 * 64;
-  return {(max_kv + keys - 1) / keys, keys};
-}
-
 template <typename T>
 int launch_attn(const void* q, const int32_t* cu_q, const void* k, const void* v, const int64_t* kv_off,
                 const int32_t* kv_len, int32_t B, int32_t total_q, int32_t Hq, int32_t Hkv, float scale,
@@ -266,9 +248,20 @@ extern "C" int msa_sparse_attn(const void* q, const int32_t* cu_q, const void* k
   float* part_ml = static_cast<float*>(workspace);
   float* part_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + align_up(n * 2 * sizeof(float), 256));
   hipStream_t st = as_stream(stream);
+  if (dtype == MSA_BF16 && max_sq >= 8) {
+    // bf16 query blocks: MFMA partial pass (K / V tiles through LDS) + the common combine; single rows
+    // (decode) stay on the split-KV kernel below, which keeps more loads in flight per wavefront
+    int rc = flash_attn_split_launch(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, plan, part_ml,
+                                     part_acc, st);
+    if (rc != MSA_OK) return rc;
+    attn_combine_kernel<bf16_t><<<(unsigned)((int64_t)total_q * Hq), kHeadDim, 0, st>>>(part_ml, part_acc, n_split,
+                                                                                      static_cast<bf16_t*>(out));
+    MSA_LAUNCH_CHECK();
+    return MSA_OK;
+  }
   if (dtype == MSA_BF16)
-    return launch_attn<bf16_t>(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, plan, out,
-                               part_ml, part_acc, st);
+    return launch_attn<bf16_t>(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, plan, out, part_ml,
+                               part_acc, st);
   return launch_attn<float>(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, plan, out, part_ml,
                             part_acc, st);
 }

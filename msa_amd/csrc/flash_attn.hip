@@ -12,9 +12,7 @@
 // leaves registers.  V is transposed on its way into LDS (16-bit stores into [dim][key] rows with
 // that key order, XOR-swizzled so the stores of a wavefront spread over all banks) and read back
 // as 16-byte operands.
-#include <algorithm>
-
-#include "common.h"
+#include "attn_internal.h"
 
 namespace {
 
@@ -33,11 +31,14 @@ __device__ __forceinline__ int vt_pos(int key, int dim) {
   return p ^ ((dim >> 4) << 3);
 }
 
-template <int G>
+// kSplit: blockIdx.z selects a range of split_keys keys; the un-normalised accumulators and the
+// (reference max, sum) pair of every column go to part_acc / part_ml for the combine kernel.
+template <int G, bool kSplit>
 __global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
     const bf16_t* __restrict__ q, const int32_t* __restrict__ cu_q, const bf16_t* __restrict__ k,
     const bf16_t* __restrict__ v, const int64_t* __restrict__ kv_off, const int32_t* __restrict__ kv_len, int32_t B,
-    int32_t Hq, int32_t Hkv, float scale_log2e, int32_t causal, bf16_t* __restrict__ out) {
+    int32_t Hq, int32_t Hkv, float scale_log2e, int32_t causal, bf16_t* __restrict__ out, int32_t n_split,
+    int32_t split_keys, float* __restrict__ part_ml, float* __restrict__ part_acc) {
   constexpr int kTokPerWave = 32 / G;
   constexpr int kTokPerBlock = kFlashWaves * kTokPerWave;
   __shared__ __align__(16) char lds_k[kKeysPerTile * kTileStride];
@@ -67,8 +68,13 @@ __global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
   const bool col_ok = tok < sq;
   const int limit = col_ok ? (causal ? max(0, L - sq + tok + 1) : L) : 0;   // this column sees keys [0, limit)
   const int last_tok = min(sq, t0 + kTokPerBlock) - 1;
-  const int kmax = causal ? max(0, min(L, L - sq + last_tok + 1)) : L;       // the block sees keys [0, kmax)
-  const int n_tiles = (kmax + kKeysPerTile - 1) / kKeysPerTile;
+  int kmax = causal ? max(0, min(L, L - sq + last_tok + 1)) : L;             // the block sees keys [0, kmax)
+  int first_tile = 0;
+  if constexpr (kSplit) {
+    first_tile = blockIdx.z * (split_keys / kKeysPerTile);
+    kmax = min(kmax, (int)(blockIdx.z + 1) * split_keys);
+  }
+  const int n_tiles = (kmax + kKeysPerTile - 1) / kKeysPerTile;              // tiles first_tile .. n_tiles - 1
   const int row_elems = Hkv * kHeadDim;
 
   // Q^T operand fragments stay in registers for the whole pass: lane (col, half), step s holds
@@ -124,8 +130,8 @@ __global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
     }
   };
 
-  if (n_tiles > 0) gload(0);
-  for (int t = 0; t < n_tiles; ++t) {
+  if (first_tile < n_tiles) gload(first_tile);
+  for (int t = first_tile; t < n_tiles; ++t) {
     __syncthreads();                 // everyone is done reading the previous tile
     lstore();
     __syncthreads();
@@ -211,7 +217,19 @@ __global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
       }
   }
 
-  if (col_ok) {
+  if constexpr (kSplit) {
+    if (col_ok) {
+      const int64_t slot = ((int64_t)(q_first + tok) * Hq + head) * n_split + blockIdx.z;
+      if (half == 0) { part_ml[slot * 2] = m; part_ml[slot * 2 + 1] = l; }
+      float* prow = part_acc + slot * kHeadDim;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+#pragma unroll
+        for (int e4 = 0; e4 < 4; ++e4)
+          *reinterpret_cast<float4*>(prow + 32 * d + 8 * e4 + 4 * half) =
+              make_float4(o[d][4 * e4], o[d][4 * e4 + 1], o[d][4 * e4 + 2], o[d][4 * e4 + 3]);
+    }
+  } else if (col_ok) {
     const float inv = l > 0.f ? 1.0f / l : 0.f;        // a row that sees no key yields zeros
     bf16_t* orow = out + ((int64_t)(q_first + tok) * Hq + head) * kHeadDim;
 #pragma unroll
@@ -247,9 +265,9 @@ extern "C" int msa_flash_attn(const void* q, const int32_t* cu_q, const void* k,
   hipStream_t st = as_stream(stream);
 #define MSA_FLASH_CASE(GG)                                                                                        \
   case GG:                                                                                                        \
-    flash_attn_kernel<GG><<<grid, kFlashWaves * 64, 0, st>>>(                                                     \
+    flash_attn_kernel<GG, false><<<grid, kFlashWaves * 64, 0, st>>>(                                              \
         static_cast<const bf16_t*>(q), cu_q, static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v), kv_off, \
-        kv_len, B, Hq, Hkv, sl2, causal, static_cast<bf16_t*>(out));                                              \
+        kv_len, B, Hq, Hkv, sl2, causal, static_cast<bf16_t*>(out), 1, 0, nullptr, nullptr);                      \
     break;
   switch (G) {
     MSA_FLASH_CASE(1)
@@ -258,6 +276,35 @@ extern "C" int msa_flash_attn(const void* q, const int32_t* cu_q, const void* k,
     MSA_FLASH_CASE(8)
   }
 #undef MSA_FLASH_CASE
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
+
+int flash_attn_split_launch(const void* q, const int32_t* cu_q, const void* k, const void* v, const int64_t* kv_off,
+                            const int32_t* kv_len, int32_t B, int32_t total_q, int32_t Hq, int32_t Hkv, float scale,
+                            int32_t causal, SplitPlan plan, float* part_ml, float* part_acc, hipStream_t st) {
+  const int G = Hq / Hkv;
+  const int tok_per_block = kFlashWaves * 32 / G;
+  const int64_t blocks = ((int64_t)total_q + tok_per_block - 1) / tok_per_block + B;   // upper bound over ragged samples
+  MSA_REQUIRE(blocks < (int64_t)1 << 31, "msa_sparse_attn: too many query rows");
+  dim3 grid((unsigned)blocks, (unsigned)Hkv, (unsigned)plan.n_split);
+  const float sl2 = scale * 1.4426950408889634f;
+#define MSA_FLASH_SPLIT_CASE(GG)                                                                                  \
+  case GG:                                                                                                        \
+    flash_attn_kernel<GG, true><<<grid, kFlashWaves * 64, 0, st>>>(                                               \
+        static_cast<const bf16_t*>(q), cu_q, static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v), kv_off, \
+        kv_len, B, Hq, Hkv, sl2, causal, nullptr, plan.n_split, plan.split_keys, part_ml, part_acc);              \
+    break;
+  switch (G) {
+    MSA_FLASH_SPLIT_CASE(1)
+    MSA_FLASH_SPLIT_CASE(2)
+    MSA_FLASH_SPLIT_CASE(4)
+    MSA_FLASH_SPLIT_CASE(8)
+    default:
+      msa_set_error("msa_sparse_attn: GQA group size %d unsupported (1, 2, 4, 8)", G);
+      return MSA_EINVAL;
+  }
+#undef MSA_FLASH_SPLIT_CASE
   MSA_LAUNCH_CHECK();
   return MSA_OK;
 }

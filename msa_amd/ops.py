@@ -262,7 +262,9 @@ def sparse_attn(q, k, v, kv_off, kv_len, max_kv: int, cu_q=None, max_sq: int = 1
         raise ValueError("kv_off int64, kv_len / cu_q int32")
     lib = _lib.load()
     sc = D ** -0.5 if scale is None else scale
-    if q.dtype == torch.bfloat16 and max_sq >= FLASH_MIN_ROWS:
+    # long bf16 query blocks: one-pass MFMA flash kernel when there are enough blocks to fill the chip, otherwise the
+    # split-KV entry point below (which runs the same MFMA kernel per key range for bf16 blocks of >= 8 rows)
+    if q.dtype == torch.bfloat16 and max_sq >= FLASH_MIN_ROWS and total_q * Hkv >= 32 * 512:
         out = torch.empty_like(q)
         check(lib.msa_flash_attn(ptr(q), ptr(cu_q), ptr(k), ptr(v), ptr(kv_off), ptr(kv_len), B, total_q, Hq, Hkv, D, sc,
                                  int(causal), ptr(out), _stream()), "msa_flash_attn")

@@ -131,6 +131,16 @@ int msa_gather_kv(const msa_bank* bank, int32_t layer, const int32_t* doc_sel_ho
                   int32_t k, void* k_out, void* v_out, int64_t out_capacity_chunks,
                   void* copy_stream);
 
+/* Device-side variant of the same gather: the selection stays on the device (doc_sel[B, k] int32, e.g. msa_route_topk's
+ * doc_out; -1 or out-of-range entries are skipped), a planning kernel sorts / de-duplicates it per sample and writes
+ * cu_sel[B+1] (device int32), and a copy kernel reads the rows straight from the pinned host bank.  Nothing
+ * synchronises and nothing is copied to the host; rows past out_capacity_chunks are dropped, so size the outputs for
+ * B * k * (largest document's chunks).  k <= 64. */
+size_t msa_gather_device_workspace_bytes(int32_t B, int32_t k);
+int msa_gather_kv_device(const msa_bank* bank, int32_t layer, const int32_t* doc_sel, int32_t B,
+                         int32_t k, void* k_out, void* v_out, int64_t out_capacity_chunks,
+                         int32_t* cu_sel, void* workspace, size_t workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Context assembly.  Replaces the ragged scatter of src/msa/memory_sparse_attention.py:282-329
  * and the compact cache of :344-351: for every sample b writes

@@ -34,6 +34,8 @@ SIGNATURES = {
     "msa_profile_collect": (C.c_int, [_vp, _i32, _vp]),
     "msa_gather_plan": (C.c_int, [_vp, _vp, _i32, _i32, _vp]),
     "msa_gather_kv": (C.c_int, [_vp, _i32, _vp, _i32, _i32, _vp, _vp, _i64, _vp]),
+    "msa_gather_device_workspace_bytes": (_sz, [_i32, _i32]),
+    "msa_gather_kv_device": (C.c_int, [_vp, _i32, _vp, _i32, _i32, _vp, _vp, _i64, _vp, _vp, _sz, _vp]),
     "msa_assemble_context": (C.c_int, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp,
                                        _vp, _i32, _vp, _vp]),
     "msa_cache_append": (C.c_int, [_vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp]),

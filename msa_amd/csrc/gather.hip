@@ -88,3 +88,126 @@ extern "C" int msa_gather_kv(const msa_bank* bank, int32_t layer, const int32_t*
   }
   return MSA_OK;
 }
+
+// ------------------------------------------------------------------------------------------
+// Device-side gather: no ids on the host, no per-document copies.  A one-workgroup planning
+// kernel sorts and de-duplicates each sample's selection (one wavefront per sample, bitonic
+// network over the <= 64 picks), prefix-sums the chunk counts into cu_sel and emits one
+// (source chunk, rows, destination row) entry per kept document; a copy kernel then pulls the
+// rows straight out of the pinned host bank (the pointers are device-visible) with 16-byte loads.
+// ------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int kPlanWaves = 4;
+
+__global__ __launch_bounds__(kPlanWaves * 64) void gather_plan_kernel(const int32_t* __restrict__ doc_sel,
+                                                                      const int32_t* __restrict__ doc_chunk_off,
+                                                                      int32_t n_docs, int32_t B, int32_t k,
+                                                                      int32_t* __restrict__ cu_sel,
+                                                                      int32_t* __restrict__ plan /* [B*k][3] */) {
+  extern __shared__ int32_t totals[];          // [B + 1]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // pass 1 and 2 share this per-sample routine: sorted unique documents in lanes, chunk counts, in-sample offsets
+  auto sample = [&](int b, int32_t& d_out, int32_t& n_out, int32_t& off_out) -> int32_t {
+    int32_t d = 0x7fffffff;
+    if (lane < k) {
+      const int32_t x = doc_sel[(int64_t)b * k + lane];
+      if (x >= 0 && x < n_docs) d = x;
+    }
+#pragma unroll
+    for (int kk = 2; kk <= 64; kk <<= 1)
+#pragma unroll
+      for (int j = kk >> 1; j > 0; j >>= 1) {            // ascending bitonic sort
+        const int32_t o = __shfl_xor(d, j);
+        const bool asc = (lane & kk) == 0, lower = (lane & j) == 0;
+        d = (lower == asc) ? min(d, o) : max(d, o);
+      }
+    const int32_t prev = __shfl_up(d, 1);
+    const bool keep = d != 0x7fffffff && (lane == 0 || prev != d);
+    int32_t n = keep ? doc_chunk_off[d + 1] - doc_chunk_off[d] : 0;
+    int32_t incl = n;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int32_t t = __shfl_up(incl, o);
+      if (lane >= o) incl += t;
+    }
+    d_out = keep ? d : -1; n_out = n; off_out = incl - n;
+    return __shfl(incl, 63);
+  };
+  for (int b = wave; b < B; b += kPlanWaves) {
+    int32_t d, n, off;
+    const int32_t total = sample(b, d, n, off);
+    if (lane == 0) totals[b + 1] = total;
+  }
+  if (threadIdx.x == 0) totals[0] = 0;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t run = 0;
+    for (int b = 0; b < B; ++b) { run += totals[b + 1]; totals[b + 1] = run; }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i <= B; i += kPlanWaves * 64) cu_sel[i] = totals[i];
+  for (int b = wave; b < B; b += kPlanWaves) {
+    int32_t d, n, off;
+    sample(b, d, n, off);
+    if (lane < k) {
+      int32_t* e = plan + ((int64_t)b * k + lane) * 3;
+      e[0] = d >= 0 ? doc_chunk_off[d] : 0;
+      e[1] = n;
+      e[2] = totals[b] + off;
+    }
+  }
+}
+
+// grid.x = plan entry, grid.y = row group; 128 lanes move one 2 KB row of K and of V per step.
+__global__ __launch_bounds__(128) void gather_copy_kernel(const uint4* __restrict__ k_src, const uint4* __restrict__ v_src,
+                                                          const int32_t* __restrict__ plan, int32_t row_vecs,
+                                                          int64_t capacity_rows, uint4* __restrict__ k_dst,
+                                                          uint4* __restrict__ v_dst) {
+  const int32_t* e = plan + (int64_t)blockIdx.x * 3;
+  const int32_t src0 = e[0], n = e[1], dst0 = e[2];
+  for (int r = blockIdx.y; r < n; r += gridDim.y) {
+    if ((int64_t)dst0 + r >= capacity_rows) return;
+    const uint4* ks = k_src + ((int64_t)src0 + r) * row_vecs;
+    const uint4* vs = v_src + ((int64_t)src0 + r) * row_vecs;
+    uint4* kd = k_dst + ((int64_t)dst0 + r) * row_vecs;
+    uint4* vd = v_dst + ((int64_t)dst0 + r) * row_vecs;
+    for (int i = threadIdx.x; i < row_vecs; i += 128) { kd[i] = ks[i]; vd[i] = vs[i]; }
+  }
+}
+
+}  // namespace
+
+extern "C" size_t msa_gather_device_workspace_bytes(int32_t B, int32_t k) {
+  return B > 0 && k > 0 ? align_up((size_t)B * k * 3 * sizeof(int32_t), 256) : 0;
+}
+
+extern "C" int msa_gather_kv_device(const msa_bank* bank, int32_t layer, const int32_t* doc_sel, int32_t B, int32_t k,
+                                    void* k_out, void* v_out, int64_t out_capacity_chunks, int32_t* cu_sel,
+                                    void* workspace, size_t workspace_bytes, void* stream) {
+  MSA_REQUIRE(bank && doc_sel && k_out && v_out && cu_sel && workspace, "msa_gather_kv_device: null pointer");
+  MSA_REQUIRE(B > 0 && B <= 8192 && k > 0 && k <= 64, "msa_gather_kv_device: B=%d k=%d out of range", B, k);
+  MSA_REQUIRE(layer >= 0 && layer < bank->n_layers, "msa_gather_kv_device: layer %d out of range", layer);
+  MSA_REQUIRE(out_capacity_chunks > 0, "msa_gather_kv_device: empty output");
+  if (!bank->k_host[layer] || !bank->v_host[layer]) {
+    msa_set_error("msa_gather_kv_device: layer %d has no host K / V set", layer);
+    return MSA_ESTATE;
+  }
+  if (workspace_bytes < msa_gather_device_workspace_bytes(B, k)) {
+    msa_set_error("msa_gather_kv_device: workspace of %zu bytes, need %zu", workspace_bytes,
+                  msa_gather_device_workspace_bytes(B, k));
+    return MSA_ESIZE;
+  }
+  hipStream_t st = as_stream(stream);
+  int32_t* plan = static_cast<int32_t*>(workspace);
+  gather_plan_kernel<<<1, kPlanWaves * 64, (size_t)(B + 1) * sizeof(int32_t), st>>>(
+      doc_sel, bank->doc_chunk_off_dev, (int32_t)bank->n_docs, B, k, cu_sel, plan);
+  MSA_LAUNCH_CHECK();
+  const int32_t row_vecs = (int32_t)((size_t)bank->Hkv * bank->D * elem_bytes(bank->dtype) / 16);
+  dim3 grid((unsigned)(B * k), 8);
+  gather_copy_kernel<<<grid, 128, 0, st>>>(static_cast<const uint4*>(bank->k_host[layer]),
+                                           static_cast<const uint4*>(bank->v_host[layer]), plan, row_vecs,
+                                           out_capacity_chunks, static_cast<uint4*>(k_out), static_cast<uint4*>(v_out));
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}

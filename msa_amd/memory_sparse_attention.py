@@ -204,26 +204,35 @@ class MemorySparseAttention(nn.Module):
 
         valid = attention_mask == 1
         n_q = valid.sum(dim=1)
-        n_q_host = n_q.tolist()
+        n_q_host = cache.meta.get("q_lens_host")              # the model computes it once per forward
+        if n_q_host is None or len(n_q_host) != B:
+            n_q_host = n_q.tolist()
         mem_k = mem_v = cu_sel = None
-        n_sel_host = [0] * B
+        max_sel = 0
         if self.is_router_layer:
             rq = self.router_q_proj(hidden_states).view(B, S, Hq, D) if self.decouple_router else q
             query_mask = (doc_ids == 0) & valid
-            mem_k, mem_v, scores, n_sel, gids = self.memory_client.doc_query(
-                rq.transpose(1, 2), query_mask, self.layer_idx, fused_normalize=(self.aux_loss_method == "INFONCE"),
-                native_layout=True)
-            n_sel_host = n_sel.tolist()
-            cu_sel = F.pad(n_sel.cumsum(0), (1, 0)).to(torch.int32)
+            fused = self.aux_loss_method == "INFONCE"
+            if hasattr(self.memory_client, "doc_query_device"):
+                # native client: routing, gather plan and host->device gather are enqueued without any host sync
+                mem_k, mem_v, cu_sel, scores, gids = self.memory_client.doc_query_device(rq.contiguous(), query_mask,
+                                                                                         self.layer_idx, fused)
+                max_sel = self.top_k_docs * self.memory_client.bank.max_doc_chunks
+            else:
+                mem_k, mem_v, scores, n_sel, gids = self.memory_client.doc_query(rq.transpose(1, 2), query_mask,
+                                                                                 self.layer_idx)
+                mem_k, mem_v = mem_k.permute(1, 0, 2).contiguous(), mem_v.permute(1, 0, 2).contiguous()
+                cu_sel = F.pad(n_sel.cumsum(0), (1, 0)).to(torch.int32)
+                max_sel = int(n_sel.max())
             if cache.meta.get("require_recall_topk", False):
                 ck["recall_topk"] = [{"topk_doc_ids": gids[i].tolist(), "score": scores[i].float().tolist()} for i in range(B)]
         local_k, local_v, q_rows = k[valid], v[valid], q[valid]           # ragged [sum S_b, H, D]
         cu_local = F.pad(n_q.cumsum(0), (1, 0)).to(torch.int32)
-        kv_host = [n_prefix + a + b for a, b in zip(n_sel_host, n_q_host)]
-        Lcap = max(kv_host) + self.decode_reserve
+        max_kv = n_prefix + max_sel + max(n_q_host)                       # upper bound of any sample's context rows
+        Lcap = max_kv + self.decode_reserve
         kc, vc, kv_len = ops.assemble_context(prefix_k, prefix_v, mem_k, mem_v, cu_sel, local_k, local_v, cu_local, B, Lcap)
         kv_off = torch.arange(B, dtype=torch.int64, device=dev) * Lcap
-        out_rows = ops.sparse_attn(q_rows, kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), kv_off, kv_len, max(kv_host),
+        out_rows = ops.sparse_attn(q_rows, kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), kv_off, kv_len, max_kv,
                                    cu_q=cu_local, max_sq=max(n_q_host), scale=self.scaling, causal=True)
         attn = torch.zeros((B, S, Hq * D), device=dev, dtype=dtype)
         attn[valid] = out_rows.view(-1, Hq * D)

@@ -66,6 +66,8 @@ class MSAModel(nn.Module):
 
     def forward(self, input_ids, attention_mask, position_ids, past_key_values, doc_ids):
         h = self.embed_tokens(input_ids)
+        if past_key_values is not None and attention_mask is not None and input_ids.shape[1] > 1:
+            past_key_values.meta["q_lens_host"] = attention_mask.sum(dim=1).tolist()   # one sync per forward, not per layer
         if h.is_cuda:
             for layer in self.layers:
                 h = layer(h, doc_ids, attention_mask, None, past_key_values, position_ids=position_ids)

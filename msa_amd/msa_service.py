@@ -249,6 +249,24 @@ class MSAService(Memory, MemoryClientBase):
             if callable(getattr(module, "set_memory_client", None)):
                 module.set_memory_client(self)
 
+    def doc_query_device(self, q_bshd: torch.Tensor, query_mask: Optional[torch.Tensor], layer_idx: int,
+                         fused_normalize: bool = True):
+        """The sync-free form the native layer uses: ``q_bshd [B, S, Hq, D]`` contiguous.  Routing, plan and gather
+        are all enqueued on the current stream; nothing is copied to the host.  Returns ``(K, V)`` buffers of
+        ``B * k * max_doc_chunks`` rows ``[rows, Hkv, D]``, ``cu_sel`` (device int32 ``[B + 1]``: rows
+        ``cu_sel[b] .. cu_sel[b + 1]`` are sample b's, documents in ascending bank order, each once), ``scores
+        [B, k]`` fp32 and ``global_ids [B, k]`` (0 where nothing was selected)."""
+        if fused_normalize:
+            mode, scale = "cosine", 1.0
+        else:
+            mode, scale = "scaled_dot", (1.0 if self.scaling < 0 else self.scaling)
+        scores, doc, gid = self._route(layer_idx, q_bshd, query_mask, mode, scale)
+        doc = torch.where(scores > -1e9, doc, torch.full_like(doc, -1))      # drop invalid picks (:1190-1191)
+        B, k = doc.shape
+        cap = B * k * self.bank.max_doc_chunks
+        k_sel, v_sel, cu = ops.gather_kv_device(self.bank, self._layer_slot[layer_idx], doc.contiguous(), cap)
+        return k_sel, v_sel, cu, scores, torch.where(doc >= 0, gid, torch.zeros_like(gid))
+
     def doc_query(self, query_states: torch.Tensor, query_mask: torch.Tensor, layer_idx: int,
                   fused_normalize: bool = False, native_layout: bool = False):
         """``query_states [B, Hq, S, D]`` (the layer's ``.transpose(1, 2)`` view, normalised by the

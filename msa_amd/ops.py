@@ -114,6 +114,7 @@ class Bank:
         if self.off_host.numel() != self.n_docs + 1:
             raise ValueError("doc_chunk_off must have n_docs + 1 entries")
         self.C = int(self.off_host[-1])
+        self.max_doc_chunks = int((self.off_host[1:] - self.off_host[:-1]).max())
         self.n_layers, self.Hkv, self.D, self.dtype = n_layers, Hkv, D, dtype
         self._keep = {}
         self._ws: Optional[torch.Tensor] = None
@@ -210,6 +211,29 @@ def gather_kv(bank: Bank, layer: int, doc_sel_host: torch.Tensor, device, stream
         v_out = torch.empty_like(k_out)
     check(lib.msa_gather_kv(bank.handle, layer, ptr(sel), B, k, ptr(k_out), ptr(v_out), total, _stream(stream)),
           "msa_gather_kv")
+    return k_out, v_out, cu
+
+
+def gather_kv_device(bank: Bank, layer: int, doc_sel: torch.Tensor, capacity_chunks: int,
+                     out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
+    """Device-side gather: ``doc_sel [B, k]`` int32 on the device (e.g. ``route_topk``'s documents).  Returns
+    ``(K [capacity, Hkv, D], V, cu_sel int32 [B + 1] on the device)``; rows ``cu_sel[b] .. cu_sel[b + 1]`` belong to
+    sample ``b``.  No host synchronisation."""
+    _need_cuda(doc_sel)
+    if doc_sel.dtype != torch.int32 or doc_sel.dim() != 2:
+        raise ValueError("doc_sel must be int32 [B, k]")
+    B, k = doc_sel.shape
+    lib = _lib.load()
+    dev = doc_sel.device
+    if out is None:
+        k_out = torch.empty((capacity_chunks, bank.Hkv, bank.D), dtype=bank.dtype, device=dev)
+        v_out = torch.empty_like(k_out)
+    else:
+        k_out, v_out = out
+    cu = torch.empty(B + 1, dtype=torch.int32, device=dev)
+    ws = torch.empty(lib.msa_gather_device_workspace_bytes(B, k), dtype=torch.uint8, device=dev)
+    check(lib.msa_gather_kv_device(bank.handle, layer, ptr(doc_sel), B, k, ptr(k_out), ptr(v_out), capacity_chunks, ptr(cu),
+                                   ptr(ws), ws.numel(), _stream()), "msa_gather_kv_device")
     return k_out, v_out, cu
 
 

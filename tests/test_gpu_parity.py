@@ -254,6 +254,20 @@ def test_gather_kv_exact(ops, dtype):
     wk, wv, wcu, _ = cf.gather_selected(kh, vh, dco, sel)
     assert cu.tolist() == wcu.tolist()
     assert torch.equal(K.cpu(), wk) and torch.equal(V.cpu(), wv)
+    # device-side gather: same rows, same order, ids never leave the device; out-of-range ids are skipped
+    sel_dev = torch.cat([sel, torch.tensor([[300, -5, 7, 7, 7, 7, 7, 6]], dtype=torch.int32)]).cuda()
+    cap = sel_dev.shape[0] * sel_dev.shape[1] * bank.max_doc_chunks
+    Kd, Vd, cud = ops.gather_kv_device(bank, 1, sel_dev, cap)
+    torch.cuda.synchronize()
+    sel_ref = torch.cat([sel, torch.tensor([[-1, -1, 7, 7, 7, 7, 7, 6]], dtype=torch.int32)])
+    wk2, wv2, wcu2, _ = cf.gather_selected(kh, vh, dco, sel_ref)
+    assert cud.cpu().tolist() == wcu2.tolist()
+    n = int(wcu2[-1])
+    assert torch.equal(Kd[:n].cpu(), wk2) and torch.equal(Vd[:n].cpu(), wv2)
+    # a short output drops the overflowing rows instead of writing past the end
+    Ks, Vs, cus = ops.gather_kv_device(bank, 1, sel_dev, 10)
+    torch.cuda.synchronize()
+    assert torch.equal(Ks.cpu(), wk2[:10]) and cus.cpu().tolist() == wcu2.tolist()
     with pytest.raises(Exception, match="outside"):
         ops.gather_kv(bank, 1, torch.tensor([[300]], dtype=torch.int32), "cuda")
     with pytest.raises(Exception, match="no host K"):

@@ -209,6 +209,9 @@ def main():
     ap.add_argument("--seq", type=int, default=128)
     ap.add_argument("--host-kv-layers", type=int, default=2,
                     help="distinct pinned host K/V layer buffers (routed layers share them round-robin)")
+    ap.add_argument("--gather", choices=["device", "memcpy"], default="memcpy",
+                    help="device: plan + copy kernels read the pinned bank directly, no ids on the host; "
+                         "memcpy: ids to the host, one hipMemcpyAsync per document run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the pooling and decode-attention side measurements")
@@ -289,7 +292,21 @@ def main():
         _lib.check(lib.msa_gather_kv(bank.handle, li, docs_host[li].data_ptr(), B, TOPK, gk[li & 1].data_ptr(),
                                      gv[li & 1].data_ptr(), cap_chunks, side.cuda_stream), "msa_gather_kv")
 
+    cu_dev = [torch.empty(B + 1, dtype=torch.int32, device=dev) for _ in range(L)]
+    gws = torch.empty(lib.msa_gather_device_workspace_bytes(B, TOPK), dtype=torch.uint8, device=dev)
+
+    def gather_device(li):
+        side.wait_event(ready[li])         # no host wait: the side stream picks the ids up on the device
+        _lib.check(lib.msa_gather_kv_device(bank.handle, li, docs[li].data_ptr(), B, TOPK, gk[li & 1].data_ptr(),
+                                            gv[li & 1].data_ptr(), cap_chunks, cu_dev[li].data_ptr(), gws.data_ptr(),
+                                            gws.numel(), side.cuda_stream), "msa_gather_kv_device")
+
     def step():
+        if args.gather == "device":
+            for li in range(L):
+                route(li)
+                gather_device(li)          # runs on the side stream under the next layer's scan
+            return
         for li in range(L):
             route(li)                      # layer li is being scored ...
             if li > 0:
@@ -326,6 +343,8 @@ def main():
     wk, wv, wcu, _ = cf.gather_selected(host_k[last % n_host], host_v[last % n_host], doc_chunk_off,
                                         torch.as_tensor(wants[last]))
     n_sel = int(wcu[-1])
+    if args.gather == "device":
+        sel_chunks = [int(c[-1]) for c in cu_dev]
     if n_sel != sel_chunks[last] or not torch.equal(gk[last & 1][:n_sel].cpu(), wk) or \
             not torch.equal(gv[last & 1][:n_sel].cpu(), wv):
         sys.exit("bench.py: PARITY FAILURE: gathered K / V rows differ from the host bank")
@@ -407,7 +426,7 @@ def main():
         "config": {"workload": "configs[3]: 100M-token bank, K_r HBM-resident, K/V pinned host, B=16 x S=128, top-16",
                    "bank_tokens": args.tokens, "chunks": C_total, "docs": n_docs, "routed_layers": L, "batch": B,
                    "query_tokens": S, "top_k": TOPK, "kr_hbm_gb": round(C_total * HKV * D * 2 * L / 1e9, 1),
-                   "host_kv_layer_buffers": n_host, "selected_chunks_per_layer": int(np.mean(sel_chunks)),
+                   "host_kv_layer_buffers": n_host, "gather": args.gather, "selected_chunks_per_layer": int(np.mean(sel_chunks)),
                    "mode": "cosine/mean-heads/max-tokens/max-chunks"},
         "roofline": roof, "cpu_baseline": cpu, "hbm_regime_sweep": sweep, "other_kernels": extras, "parity": "needles exact on all layers",
     }

@@ -436,7 +436,7 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
     // Tile choice by query rows: small M is HBM-bound (narrow M tile, more workgroups in flight),
     // large M is MFMA-bound (256 x 256 tile, 8 wavefronts).  MSA_SCORE_TILE overrides for tuning.
     const char* ev = getenv("MSA_SCORE_TILE");
-    const int variant = ev ? atoi(ev) : (w.M_rows <= 64 ? 0 : w.M_rows <= 128 ? 1 : 2);
+    const int variant = ev ? atoi(ev) : (w.M_rows <= 64 ? 0 : w.M_rows <= 128 ? 6 : 2);
 #define MSA_GEMM(BM_, BN_, WM_, WN_)                                                                              \
   launch_gemm<bf16_t, BM_, BN_, WM_, WN_>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C, \
                                           K, bpq, st)
@@ -447,6 +447,10 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
       case 3: rc = MSA_GEMM(256, 256, 4, 2); break;
       case 4: rc = MSA_GEMM(128, 128, 2, 2); break;
       case 5: rc = MSA_GEMM(128, 128, 2, 4); break;
+      case 6: rc = MSA_GEMM(128, 384, 2, 4); break;
+      case 7: rc = MSA_GEMM(128, 256, 4, 2); break;
+      case 8: rc = MSA_GEMM(128, 256, 1, 8); break;
+      case 9: rc = MSA_GEMM(128, 192, 2, 2); break;
       default: msa_set_error("MSA_SCORE_TILE=%d unknown", variant); return MSA_EINVAL;
     }
 #undef MSA_GEMM

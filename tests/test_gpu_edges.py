@@ -1,0 +1,134 @@
+"""GPU edge cases of the C ABI: odd head counts, tiny and ragged shapes, extreme top-k, error codes.
+Everything is compared with the fp64 oracle on the same seeded inputs."""
+import ctypes as C
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import closed_form as cf
+
+pytestmark = pytest.mark.gpu
+
+
+def say(msg):
+    print(f"[case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not torch.cuda.is_available():
+        pytest.fail("no GPU visible")
+    from msa_amd import ops as _ops
+    return _ops
+
+
+def _randn(shape, seed, dtype):
+    return torch.randn(shape, generator=torch.Generator().manual_seed(seed)).to(dtype)
+
+
+def _bank(ops, doc_chunks, Hkv, dtype, seed):
+    _, dco, _, _, _ = cf.chunk_table([n * 4 for n in doc_chunks], 4)
+    kr = cf.l2_normalize(_randn((int(dco[-1]), Hkv, 128), seed, torch.float32)).float().to(dtype)
+    bank = ops.Bank(1, dco.tolist(), list(range(len(doc_chunks))), Hkv, 128, dtype)
+    dev = kr.cuda()
+    bank.set_layer(0, dev)
+    return bank, kr, dco, dev
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(8, 2), (16, 16), (4, 1), (64, 8)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_scores_head_layouts(ops, Hq, Hkv, dtype):
+    say(f"scores Hq={Hq} Hkv={Hkv} {dtype}")
+    bank, kr, dco, _ = _bank(ops, [3, 1, 7, 2, 9, 4] * 30, Hkv, dtype, 300 + Hq)
+    q = _randn((3, 37, Hq, 128), 301, dtype)
+    mask = torch.ones(3, 37, dtype=torch.bool); mask[0, 30:] = False
+    got = ops.chunk_scores(bank, 0, q.cuda(), mask.cuda())
+    assert cf.rel_err(got.cpu(), cf.chunk_scores(q, mask, kr, "cosine")) < (1e-2 if dtype == torch.bfloat16 else 1e-5)
+
+
+@pytest.mark.parametrize("B,S,topk", [(1, 1, 1), (33, 3, 64), (2, 200, 16), (300, 2, 5)])
+def test_route_extreme_shapes(ops, B, S, topk):
+    say(f"route B={B} S={S} topk={topk}")
+    bank, kr, dco, _ = _bank(ops, list(np.random.default_rng(3).integers(1, 5, size=700)), 8, torch.float32, 310)
+    q = _randn((B, S, 32, 128), 311, torch.float32)
+    s, d, g = ops.route_topk(bank, 0, q.cuda(), None, "cosine", 1.0, topk)
+    ds = cf.doc_scores(cf.chunk_scores(q, torch.ones(B, S, dtype=torch.bool), kr, "cosine"), dco)
+    assert not cf.topk_acceptable(ds, d.cpu().long(), topk, gap=1e-5)
+    ws, wi = cf.topk_docs(ds, topk)
+    assert cf.rel_err(s.cpu(), ws) < 1e-5
+    assert torch.equal(g.cpu(), d.cpu().long())
+
+
+def test_tiny_bank_and_single_chunk(ops):
+    say("bank smaller than one tile; one document of one chunk")
+    for doc_chunks in ([1], [2, 1, 1], [5]):
+        bank, kr, dco, _ = _bank(ops, doc_chunks, 8, torch.bfloat16, 320)
+        q = _randn((2, 9, 32, 128), 321, torch.bfloat16)
+        got = ops.chunk_scores(bank, 0, q.cuda())
+        assert cf.rel_err(got.cpu(), cf.chunk_scores(q, torch.ones(2, 9, dtype=torch.bool), kr, "cosine")) < 1e-2
+        s, d, _ = ops.route_topk(bank, 0, q.cuda(), None, "cosine", 1.0, 16)
+        n = len(doc_chunks)
+        assert (d.cpu()[:, n:] == -1).all() and sorted(d.cpu()[0, :n].tolist()) == list(range(n))
+
+
+@pytest.mark.parametrize("H", [1, 2, 4, 16, 32])
+@pytest.mark.parametrize("P", [1, 7, 64])
+def test_pool_head_counts_and_chunk_sizes(ops, H, P):
+    say(f"pool H={H} P={P}")
+    lens = [1, 2, P, P + 1, 3 * P + 2, 5]
+    T = sum(lens) + 1
+    x = _randn((T, H, 128), 330 + H, torch.float32)
+    t = ops.chunk_table(lens, P, first_token=1)
+    rope = ops.rope_tables(256, 128, 1e4)
+    pk, pv, pr = ops.pool_chunks(x.cuda(), x.cuda(), x.cuda(), t, rope=rope, normalize_kr=True)
+    _, _, cs, cl, _ = cf.chunk_table(lens, P, 1)
+    pos = torch.as_tensor(cf.doc_positions(lens, 1))
+    assert cf.rel_err(pv.cpu(), cf.pool_chunks(x, cs, cl)) < 1e-5
+    assert cf.rel_err(pr.cpu(), cf.l2_normalize(cf.pool_chunks(x, cs, cl))) < 1e-5
+    assert cf.rel_err(pk.cpu(), cf.pool_chunks(cf.apply_rope(x, pos, 1e4), cs, cl)) < 2e-5
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(8, 1), (8, 8), (16, 2)])
+def test_decode_attention_group_sizes(ops, Hq, Hkv):
+    say(f"decode attention Hq={Hq} Hkv={Hkv}")
+    L = [1, 63, 64, 65, 700]
+    B, cap = len(L), max(L)
+    for dtype, tol in ((torch.bfloat16, 1e-2), (torch.float32, 1e-5)):
+        k, v = _randn((B, cap, Hkv, 128), 340, dtype), _randn((B, cap, Hkv, 128), 341, dtype)
+        q = _randn((B, Hq, 128), 342, dtype)
+        out = ops.sparse_attn(q.cuda(), k.cuda().view(-1, Hkv, 128), v.cuda().view(-1, Hkv, 128),
+                              (torch.arange(B, dtype=torch.int64) * cap).cuda(), torch.tensor(L, dtype=torch.int32).cuda(), cap)
+        for b in range(B):
+            assert cf.rel_err(out[b:b + 1].cpu(), cf.attention(q[b:b + 1], k[b, :L[b]], v[b, :L[b]])) < tol
+
+
+def test_error_codes(ops):
+    say("error codes")
+    from msa_amd import _lib
+    lib = _lib.load()
+    bank, kr, dco, kr_dev = _bank(ops, [2, 3], 8, torch.bfloat16, 350)
+    q = _randn((1, 4, 32, 128), 351, torch.bfloat16).cuda()
+    out = torch.empty(1, bank.C, device="cuda")
+    ws = torch.empty(1024, dtype=torch.uint8, device="cuda")
+    rc = lib.msa_chunk_scores(bank.handle, 0, q.data_ptr(), None, 1, 4, 32, 0, 1.0, out.data_ptr(), ws.data_ptr(), 1024, None)
+    assert rc == -3 and b"workspace" in lib.msa_last_error()                      # MSA_ESIZE
+    two = ops.Bank(2, dco.tolist(), [0, 1], 8, 128, torch.bfloat16)
+    two.set_layer(0, kr_dev)
+    with pytest.raises(_lib.MsaError, match="no K_r") as ei:
+        ops.chunk_scores(two, 1, q)
+    assert ei.value.code == -4                                                    # MSA_ESTATE
+    with pytest.raises(_lib.MsaError, match="out of range"):
+        ops.chunk_scores(two, 2, q)
+    with pytest.raises(_lib.MsaError, match="multiple of Hkv"):
+        ops.chunk_scores(two, 0, _randn((1, 4, 12, 128), 352, torch.bfloat16).cuda())
+    with pytest.raises(NotImplementedError):
+        ops.chunk_scores(two, 0, q, mode="l2")
+    with pytest.raises(ValueError, match="pinned"):
+        two.set_layer(1, kr_dev, kr.clone(), kr.clone())
+    with pytest.raises(_lib.MsaError, match="rotary table"):
+        t = ops.chunk_table([300], 64)
+        x = _randn((300, 8, 128), 353, torch.bfloat16).cuda()
+        ops.pool_chunks(x, None, None, t, rope=ops.rope_tables(128, 128, 1e4))

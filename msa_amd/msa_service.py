@@ -9,6 +9,7 @@ Reference-shaped views (``[1, Hkv, C, D]``, ``[Hkv, n, D]``) are handed out wher
 """
 from __future__ import annotations
 
+import os
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -202,6 +203,50 @@ class Memory:
         self._kv_offset = self.block_desc.chunks()
         self.template_prefix_kvcache = {l: (a.to(self.device), b.to(self.device)) for l, (a, b) in template_prefix.items()}
         self._finish_bank()
+
+    # ---------------------------------------------------------------- storage (:351-479)
+    def serialize(self, path: str) -> None:
+        """Writes the bank as raw chunk-major arrays plus a JSON header (see ``bank_io``)."""
+        from . import bank_io
+        desc, mc = self.block_desc, self.msa_model_config.msa_config
+        off = torch.cat([desc.doc_offsets_cpu[1:], torch.tensor([desc.chunks()])]).tolist()
+        header = {"pooling_kernel_size": mc.pooling_kernel_size, "aux_loss_method": mc.aux_loss_method,
+                  "head_reduce_method": mc.head_reduce_method, "query_reduce_method": mc.query_reduce_method,
+                  "chunk_reduce_method": mc.chunk_reduce_method, "decouple_router": bool(mc.decouple_router)}
+        os.makedirs(path, exist_ok=True)
+        bank_io.save_docs(path, desc.docs)
+        bank_io.save_bank(path, header, off, desc.doc_ids_cpu[1:].tolist(), self._rk, self._k, self._v,
+                          self.template_prefix_kvcache)
+
+    def deserialize(self, path: str, docs: Optional[List[Document]] = None) -> None:
+        """Streams a stored bank back in: K_r to the device, K / V into freshly pinned host memory, one layer
+        at a time.  ``docs`` restores the document texts; without it placeholders carry ids and chunk counts."""
+        from . import bank_io
+        files = bank_io.BankFiles(path)
+        h = files.header
+        if h["router_layers"] != self.router_layer_ids:
+            raise ValueError(f"bank has router layers {h['router_layers']}, this model {self.router_layer_ids}")
+        mc = self.msa_model_config.msa_config
+        if h.get("aux_loss_method") != mc.aux_loss_method or h.get("pooling_kernel_size") != mc.pooling_kernel_size:
+            raise ValueError("bank was built with different scoring / pooling hyper-parameters")
+        counts = (files.doc_chunk_off[1:] - files.doc_chunk_off[:-1]).tolist()
+        if docs is None:
+            rows = bank_io.load_docs(path)
+            if rows is not None:
+                docs = [Document(doc=r["doc"], doc_id=r["doc_id"], num_chunks=r["num_chunks"]) for r in rows]
+        if docs is None:
+            docs = [Document(doc_id=int(g), num_chunks=int(n)) for g, n in zip(files.doc_global_id.tolist(), counts)]
+        if [d.num_chunks for d in docs] != counts or [d.doc_id for d in docs] != files.doc_global_id.tolist():
+            raise ValueError("documents do not match the stored bank")
+        rk, k, v = {}, {}, {}
+        for layer in self.router_layer_ids:
+            rk[layer] = torch.empty(files.shape, dtype=files.torch_dtype, device=self.device)
+            k[layer] = torch.empty(files.shape, dtype=files.torch_dtype, pin_memory=True)
+            v[layer] = torch.empty(files.shape, dtype=files.torch_dtype, pin_memory=True)
+            files.copy_into(layer, "rk", rk[layer])
+            files.copy_into(layer, "k", k[layer])
+            files.copy_into(layer, "v", v[layer])
+        self.load_pooled(docs, rk, k, v, files.prefix())
 
     def get_max_local_pool_doc_id(self) -> int:
         return int(self.block_desc.pool_ids_cpu[-1])

@@ -197,6 +197,22 @@ def test_layer_stage1_stage2_decode_against_oracle(env):
     assert float(s[0, -1]) == torch.finfo(torch.float32).min
     assert sorted(local[0, :-1].cpu().tolist()) == list(range(1, len(lens) + 1))
 
+    # ---- stored bank: serialize, stream back into a fresh service, same answers bit for bit
+    import tempfile
+    with tempfile.TemporaryDirectory() as tmp:
+        service.serialize(tmp)
+        fresh = svc_mod.MSAService(0, env["config"].GenerateConfig(devices=[0]),
+                                   env["config"].ModelConfig(doc_top_k=TOPK, pooling_kernel_size=P, router_layer_idx="1"),
+                                   env["config"].MemoryConfig(pooling_kernel_size=P), env["cfg"])
+        fresh.deserialize(tmp)
+    assert [d.doc for d in fresh.block_desc.docs] == [d.doc for d in docs]
+    assert torch.equal(fresh.block_desc.pool_ids_cpu, service.block_desc.pool_ids_cpu)
+    K2, V2, s3, n2, g3 = fresh.doc_query(rq, mask.bool().cuda(), 1)
+    assert torch.equal(K2, K) and torch.equal(V2, V) and torch.equal(s3, s2) and torch.equal(g3, g2) and torch.equal(n2, n_sel)
+    pk_a, pv_a = service.get_template_prefix_kvcaches(1)
+    pk_b, pv_b = fresh.get_template_prefix_kvcaches(1)
+    assert torch.equal(pk_a, pk_b) and torch.equal(pv_a, pv_b)
+
 
 def test_unsupported_reductions_raise(env):
     say("unsupported reduce methods")

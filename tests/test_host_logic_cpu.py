@@ -91,3 +91,38 @@ def test_configs():
     assert cfg.msa_config.top_k_docs == 4 and cfg.msa_config.missing is None
     d = mconfig.MSAConfig()
     assert d.msa_config.router_layer_idx.split(",")[0] == "18" and d.num_key_value_heads == 8
+
+
+def test_bank_files_round_trip(tmp_path):
+    """The on-disk bank format: raw arrays + JSON header, memory-mapped back bit for bit."""
+    from msa_amd import bank_io
+    g = torch.Generator().manual_seed(0)
+    off = [0, 2, 5, 6]
+    C, Hkv, D = 6, 2, 128
+    for dtype in (torch.bfloat16, torch.float32):
+        mk = lambda: torch.randn((C, Hkv, D), generator=g).to(dtype)
+        rk, k, v = {3: mk(), 5: mk()}, {3: mk(), 5: mk()}, {3: mk(), 5: mk()}
+        prefix = {l: (torch.randn((1, Hkv, 3, D), generator=g).to(dtype), torch.randn((1, Hkv, 3, D), generator=g).to(dtype))
+                  for l in range(6)}
+        path = str(tmp_path / f"bank_{dtype}".replace(".", "_"))
+        bank_io.save_bank(path, {"pooling_kernel_size": 64, "aux_loss_method": "INFONCE"}, off, [10, 11, 12], rk, k, v, prefix)
+        f = bank_io.BankFiles(path)
+        assert f.header["chunks"] == C and f.header["router_layers"] == [3, 5] and f.header["pooling_kernel_size"] == 64
+        assert f.doc_chunk_off.tolist() == off and f.doc_global_id.tolist() == [10, 11, 12]
+        for layer in (3, 5):
+            for tag, store in (("rk", rk), ("k", k), ("v", v)):
+                dst = torch.empty((C, Hkv, D), dtype=dtype)
+                f.copy_into(layer, tag, dst, rows_per_step=4)
+                assert torch.equal(dst, store[layer])
+        back = f.prefix()
+        assert sorted(back) == list(range(6))
+        assert torch.equal(back[4][0], prefix[4][0]) and torch.equal(back[4][1], prefix[4][1])
+    # a truncated layer file is refused, and so is a missing header
+    with open(f"{path}/layer_3.k.bin", "r+b") as fh:
+        fh.truncate(100)
+    with pytest.raises(ValueError, match="bytes, expected"):
+        bank_io.BankFiles(path).layer(3, "k")
+    import os
+    os.remove(f"{path}/bank.json")
+    with pytest.raises(FileNotFoundError):
+        bank_io.BankFiles(path)

@@ -200,6 +200,22 @@ int msa_rmsnorm(const void* x, void* residual, const void* weight, int32_t dtype
                 int32_t H, float eps, void* out, void* stream);
 int msa_silu_mul(const void* gate_up, int32_t dtype, int64_t N, int32_t I, void* out, void* stream);
 
+/* Linear layer for the few rows of a decode step: y[M, N] = x[M, K] . w[N, K]^T, bf16, M <= 16,
+ * K a multiple of 128, w in torch.nn.Linear layout (the F.linear calls behind q/k/v/o_proj and the MLP at
+ * src/msa/memory_sparse_attention.py:125-127, 405 when one token per sample is decoded).  The weight matrix is
+ * streamed from HBM once.  epilogue 0: plain; 1: y = residual + bf16(x w^T) (residual [M, N]); 2: w holds
+ * alternating 16-row groups of gate and up rows (N = 2 I) and y[M, I] = silu(gate) * up, both products rounded
+ * to bf16 first as the unfused sequence does.  With norm_w [K] the RMSNorm in front of the projection is folded
+ * in: the operand is bf16(x * rsqrt(mean(x^2) + eps) * norm_w) (input_layernorm / post_attention_layernorm of
+ * src/msa/model.py's decoder layer).  Partial sums are added in a fixed order: results are
+ * reproducible run to run. */
+#define MSA_EPI_PLAIN 0
+#define MSA_EPI_RESIDUAL 1
+#define MSA_EPI_SILU_MUL 2
+int msa_skinny_linear(const void* x, const void* w, const void* residual, const void* norm_w, float eps,
+                      int32_t epilogue, int32_t dtype, int32_t M, int32_t N, int32_t K, void* y,
+                      void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -119,17 +119,41 @@ class MemorySparseAttention(nn.Module):
         weights, then per-head RMSNorm + rotary (+ the dense copy of V) in one HIP kernel."""
         B, S, _ = hidden_states.shape
         Hq, Hkv, D = self.config.num_attention_heads, self.num_kv_heads, self.head_dim
-        if self._qkv_weight is None or self._qkv_weight.device != hidden_states.device:
-            self._qkv_weight = torch.cat([self.q_proj.weight, self.k_proj.weight, self.v_proj.weight], dim=0).contiguous()
-        dev = hidden_states.device
-        rows = min(self.config.max_position_embeddings, 32768)
-        key = (dev, rows, float(self.config.rope_theta))
-        if key not in _ROPE_TABLES:
-            _ROPE_TABLES[key] = ops.rope_tables(rows, D, self.config.rope_theta, device=dev)
-        qkv = F.linear(hidden_states.reshape(B * S, -1), self._qkv_weight)
+        w_qkv, tables = self._fused_weight(hidden_states.device), self._rope_tables(hidden_states.device)
+        qkv = F.linear(hidden_states.reshape(B * S, -1), w_qkv)
         q, k, v = ops.qk_norm_rope(qkv, Hq, Hkv, D, position_ids.reshape(-1).contiguous(), self.q_norm.weight,
-                                   self.k_norm.weight, self.q_norm.variance_epsilon, _ROPE_TABLES[key])
+                                   self.k_norm.weight, self.q_norm.variance_epsilon, tables)
         return q.view(B, S, Hq, D), k.view(B, S, Hkv, D), v.view(B, S, Hkv, D)
+
+    def _fused_weight(self, device):
+        if self._qkv_weight is None or self._qkv_weight.device != device:
+            self._qkv_weight = torch.cat([self.q_proj.weight, self.k_proj.weight, self.v_proj.weight], dim=0).contiguous()
+        return self._qkv_weight
+
+    def _rope_tables(self, device):
+        rows = min(self.config.max_position_embeddings, 32768)
+        key = (device, rows, float(self.config.rope_theta))
+        if key not in _ROPE_TABLES:
+            _ROPE_TABLES[key] = ops.rope_tables(rows, self.head_dim, self.config.rope_theta, device=device)
+        return _ROPE_TABLES[key]
+
+    def decode_rows(self, residual, norm_weight, eps, position_ids, cache):
+        """The decode step of :meth:`_generate` on the residual stream ``[B, hidden]`` (B <= 16, bf16) with the
+        layer's dense parts on the weight-streaming kernel: RMSNorm folded into the fused q/k/v projection, and
+        the residual add folded into the output projection.  Returns the new residual stream."""
+        B = residual.shape[0]
+        Hq, Hkv, D = self.config.num_attention_heads, self.num_kv_heads, self.head_dim
+        ck = cache.cache_kwargs[self.layer_idx]
+        if "compacked_key_cache" not in ck:
+            raise ValueError("compact KV cache not found: did prefill stage 2 run?")
+        qkv = ops.skinny_linear(residual, self._fused_weight(residual.device), norm_weight=norm_weight, eps=eps)
+        q, k, v = ops.qk_norm_rope(qkv, Hq, Hkv, D, position_ids.reshape(-1), self.q_norm.weight, self.k_norm.weight,
+                                   self.q_norm.variance_epsilon, self._rope_tables(residual.device))
+        kc, vc, kv_len = ck["compacked_key_cache"], ck["compacked_value_cache"], ck["kv_lengths"]
+        ops.cache_append(k.view(B, Hkv, D), v.view(B, Hkv, D), kc, vc, kv_len)
+        out = ops.sparse_attn(q.view(B, Hq, D), kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), ck["kv_offsets"], kv_len,
+                              ck["kv_capacity"], scale=self.scaling, causal=True)
+        return ops.skinny_linear(out.view(B, Hq * D), self.o_proj.weight, residual=residual)
 
     def forward_with_kvcache_for_batch_parrallel(self, hidden_states, doc_ids, attention_mask=None,
                                                  position_embeddings=None, past_key_value=None, position_ids=None,

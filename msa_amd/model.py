@@ -25,6 +25,16 @@ class MLP(nn.Module):
         self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=False)
 
         self._gate_up_weight = None
+        self._gate_up_interleaved = None
+
+    def decode_rows(self, residual, norm_weight, eps):
+        """``residual + down(silu(gate(n)) * up(n))`` with ``n = rmsnorm(residual)`` for up to 16 bf16 rows:
+        two weight-streaming launches, the norm folded into the first, silu-mul into its epilogue, the residual
+        add into the second."""
+        if self._gate_up_interleaved is None or self._gate_up_interleaved.device != residual.device:
+            self._gate_up_interleaved = ops.interleave_gate_up(self.gate_proj.weight, self.up_proj.weight)
+        act = ops.skinny_linear(residual, self._gate_up_interleaved, silu_mul=True, norm_weight=norm_weight, eps=eps)
+        return ops.skinny_linear(act, self.down_proj.weight, residual=residual)
 
     def forward(self, x):
         if x.is_cuda and x.dtype in (torch.bfloat16, torch.float32):
@@ -43,9 +53,14 @@ class MSADecoderLayer(nn.Module):
         self.post_attention_layernorm = RMSNorm(config.hidden_size, config.rms_norm_eps)
 
     def forward(self, hidden_states, doc_ids, attention_mask, position_embeddings, past_key_value, position_ids=None):
+        n1, n2 = self.input_layernorm, self.post_attention_layernorm
+        if self._decode_rows_ok(hidden_states, past_key_value, position_ids):
+            B = hidden_states.shape[0]
+            h = self.self_attn.decode_rows(hidden_states.view(B, -1), n1.weight, n1.variance_epsilon, position_ids,
+                                           past_key_value)
+            return self.mlp.decode_rows(h, n2.weight, n2.variance_epsilon).view(B, 1, -1)
         if hidden_states.is_cuda and hidden_states.dtype in (torch.bfloat16, torch.float32):
             # HIP glue: norm kernels with the residual add folded in; hidden_states is updated in place
-            n1, n2 = self.input_layernorm, self.post_attention_layernorm
             h, _ = self.self_attn(ops.rmsnorm(hidden_states, n1.weight, n1.variance_epsilon), doc_ids, attention_mask,
                                   position_embeddings, past_key_value, position_ids=position_ids)
             x = ops.rmsnorm(h.contiguous(), n2.weight, n2.variance_epsilon, residual=hidden_states)
@@ -56,6 +71,21 @@ class MSADecoderLayer(nn.Module):
         return hidden_states + self.mlp(self.post_attention_layernorm(hidden_states))
 
 
+    def _decode_rows_ok(self, hidden_states, cache, position_ids) -> bool:
+        """One new token for at most 16 samples, bf16 on the GPU, no projection biases, hidden sizes the
+        weight-streaming kernel takes: the decode step runs on it end to end."""
+        if not (hidden_states.is_cuda and hidden_states.dtype == torch.bfloat16 and position_ids is not None):
+            return False
+        B, S, H = hidden_states.shape
+        if S != 1 or B > ops.SKINNY_MAX_ROWS or cache is None or not hidden_states.is_contiguous():
+            return False
+        a = self.self_attn
+        if cache.cache_kwargs[a.layer_idx].get("stage") != "generate" or a.q_proj.bias is not None:
+            return False
+        inter = self.mlp.gate_proj.weight.shape[0]
+        return H % 128 == 0 and inter % 128 == 0 and (a.config.num_attention_heads * a.head_dim) % 128 == 0
+
+
 class MSAModel(nn.Module):
     def __init__(self, config: MSAConfig):
         super().__init__()
@@ -64,14 +94,16 @@ class MSAModel(nn.Module):
         self.layers = nn.ModuleList(MSADecoderLayer(config, i) for i in range(config.num_hidden_layers))
         self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps)
 
-    def forward(self, input_ids, attention_mask, position_ids, past_key_values, doc_ids):
+    def forward(self, input_ids, attention_mask, position_ids, past_key_values, doc_ids, final_norm: bool = True):
         h = self.embed_tokens(input_ids)
         if past_key_values is not None and attention_mask is not None and input_ids.shape[1] > 1:
             past_key_values.meta["q_lens_host"] = attention_mask.sum(dim=1).tolist()   # one sync per forward, not per layer
         if h.is_cuda:
             for layer in self.layers:
                 h = layer(h, doc_ids, attention_mask, None, past_key_values, position_ids=position_ids)
-            return ops.rmsnorm(h, self.norm.weight, self.norm.variance_epsilon)
+            if final_norm:
+                return ops.rmsnorm(h, self.norm.weight, self.norm.variance_epsilon)
+            return h
         pe = rotary_embedding(position_ids, self.config.head_dim, self.config.rope_theta, h.dtype)
         for layer in self.layers:
             h = layer(h, doc_ids, attention_mask, pe, past_key_values)
@@ -148,10 +180,18 @@ class MSAForCausalLM(nn.Module):
         out_buf[:, :1] = tok
         col = torch.ones((B, 1), dtype=torch.long, device=dev)
 
+        fold_head = (dev.type == "cuda" and self.lm_head.weight.dtype == torch.bfloat16 and B <= ops.SKINNY_MAX_ROWS
+                     and cfg.hidden_size % 128 == 0 and self.lm_head.bias is None)
+
         def step():
             # everything is in-place on fixed buffers so the same launches can be replayed as a graph
-            h = self.model(tok_buf, ones, pos_buf, cache, gen_ids)
-            new_tok = self.lm_head(h).argmax(-1)
+            if fold_head:                          # final norm folded into the weight-streaming LM head
+                h = self.model(tok_buf, ones, pos_buf, cache, gen_ids, final_norm=False)
+                logits = ops.skinny_linear(h.view(B, -1), self.lm_head.weight, norm_weight=self.model.norm.weight,
+                                           eps=self.model.norm.variance_epsilon).view(B, 1, -1)
+            else:
+                logits = self.lm_head(self.model(tok_buf, ones, pos_buf, cache, gen_ids))
+            new_tok = logits.argmax(-1)
             tok_buf.copy_(new_tok)
             pos_buf.add_(1)
             out_buf.scatter_(1, col, new_tok)

@@ -344,3 +344,39 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     check(_lib.load().msa_silu_mul(ptr(gate_up), dtype_code(gate_up.dtype), gate_up.numel() // (2 * I), I, ptr(out),
                                    _stream()), "msa_silu_mul")
     return out
+
+
+SKINNY_MAX_ROWS = 16
+
+
+def interleave_gate_up(gate_w: torch.Tensor, up_w: torch.Tensor) -> torch.Tensor:
+    """``[2 I, K]`` weight with alternating 16-row groups of gate and up rows: the layout the silu-mul epilogue
+    of ``skinny_linear`` expects (``I`` a multiple of 16)."""
+    I, K = gate_w.shape
+    if I % 16 or up_w.shape != gate_w.shape:
+        raise ValueError("gate / up weights must be [I, K] with I a multiple of 16")
+    return torch.stack([gate_w.view(I // 16, 16, K), up_w.view(I // 16, 16, K)], dim=1).reshape(2 * I, K).contiguous()
+
+
+def skinny_linear(x: torch.Tensor, w: torch.Tensor, residual: Optional[torch.Tensor] = None,
+                  silu_mul: bool = False, norm_weight: Optional[torch.Tensor] = None, eps: float = 1e-6) -> torch.Tensor:
+    """``x @ w.T`` for up to 16 rows of bf16 ``x [M, K]`` against ``w [N, K]``, streaming ``w`` once.
+    ``residual [M, N]`` is added to the bf16-rounded product; ``silu_mul`` takes ``w`` from ``interleave_gate_up``
+    and returns ``silu(gate) * up`` of width ``N / 2``; ``norm_weight [K]`` applies RMSNorm to ``x`` first."""
+    _need_cuda(x, w)
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1] or not x.is_contiguous() or not w.is_contiguous():
+        raise ValueError("skinny_linear: x [M, K] and w [N, K], both contiguous")
+    if residual is not None and silu_mul:
+        raise ValueError("skinny_linear: residual and silu_mul are exclusive")
+    M, K = x.shape
+    N = w.shape[0]
+    out = torch.empty((M, N // 2 if silu_mul else N), dtype=x.dtype, device=x.device)
+    if residual is not None and (residual.shape != out.shape or not residual.is_contiguous() or residual.dtype != x.dtype):
+        raise ValueError("skinny_linear: residual must be a contiguous [M, N] tensor of x's dtype")
+    epi = 2 if silu_mul else (1 if residual is not None else 0)
+    if norm_weight is not None and (norm_weight.shape != (K,) or norm_weight.dtype != x.dtype or not norm_weight.is_contiguous()):
+        raise ValueError("skinny_linear: norm_weight must be a contiguous [K] tensor of x's dtype")
+    check(_lib.load().msa_skinny_linear(ptr(x), ptr(w), ptr(residual) if residual is not None else None,
+                                        ptr(norm_weight) if norm_weight is not None else None, float(eps), epi,
+                                        dtype_code(x.dtype), M, N, K, ptr(out), _stream()), "msa_skinny_linear")
+    return out

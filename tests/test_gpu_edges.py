@@ -132,3 +132,58 @@ def test_error_codes(ops):
         t = ops.chunk_table([300], 64)
         x = _randn((300, 8, 128), 353, torch.bfloat16).cuda()
         ops.pool_chunks(x, None, None, t, rope=ops.rope_tables(128, 128, 1e4))
+
+
+# ---------------------------------------------------------------------------------------------
+# weight-streaming linear layer of the decode step
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("M,N,K", [(1, 48, 128), (5, 500, 256), (16, 2560, 4096), (16, 6144, 2560), (7, 2560, 9728),
+                                   (16, 20, 384)])
+def test_skinny_linear_plain_and_residual(ops, M, N, K):
+    say(f"skinny_linear M={M} N={N} K={K}")
+    g = torch.Generator().manual_seed(M * 1000 + N + K)
+    x = torch.randn((M, K), generator=g).bfloat16()
+    w = (torch.randn((N, K), generator=g) * K ** -0.5).bfloat16()
+    res = torch.randn((M, N), generator=g).bfloat16()
+    want = x.double() @ w.double().T
+    got = ops.skinny_linear(x.cuda(), w.cuda()).cpu()
+    assert got.shape == (M, N) and cf.rel_err(got, want) < 1e-2
+    got_r = ops.skinny_linear(x.cuda(), w.cuda(), residual=res.cuda()).cpu()
+    assert cf.rel_err(got_r, want.bfloat16().double() + res.double()) < 1e-2
+    # a fixed summation order: the same call twice gives the same bits
+    assert torch.equal(ops.skinny_linear(x.cuda(), w.cuda()).cpu(), got)
+
+
+@pytest.mark.parametrize("M,I,K", [(16, 9728, 2560), (3, 64, 256), (16, 528, 1024)])
+def test_skinny_linear_norm_and_silu_mul(ops, M, I, K):
+    say(f"skinny_linear norm + silu-mul M={M} I={I} K={K}")
+    g = torch.Generator().manual_seed(I + K)
+    x = (torch.randn((M, K), generator=g) * 3).bfloat16()
+    gate = (torch.randn((I, K), generator=g) * K ** -0.5).bfloat16()
+    up = (torch.randn((I, K), generator=g) * K ** -0.5).bfloat16()
+    nw = (1 + 0.1 * torch.randn((K,), generator=g)).bfloat16()
+    eps = 1e-6
+    xd = x.double()
+    normed = (xd * torch.rsqrt((xd * xd).mean(-1, keepdim=True) + eps) * nw.double()).bfloat16().double()
+    # RMSNorm folded in, plain epilogue
+    want = normed @ gate.double().T
+    got = ops.skinny_linear(x.cuda(), gate.cuda(), norm_weight=nw.cuda(), eps=eps).cpu()
+    assert cf.rel_err(got, want) < 1e-2
+    # and with the silu-mul epilogue over interleaved gate / up row groups
+    wi = ops.interleave_gate_up(gate.cuda(), up.cuda())
+    assert wi.shape == (2 * I, K) and torch.equal(wi[:16].cpu(), gate[:16]) and torch.equal(wi[16:32].cpu(), up[:16])
+    a, b = (normed @ gate.double().T).bfloat16().double(), (normed @ up.double().T).bfloat16().double()
+    got = ops.skinny_linear(x.cuda(), wi, silu_mul=True, norm_weight=nw.cuda(), eps=eps).cpu()
+    assert got.shape == (M, I) and cf.rel_err(got, torch.nn.functional.silu(a) * b) < 1.5e-2
+
+
+def test_skinny_linear_errors(ops):
+    say("skinny_linear argument checks")
+    from msa_amd import _lib
+    x, w = torch.zeros((17, 128), dtype=torch.bfloat16).cuda(), torch.zeros((16, 128), dtype=torch.bfloat16).cuda()
+    with pytest.raises(_lib.MsaError, match="rows"):
+        ops.skinny_linear(x, w)
+    with pytest.raises(_lib.MsaError, match="multiple of 128"):
+        ops.skinny_linear(torch.zeros((2, 96), dtype=torch.bfloat16).cuda(), torch.zeros((16, 96), dtype=torch.bfloat16).cuda())
+    with pytest.raises(_lib.MsaError, match="bf16 only"):
+        ops.skinny_linear(torch.zeros((2, 128)).cuda(), torch.zeros((16, 128)).cuda())

@@ -258,3 +258,40 @@ def test_model_greedy_generation_runs_and_is_deterministic(env):
     assert len(rec) == 2 and all(len(set(r["topk_doc_ids"])) == TOPK for r in rec)
     assert "recall_topk" not in c1.cache_kwargs[0]                           # layer 0 is not a router layer
     assert c1.cache_kwargs[1]["kv_lengths"].cpu().tolist()[0] > c1.cache_kwargs[0]["kv_lengths"].cpu().tolist()[0]
+
+
+def test_decode_rows_path_matches_generic_layer_path(env):
+    """The weight-streaming decode step (norms, silu-mul and residual adds folded into the projections) against
+    the same decoder layers run through the separate norm / projection / activation kernels."""
+    say("model: weight-streaming decode step vs generic layer path")
+    pf, svc_mod, M = env["prefill"], env["svc"], env["model"]
+    model = M.MSAForCausalLM(env["cfg"]).init_random(0.05, seed=4).to(torch.bfloat16).cuda().eval()
+    docs = _docs(env, [20, 33, 9, 41], first_id=0)
+    service = svc_mod.MSAService(0, env["config"].GenerateConfig(devices=[0]),
+                                 env["config"].ModelConfig(doc_top_k=TOPK, pooling_kernel_size=P, router_layer_idx="1"),
+                                 env["config"].MemoryConfig(pooling_kernel_size=P), env["cfg"])
+    service.begin(docs)
+    for blk in pf.split_docs(docs, 12):
+        service.add_block(M.encode_block(model, pf.prepare_block_inputs(blk, HEAD_IDS, P), "cuda"))
+    service.finish()
+    service.setup_memory_client(model)
+    ids = torch.tensor([[5, 6, 7, 8, 9, 10], [0, 0, 11, 12, 13, 14]]).cuda()
+    mask = torch.tensor([[1] * 6, [0, 0, 1, 1, 1, 1]]).cuda()
+    _, cache = model.generate_greedy(ids, mask, torch.zeros_like(ids), 1)
+    for i in range(env["cfg"].num_hidden_layers):
+        cache.cache_kwargs[i]["stage"] = "generate"
+    layer = model.model.layers[1]
+    h = (torch.randn((2, 1, HID), generator=torch.Generator().manual_seed(9)) * 2).bfloat16().cuda()
+    pos = torch.tensor([[30], [28]]).cuda()
+    gen_ids = torch.full((2, 1), -1).cuda()
+    ones = torch.ones((2, 1), dtype=torch.long).cuda()
+    lens0 = cache.cache_kwargs[1]["kv_lengths"].clone()
+    assert layer._decode_rows_ok(h, cache, pos)
+    with torch.no_grad():
+        fast = layer(h.clone(), gen_ids, ones, None, cache, position_ids=pos)
+        cache.cache_kwargs[1]["kv_lengths"].copy_(lens0)                     # same cache row for the second run
+        layer._decode_rows_ok = lambda *a: False
+        slow = layer(h.clone(), gen_ids, ones, None, cache, position_ids=pos)
+        del layer._decode_rows_ok
+    assert fast.shape == slow.shape == (2, 1, HID)
+    assert cf.rel_err(fast.cpu(), slow.double().cpu()) < 1e-2

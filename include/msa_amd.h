@@ -196,6 +196,16 @@ int msa_qk_norm_rope(const void* q, const void* k, const void* v, int64_t q_row_
                      const void* q_norm_w, const void* k_norm_w, float eps, const float* rope_cos,
                      const float* rope_sin, int32_t rope_rows, int32_t dtype, int64_t N, int32_t Hq,
                      int32_t Hkv, int32_t D, void* q_out, void* k_out, void* v_out, void* stream);
+/* msa_qk_norm_rope for a decode step (one new token per sample, N = B) fused with msa_cache_append: the
+ * normalised, rotated k row and the v row of sample b are written to kcache / vcache [b][kv_len[b]] and
+ * kv_len[b] is incremented (src/msa/memory_sparse_attention.py:129-133 followed by the cache update at
+ * :372-379).  A full cache (kv_len[b] == Lcap) drops the row. */
+int msa_qk_norm_rope_append(const void* q, const void* k, const void* v, int64_t q_row_stride,
+                            int64_t k_row_stride, int64_t v_row_stride, const int64_t* positions,
+                            const void* q_norm_w, const void* k_norm_w, float eps,
+                            const float* rope_cos, const float* rope_sin, int32_t rope_rows,
+                            int32_t dtype, int32_t B, int32_t Hq, int32_t Hkv, int32_t D, void* q_out,
+                            void* kcache, void* vcache, int32_t Lcap, int32_t* kv_len, void* stream);
 int msa_rmsnorm(const void* x, void* residual, const void* weight, int32_t dtype, int64_t N,
                 int32_t H, float eps, void* out, void* stream);
 int msa_silu_mul(const void* gate_up, int32_t dtype, int64_t N, int32_t I, void* out, void* stream);

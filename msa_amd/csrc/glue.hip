@@ -52,22 +52,34 @@ __global__ void qk_norm_rope_kernel(const T* __restrict__ q, const T* __restrict
                                     const int64_t* __restrict__ pos, const T* __restrict__ qw,
                                     const T* __restrict__ kw, float eps, const float* __restrict__ cos_t,
                                     const float* __restrict__ sin_t, int32_t rope_rows, int32_t Hq, int32_t Hkv,
-                                    T* __restrict__ q_out, T* __restrict__ k_out, T* __restrict__ v_out) {
+                                    T* __restrict__ q_out, T* __restrict__ k_out, T* __restrict__ v_out,
+                                    int32_t Lcap, int32_t* __restrict__ kv_len) {
   const int64_t n = blockIdx.x;
   const int head = threadIdx.x >> 4, j = threadIdx.x & 15;
+  // Append mode (kv_len given; token n is the one new token of sample n): k / v rows go straight into the
+  // sample's cache [n][kv_len[n]] and the length is bumped; a full cache drops the row.
+  int64_t kv_row = n;
+  bool keep_kv = true;
+  if (kv_len != nullptr) {
+    const int at = kv_len[n];
+    __syncthreads();                     // every lane has read the old length before lane 0 bumps it
+    keep_kv = at < Lcap;
+    kv_row = n * Lcap + at;
+    if (threadIdx.x == 0 && keep_kv) kv_len[n] = at + 1;
+  }
   if (head >= Hq + Hkv) {                       // optional V heads: a straight copy into a dense row
     const int hv = head - Hq - Hkv;
-    if (v != nullptr && hv < Hkv) {
+    if (v != nullptr && hv < Hkv && keep_kv) {
       float t[8];
       load8g<T>(v + n * v_stride + hv * kHeadDim + 8 * j, t);
-      store8g<T>(v_out + (n * Hkv + hv) * kHeadDim + 8 * j, t);
+      store8g<T>(v_out + (kv_row * Hkv + hv) * kHeadDim + 8 * j, t);
     }
     return;
   }
   const bool is_q = head < Hq;
   const int h = is_q ? head : head - Hq;
   const T* src = is_q ? q + n * q_stride + h * kHeadDim : k + n * k_stride + h * kHeadDim;
-  T* dst = is_q ? q_out + (n * Hq + h) * kHeadDim : k_out + (n * Hkv + h) * kHeadDim;
+  T* dst = is_q ? q_out + (n * Hq + h) * kHeadDim : k_out + (kv_row * Hkv + h) * kHeadDim;
   float x[8], w[8];
   load8g<T>(src + 8 * j, x);
   load8g<T>((is_q ? qw : kw) + 8 * j, w);
@@ -85,7 +97,7 @@ __global__ void qk_norm_rope_kernel(const T* __restrict__ q, const T* __restrict
     const float c = cos_t[p * 64 + f + i], s = sin_t[p * 64 + f + i];
     out[i] = j < 8 ? y * c - other * s : y * c + other * s;
   }
-  store8g<T>(dst + 8 * j, out);
+  if (is_q || keep_kv) store8g<T>(dst + 8 * j, out);
 }
 
 // One workgroup per row.  With `residual`: residual <- residual + x (stored in T), then normalised.
@@ -138,37 +150,59 @@ __global__ void silu_mul_kernel(const T* __restrict__ gate_up, int64_t N, int32_
 
 }  // namespace
 
-extern "C" int msa_qk_norm_rope(const void* q, const void* k, const void* v, int64_t q_row_stride,
-                                int64_t k_row_stride, int64_t v_row_stride, const int64_t* positions, const void* q_norm_w, const void* k_norm_w, float eps,
-                                const float* rope_cos, const float* rope_sin, int32_t rope_rows, int32_t dtype,
-                                int64_t N, int32_t Hq, int32_t Hkv, int32_t D, void* q_out, void* k_out,
-                                void* v_out, void* stream) {
+static int qk_norm_rope_launch(const char* who, const void* q, const void* k, const void* v, int64_t q_row_stride,
+                               int64_t k_row_stride, int64_t v_row_stride, const int64_t* positions,
+                               const void* q_norm_w, const void* k_norm_w, float eps, const float* rope_cos,
+                               const float* rope_sin, int32_t rope_rows, int32_t dtype, int64_t N, int32_t Hq,
+                               int32_t Hkv, int32_t D, void* q_out, void* k_out, void* v_out, int32_t Lcap,
+                               int32_t* kv_len, void* stream) {
   MSA_REQUIRE(q && k && positions && q_norm_w && k_norm_w && rope_cos && rope_sin && q_out && k_out,
-              "msa_qk_norm_rope: null pointer");
-  MSA_REQUIRE(D == kHeadDim, "msa_qk_norm_rope: head dim %d unsupported (need %d)", D, kHeadDim);
-  MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "msa_qk_norm_rope: bad dtype %d", dtype);
-  MSA_REQUIRE(N > 0 && N < (int64_t)1 << 31, "msa_qk_norm_rope: N=%lld out of range", (long long)N);
-  MSA_REQUIRE((v == nullptr) == (v_out == nullptr), "msa_qk_norm_rope: v and v_out go together");
+              "%s: null pointer", who);
+  MSA_REQUIRE(D == kHeadDim, "%s: head dim %d unsupported (need %d)", who, D, kHeadDim);
+  MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "%s: bad dtype %d", who, dtype);
+  MSA_REQUIRE(N > 0 && N < (int64_t)1 << 31, "%s: N=%lld out of range", who, (long long)N);
+  MSA_REQUIRE((v == nullptr) == (v_out == nullptr), "%s: v and v_out go together", who);
   const int heads = Hq + Hkv + (v ? Hkv : 0);
-  MSA_REQUIRE(Hq > 0 && Hkv > 0 && heads * 16 <= 1024, "msa_qk_norm_rope: Hq=%d Hkv=%d unsupported", Hq, Hkv);
-  MSA_REQUIRE(v == nullptr || (v_row_stride >= (int64_t)Hkv * D && v_row_stride % 8 == 0),
-              "msa_qk_norm_rope: bad V row stride");
-  MSA_REQUIRE(rope_rows > 0, "msa_qk_norm_rope: empty rotary table");
+  MSA_REQUIRE(Hq > 0 && Hkv > 0 && heads * 16 <= 1024, "%s: Hq=%d Hkv=%d unsupported", who, Hq, Hkv);
+  MSA_REQUIRE(v == nullptr || (v_row_stride >= (int64_t)Hkv * D && v_row_stride % 8 == 0), "%s: bad V row stride", who);
+  MSA_REQUIRE(rope_rows > 0, "%s: empty rotary table", who);
   MSA_REQUIRE(q_row_stride >= (int64_t)Hq * D && k_row_stride >= (int64_t)Hkv * D && q_row_stride % 8 == 0 &&
-                  k_row_stride % 8 == 0, "msa_qk_norm_rope: bad row strides");
+                  k_row_stride % 8 == 0, "%s: bad row strides", who);
   const int threads = (heads * 16 + 63) / 64 * 64;
   if (dtype == MSA_BF16)
     qk_norm_rope_kernel<bf16_t><<<(unsigned)N, threads, 0, as_stream(stream)>>>(
         (const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v, q_row_stride, k_row_stride, v_row_stride, positions,
         (const bf16_t*)q_norm_w, (const bf16_t*)k_norm_w, eps, rope_cos, rope_sin, rope_rows, Hq, Hkv,
-        (bf16_t*)q_out, (bf16_t*)k_out, (bf16_t*)v_out);
+        (bf16_t*)q_out, (bf16_t*)k_out, (bf16_t*)v_out, Lcap, kv_len);
   else
     qk_norm_rope_kernel<float><<<(unsigned)N, threads, 0, as_stream(stream)>>>(
         (const float*)q, (const float*)k, (const float*)v, q_row_stride, k_row_stride, v_row_stride, positions,
         (const float*)q_norm_w, (const float*)k_norm_w, eps, rope_cos, rope_sin, rope_rows, Hq, Hkv, (float*)q_out,
-        (float*)k_out, (float*)v_out);
+        (float*)k_out, (float*)v_out, Lcap, kv_len);
   MSA_LAUNCH_CHECK();
   return MSA_OK;
+}
+
+extern "C" int msa_qk_norm_rope(const void* q, const void* k, const void* v, int64_t q_row_stride,
+                                int64_t k_row_stride, int64_t v_row_stride, const int64_t* positions,
+                                const void* q_norm_w, const void* k_norm_w, float eps, const float* rope_cos,
+                                const float* rope_sin, int32_t rope_rows, int32_t dtype, int64_t N, int32_t Hq,
+                                int32_t Hkv, int32_t D, void* q_out, void* k_out, void* v_out, void* stream) {
+  return qk_norm_rope_launch("msa_qk_norm_rope", q, k, v, q_row_stride, k_row_stride, v_row_stride, positions, q_norm_w,
+                             k_norm_w, eps, rope_cos, rope_sin, rope_rows, dtype, N, Hq, Hkv, D, q_out, k_out, v_out, 0,
+                             nullptr, stream);
+}
+
+extern "C" int msa_qk_norm_rope_append(const void* q, const void* k, const void* v, int64_t q_row_stride,
+                                       int64_t k_row_stride, int64_t v_row_stride, const int64_t* positions,
+                                       const void* q_norm_w, const void* k_norm_w, float eps, const float* rope_cos,
+                                       const float* rope_sin, int32_t rope_rows, int32_t dtype, int32_t B, int32_t Hq,
+                                       int32_t Hkv, int32_t D, void* q_out, void* kcache, void* vcache, int32_t Lcap,
+                                       int32_t* kv_len, void* stream) {
+  MSA_REQUIRE(v && kcache && vcache && kv_len && Lcap > 0, "msa_qk_norm_rope_append: null cache pointer or Lcap <= 0");
+  return qk_norm_rope_launch("msa_qk_norm_rope_append", q, k, v, q_row_stride, k_row_stride, v_row_stride, positions,
+                             q_norm_w, k_norm_w, eps, rope_cos, rope_sin, rope_rows, dtype, B, Hq, Hkv, D, q_out, kcache,
+                             vcache, Lcap, kv_len, stream);
 }
 
 extern "C" int msa_rmsnorm(const void* x, void* residual, const void* weight, int32_t dtype, int64_t N, int32_t H,

@@ -147,10 +147,9 @@ class MemorySparseAttention(nn.Module):
         if "compacked_key_cache" not in ck:
             raise ValueError("compact KV cache not found: did prefill stage 2 run?")
         qkv = ops.skinny_linear(residual, self._fused_weight(residual.device), norm_weight=norm_weight, eps=eps)
-        q, k, v = ops.qk_norm_rope(qkv, Hq, Hkv, D, position_ids.reshape(-1), self.q_norm.weight, self.k_norm.weight,
-                                   self.q_norm.variance_epsilon, self._rope_tables(residual.device))
         kc, vc, kv_len = ck["compacked_key_cache"], ck["compacked_value_cache"], ck["kv_lengths"]
-        ops.cache_append(k.view(B, Hkv, D), v.view(B, Hkv, D), kc, vc, kv_len)
+        q = ops.qk_norm_rope_append(qkv, Hq, Hkv, D, position_ids.reshape(-1), self.q_norm.weight, self.k_norm.weight,
+                                    self.q_norm.variance_epsilon, self._rope_tables(residual.device), kc, vc, kv_len)
         out = ops.sparse_attn(q.view(B, Hq, D), kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), ck["kv_offsets"], kv_len,
                               ck["kv_capacity"], scale=self.scaling, causal=True)
         return ops.skinny_linear(out.view(B, Hq * D), self.o_proj.weight, residual=residual)

@@ -325,6 +325,30 @@ def qk_norm_rope(qkv: torch.Tensor, Hq: int, Hkv: int, D: int, positions: torch.
     return q, k, v
 
 
+def qk_norm_rope_append(qkv: torch.Tensor, Hq: int, Hkv: int, D: int, positions: torch.Tensor, q_norm_w, k_norm_w,
+                        eps: float, rope: Tuple[torch.Tensor, torch.Tensor], kcache: torch.Tensor, vcache: torch.Tensor,
+                        kv_len: torch.Tensor) -> torch.Tensor:
+    """Decode-step form of :func:`qk_norm_rope` (one new token per sample): returns ``q [B, Hq, D]`` and writes
+    the k / v rows into ``kcache / vcache [B, Lcap, Hkv, D]`` at ``kv_len[b]``, which is incremented in place."""
+    _need_cuda(qkv, positions, q_norm_w, k_norm_w, rope[0], rope[1], kcache, vcache, kv_len)
+    B, W = qkv.shape
+    if W != (Hq + 2 * Hkv) * D or positions.dtype != torch.int64 or positions.numel() != B:
+        raise ValueError("qkv must be [B, (Hq + 2 Hkv) D] and positions int64 [B]")
+    if (kcache.shape != vcache.shape or kcache.dim() != 4 or kcache.shape[0] != B or tuple(kcache.shape[2:]) != (Hkv, D)
+            or kcache.dtype != qkv.dtype or not (kcache.is_contiguous() and vcache.is_contiguous())):
+        raise ValueError("kcache / vcache must be contiguous [B, Lcap, Hkv, D] of qkv's dtype")
+    if kv_len.dtype != torch.int32 or kv_len.numel() != B:
+        raise ValueError("kv_len must be int32 [B]")
+    q = torch.empty((B, Hq, D), dtype=qkv.dtype, device=qkv.device)
+    es, base = qkv.element_size(), qkv.data_ptr()
+    check(_lib.load().msa_qk_norm_rope_append(base, base + Hq * D * es, base + (Hq + Hkv) * D * es, W, W, W,
+                                              ptr(positions), ptr(q_norm_w), ptr(k_norm_w), eps, ptr(rope[0]),
+                                              ptr(rope[1]), rope[0].shape[0], dtype_code(qkv.dtype), B, Hq, Hkv, D,
+                                              ptr(q), ptr(kcache), ptr(vcache), kcache.shape[1], ptr(kv_len), _stream()),
+          "msa_qk_norm_rope_append")
+    return q
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Row RMSNorm of ``x [..., H]``; with ``residual`` (same shape) does ``residual += x`` in place first
     and normalises the sum."""

@@ -187,3 +187,24 @@ def test_skinny_linear_errors(ops):
         ops.skinny_linear(torch.zeros((2, 96), dtype=torch.bfloat16).cuda(), torch.zeros((16, 96), dtype=torch.bfloat16).cuda())
     with pytest.raises(_lib.MsaError, match="bf16 only"):
         ops.skinny_linear(torch.zeros((2, 128)).cuda(), torch.zeros((16, 128)).cuda())
+
+
+def test_qk_norm_rope_append_equals_separate_kernels(ops):
+    say("qk_norm_rope_append vs qk_norm_rope + cache_append")
+    B, Hq, Hkv, D, Lcap = 5, 8, 2, 128, 12
+    g = torch.Generator().manual_seed(11)
+    qkv = torch.randn((B, (Hq + 2 * Hkv) * D), generator=g).bfloat16().cuda()
+    pos = torch.tensor([3, 700, 0, 41, 9], dtype=torch.int64).cuda()
+    qw, kw = (1 + 0.1 * torch.randn(D, generator=g)).bfloat16().cuda(), (1 + 0.1 * torch.randn(D, generator=g)).bfloat16().cuda()
+    rope = ops.rope_tables(1024, D, 1e6, device="cuda")
+    lens = torch.tensor([0, 11, 12, 5, 7], dtype=torch.int32)                 # sample 2 is full: its row is dropped
+    kc0 = torch.randn((B, Lcap, Hkv, D), generator=g).bfloat16().cuda()
+    vc0 = torch.randn((B, Lcap, Hkv, D), generator=g).bfloat16().cuda()
+    q, k, v = ops.qk_norm_rope(qkv, Hq, Hkv, D, pos, qw, kw, 1e-6, rope)
+    kc1, vc1, l1 = kc0.clone(), vc0.clone(), lens.clone().cuda()
+    ops.cache_append(k, v, kc1, vc1, l1)
+    kc2, vc2, l2 = kc0.clone(), vc0.clone(), lens.clone().cuda()
+    q2 = ops.qk_norm_rope_append(qkv, Hq, Hkv, D, pos, qw, kw, 1e-6, rope, kc2, vc2, l2)
+    assert torch.equal(q2, q) and torch.equal(kc2, kc1) and torch.equal(vc2, vc1)
+    assert l2.cpu().tolist() == l1.cpu().tolist() == [1, 12, 12, 6, 8]
+    assert torch.equal(kc2[2], kc0[2]) and not torch.equal(kc2[0, 0], kc0[0, 0])

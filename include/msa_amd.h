@@ -159,6 +159,14 @@ int msa_cache_append(const void* k_new, const void* v_new, int32_t B, int32_t Hk
                      int32_t dtype, void* kcache, void* vcache, int32_t Lcap, int32_t* kv_len,
                      void* stream);
 
+/* Ragged form for a block of new tokens per sample (the source-context injection of the Memory-Interleave
+ * loop, src/msa/generate.py:190-259, which reaches the same torch.cat at memory_sparse_attention.py:372-373 with
+ * S > 1): sample b appends rows cu_new[b] .. cu_new[b+1] of k_new / v_new [total_new, Hkv, D] (device int32
+ * prefix sums, at most max_new rows per sample) at kv_len[b]; rows that do not fit in Lcap are dropped. */
+int msa_cache_append_rows(const void* k_new, const void* v_new, const int32_t* cu_new, int32_t max_new,
+                          int32_t B, int32_t Hkv, int32_t D, int32_t dtype, void* kcache, void* vcache,
+                          int32_t Lcap, int32_t* kv_len, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * GQA attention of ragged query rows over per-sample KV ranges.  Replaces repeat_kv + SDPA of the
  * decode step (src/msa/memory_sparse_attention.py:389-399) and, with several query rows per

@@ -166,7 +166,7 @@ class MemorySparseAttention(nn.Module):
             return self._stage1(hidden_states, doc_ids, attention_mask, q, k, v, past_key_value)
         if stage == "prefill_stage2":
             return self._stage2(hidden_states, doc_ids, attention_mask, q, k, v, past_key_value)
-        return self._generate(hidden_states, q, k, v, past_key_value)
+        return self._generate(hidden_states, q, k, v, past_key_value, attention_mask)
 
     # ------------------------------------------------------------------------------------------ stage 1
     def _stage1(self, hidden_states, doc_ids, attention_mask, q, k, v, cache):
@@ -265,17 +265,30 @@ class MemorySparseAttention(nn.Module):
         return self.o_proj(attn), None
 
     # ------------------------------------------------------------------------------------------ decode
-    def _generate(self, hidden_states, q, k, v, cache):
+    def _generate(self, hidden_states, q, k, v, cache, attention_mask=None):
         """One decode step over the compact cache, appended in place
-        (src/msa/memory_sparse_attention.py:361-405)."""
+        (src/msa/memory_sparse_attention.py:361-405).  With more than one token per sample (the source-context
+        block the Memory-Interleave loop injects between rounds, src/msa/generate.py:190-259, left-padded) the
+        valid tokens are appended as a ragged block and attend causally over ``[cache | block so far]``."""
         B, S, _ = hidden_states.shape
         ck = cache.cache_kwargs[self.layer_idx]
         if "compacked_key_cache" not in ck:
             raise ValueError("compact KV cache not found: did prefill stage 2 run?")
-        if S != 1:
-            raise ValueError("the decode step takes one new token per sample")
         kc, vc, kv_len = ck["compacked_key_cache"], ck["compacked_value_cache"], ck["kv_lengths"]
-        Hkv, D = self.num_kv_heads, self.head_dim
+        Hq, Hkv, D = self.config.num_attention_heads, self.num_kv_heads, self.head_dim
+        if S != 1:
+            valid = attention_mask == 1 if attention_mask is not None else torch.ones((B, S), dtype=torch.bool, device=q.device)
+            n_new = valid.sum(dim=1)
+            n_host = cache.meta.get("q_lens_host")
+            if n_host is None or len(n_host) != B:
+                n_host = n_new.tolist()
+            cu_new = F.pad(n_new.cumsum(0), (1, 0)).to(torch.int32)
+            ops.cache_append_rows(k[valid], v[valid], cu_new, max(n_host), kc, vc, kv_len)
+            rows = ops.sparse_attn(q[valid], kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), ck["kv_offsets"], kv_len,
+                                   ck["kv_capacity"], cu_q=cu_new, max_sq=max(n_host), scale=self.scaling, causal=True)
+            attn = torch.zeros((B, S, Hq * D), device=q.device, dtype=q.dtype)
+            attn[valid] = rows.view(-1, Hq * D)
+            return self.o_proj(attn), None
         # capacity is the caller's job (rows behind the context: decode_reserve); a full cache drops the
         # new row inside the kernel instead of writing out of bounds
         ops.cache_append(k[:, 0].contiguous(), v[:, 0].contiguous(), kc, vc, kv_len)

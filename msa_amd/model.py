@@ -221,6 +221,57 @@ class MSAForCausalLM(nn.Module):
         return out_buf, cache
 
 
+@torch.no_grad()
+def generate_interleaved(model: "MSAForCausalLM", input_ids, attention_mask, doc_ids, max_new_tokens: int, inject,
+                         top_k_docs: Optional[int] = None):
+    """Greedy decoding with Memory-Interleave rounds (the control flow of src/msa/generate.py:190-259 without the
+    tokenizer: text handling stays with the caller).  After every new token ``inject(step, tokens [B, step])`` may
+    return a list of ``B`` token-id lists; a non-empty list replaces the sample's just-generated token as the next
+    model input (the reference feeds the retrieved documents' text instead of the round-end marker), an empty one
+    lets the sample continue with its own token.  The lists are fed as one left-padded block whose positions
+    continue each sample's own, appended to the compact caches by the ragged path of the decode stage, and the
+    next token is read at the block's last position.  Returns ``(tokens [B, max_new_tokens], cache)``."""
+    cfg = model.config
+    B, S = input_ids.shape
+    dev = input_ids.device
+    k = cfg.msa_config.top_k_docs if top_k_docs is None else top_k_docs
+    cache = create_cache()
+    for i in range(cfg.num_hidden_layers):
+        cache.record_kwargs(i, {"stage": "prefill_stage2"})
+    n_valid = attention_mask.sum(dim=1).tolist()
+    pos = torch.tensor([query_position_ids(n, k, 3, S - n) for n in n_valid], dtype=torch.long, device=dev)
+    h = model.model(input_ids, attention_mask, pos, cache, doc_ids)
+    tok = model.lm_head(h[:, -1:]).argmax(-1)                 # [B, 1]
+    for i in range(cfg.num_hidden_layers):
+        cache.cache_kwargs[i]["stage"] = "generate"
+    last_pos = pos[:, -1].clone()                             # position of the last token each sample has fed
+    out = [tok]
+    for step in range(1, max_new_tokens):
+        blocks = inject(step, torch.cat(out, dim=1)) if inject is not None else None
+        blocks = [list(b) if b else [int(t)] for b, t in zip(blocks, tok[:, 0].tolist())] if blocks is not None else None
+        if blocks is None or all(len(b) == 1 for b in blocks):
+            ids = tok if blocks is None else torch.tensor(blocks, dtype=torch.long, device=dev)
+            p = (last_pos + 1).unsqueeze(1)
+            h = model.model(ids, torch.ones_like(ids), p, cache, torch.full_like(ids, -1))
+            last_pos += 1
+        else:
+            width = max(len(b) for b in blocks)
+            ids = torch.zeros((B, width), dtype=torch.long)
+            mask = torch.zeros((B, width), dtype=torch.long)
+            p = torch.zeros((B, width), dtype=torch.long)
+            for b, blk in enumerate(blocks):
+                n = len(blk)
+                ids[b, width - n:] = torch.tensor(blk)
+                mask[b, width - n:] = 1
+                first = int(last_pos[b]) + 1
+                p[b] = torch.tensor([first] * (width - n) + list(range(first, first + n)))   # padding repeats the first position
+            h = model.model(ids.to(dev), mask.to(dev), p.to(dev), cache, torch.zeros((B, width), dtype=torch.long, device=dev))
+            last_pos += torch.tensor([len(b) for b in blocks], device=dev)
+        tok = model.lm_head(h[:, -1:]).argmax(-1)
+        out.append(tok)
+    return torch.cat(out, dim=1), cache
+
+
 def encode_block(model: MSAForCausalLM, block_input, device) -> CustomDynamicCache:
     """Runs stage 1 over one packed block and returns the cache holding its pooled K / V / K_r
     (the inference half of src/prefill.py:248-305)."""

@@ -271,6 +271,18 @@ def cache_append(k_new, v_new, kcache, vcache, kv_len):
                                        ptr(vcache), Lcap, ptr(kv_len), _stream()), "msa_cache_append")
 
 
+def cache_append_rows(k_new, v_new, cu_new, max_new: int, kcache, vcache, kv_len):
+    """Ragged append: sample ``b`` gets rows ``cu_new[b]:cu_new[b+1]`` of ``k_new / v_new [total, Hkv, D]`` at
+    ``kv_len[b]``, which grows by that count (clamped to the capacity), in place."""
+    _need_cuda(k_new, v_new, cu_new, kcache, vcache, kv_len)
+    B, Lcap, Hkv, D = kcache.shape
+    if cu_new.dtype != torch.int32 or cu_new.numel() != B + 1 or k_new.shape[1:] != (Hkv, D) or k_new.shape != v_new.shape:
+        raise ValueError("cu_new int32 [B + 1]; k_new / v_new [total, Hkv, D]")
+    check(_lib.load().msa_cache_append_rows(ptr(k_new), ptr(v_new), ptr(cu_new), max_new, B, Hkv, D,
+                                            dtype_code(kcache.dtype), ptr(kcache), ptr(vcache), Lcap, ptr(kv_len),
+                                            _stream()), "msa_cache_append_rows")
+
+
 _attn_ws = {}
 FLASH_MIN_ROWS = 16     # bf16 query blocks at least this long go to the MFMA flash kernel
 

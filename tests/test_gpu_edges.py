@@ -208,3 +208,25 @@ def test_qk_norm_rope_append_equals_separate_kernels(ops):
     assert torch.equal(q2, q) and torch.equal(kc2, kc1) and torch.equal(vc2, vc1)
     assert l2.cpu().tolist() == l1.cpu().tolist() == [1, 12, 12, 6, 8]
     assert torch.equal(kc2[2], kc0[2]) and not torch.equal(kc2[0, 0], kc0[0, 0])
+
+
+def test_cache_append_rows_ragged_and_clamped(ops):
+    say("cache_append_rows: ragged blocks, empty block, capacity clamp")
+    B, Lcap, Hkv, D = 4, 10, 2, 128
+    g = torch.Generator().manual_seed(3)
+    kc0, vc0 = torch.randn((B, Lcap, Hkv, D), generator=g), torch.randn((B, Lcap, Hkv, D), generator=g)
+    n_new = [3, 0, 5, 1]
+    lens = [2, 4, 7, 10]                                       # sample 2 has room for 3 of its 5 rows, sample 3 for none
+    kn, vn = torch.randn((sum(n_new), Hkv, D), generator=g), torch.randn((sum(n_new), Hkv, D), generator=g)
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(n_new)]), dtype=torch.int32)
+    for dtype in (torch.float32, torch.bfloat16):
+        kc, vc = kc0.to(dtype).cuda(), vc0.to(dtype).cuda()
+        kv_len = torch.tensor(lens, dtype=torch.int32).cuda()
+        ops.cache_append_rows(kn.to(dtype).cuda(), vn.to(dtype).cuda(), cu.cuda(), max(n_new), kc, vc, kv_len)
+        want_k, want_v = kc0.to(dtype).clone(), vc0.to(dtype).clone()
+        for b in range(B):
+            fit = min(n_new[b], Lcap - lens[b])
+            want_k[b, lens[b]:lens[b] + fit] = kn.to(dtype)[cu[b]:cu[b] + fit]
+            want_v[b, lens[b]:lens[b] + fit] = vn.to(dtype)[cu[b]:cu[b] + fit]
+        assert torch.equal(kc.cpu(), want_k) and torch.equal(vc.cpu(), want_v)
+        assert kv_len.cpu().tolist() == [5, 4, 10, 10]

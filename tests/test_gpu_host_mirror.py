@@ -295,3 +295,73 @@ def test_decode_rows_path_matches_generic_layer_path(env):
         del layer._decode_rows_ok
     assert fast.shape == slow.shape == (2, 1, HID)
     assert cf.rel_err(fast.cpu(), slow.double().cpu()) < 1e-2
+
+
+def test_injected_block_equals_token_by_token_decode(env):
+    """Memory-Interleave source-context injection: a ragged left-padded block of new tokens fed in one forward of
+    the decode stage must leave the caches and the last hidden state where feeding the same tokens one decode
+    step at a time leaves them."""
+    say("model: multi-token block in the decode stage vs token-by-token")
+    pf, svc_mod, M = env["prefill"], env["svc"], env["model"]
+    model = M.MSAForCausalLM(env["cfg"]).init_random(0.05, seed=6).to(torch.bfloat16).cuda().eval()
+    docs = _docs(env, [20, 33, 9, 41], first_id=0)
+    service = svc_mod.MSAService(0, env["config"].GenerateConfig(devices=[0]),
+                                 env["config"].ModelConfig(doc_top_k=TOPK, pooling_kernel_size=P, router_layer_idx="1"),
+                                 env["config"].MemoryConfig(pooling_kernel_size=P), env["cfg"])
+    service.begin(docs)
+    for blk in pf.split_docs(docs, 12):
+        service.add_block(M.encode_block(model, pf.prepare_block_inputs(blk, HEAD_IDS, P), "cuda"))
+    service.finish()
+    service.setup_memory_client(model)
+    ids = torch.tensor([[5, 6, 7, 8, 9, 10], [0, 0, 11, 12, 13, 14]]).cuda()
+    mask = torch.tensor([[1] * 6, [0, 0, 1, 1, 1, 1]]).cuda()
+    blocks = [[21, 22, 23, 24, 25], [31, 32]]
+
+    def run(block_mode):
+        _, cache = model.generate_greedy(ids, mask, torch.zeros_like(ids), 1)
+        for i in range(env["cfg"].num_hidden_layers):
+            cache.cache_kwargs[i]["stage"] = "generate"
+        lens0 = [cache.cache_kwargs[i]["kv_lengths"].clone() for i in range(2)]
+        pos0 = torch.tensor([3 + TOPK + 6 - 1, 3 + TOPK + 4 - 1]).cuda()
+        with torch.no_grad():
+            if block_mode:
+                x = torch.tensor([blocks[0], [0, 0, 0] + blocks[1]]).cuda()
+                m = torch.tensor([[1] * 5, [0, 0, 0, 1, 1]]).cuda()
+                p = torch.stack([pos0[0] + 1 + torch.arange(5).cuda(), torch.tensor([0, 0, 0, 1, 2]).cuda() + pos0[1] + (torch.tensor([1, 1, 1, 0, 0]).cuda())])
+                h = model.model(x, m, p, cache, torch.zeros_like(x))
+                last = h[:, -1]
+            else:
+                last = [None, None]
+                for t in range(5):
+                    tok = torch.tensor([[blocks[0][t]], [blocks[1][min(t, 1)]]]).cuda()
+                    h = model.model(tok, torch.ones_like(tok), (pos0 + 1 + t).unsqueeze(1), cache, torch.full_like(tok, -1))
+                    last[0] = h[0, 0]
+                    if t == 1:
+                        last[1] = h[1, 0]
+                last = torch.stack(last)
+        return last, cache, lens0
+
+    a, ca, lens0 = run(True)
+    b, cb, _ = run(False)
+    assert cf.rel_err(a.cpu(), b.double().cpu()) < 2e-2
+    for layer in range(2):
+        la = ca.cache_kwargs[layer]["kv_lengths"].cpu()
+        assert la.tolist() == (lens0[layer].cpu() + torch.tensor([5, 2])).tolist()
+        ka, kb = ca.cache_kwargs[layer]["compacked_key_cache"], cb.cache_kwargs[layer]["compacked_key_cache"]
+        for s_, n in enumerate([5, 2]):
+            lo = int(lens0[layer][s_])
+            assert cf.rel_err(ka[s_, lo:lo + n].cpu(), kb[s_, lo:lo + n].double().cpu()) < 2e-2
+
+    # the round loop itself: a hook that injects once, every sample keeps generating afterwards
+    calls = []
+
+    def inject(step, toks):
+        calls.append((step, tuple(toks.shape)))
+        return [[21, 22, 23], []] if step == 2 else None
+
+    toks, cache = M.generate_interleaved(model, ids, mask, torch.zeros_like(ids), 5, inject)
+    assert toks.shape == (2, 5) and calls[0] == (1, (2, 1)) and calls[-1] == (4, (2, 4))
+    plain, c0 = model.generate_greedy(ids, mask, torch.zeros_like(ids), 5)
+    assert torch.equal(toks[:, :2], plain[:, :2])                           # identical until the injection
+    grown = cache.cache_kwargs[1]["kv_lengths"].cpu() - c0.cache_kwargs[1]["kv_lengths"].cpu()
+    assert grown.tolist() == [2, 0]                                         # 3 injected tokens replaced 1 generated one

@@ -215,6 +215,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the pooling and decode-attention side measurements")
+    ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end sparse decode run among the extras")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for rocprof FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -417,6 +418,15 @@ def main():
                          f"{', '.join(f'{k} {v:.2f} s' for k, v in times.items())}; best extrapolated linearly "
                          f"x{C_total / Cs:.1f} chunks x{L} layers",
                "host_cpus": os.cpu_count()}
+
+    if extras is not None and not args.no_e2e:
+        # configs[4] end to end (the "sparse decode tok/s" half of the metric); ~25 GB next to the 100M bank's 60 GB
+        from msa_amd import e2e_decode
+        r = e2e_decode.main(["--steps", "128"], quiet=True)
+        extras["e2e_sparse_decode"] = {"workload": r["config"]["workload"] + ", 10M-token bank, B=16, 4K context, greedy",
+                                       "tokens_per_s": r["value"], "ms_per_decode_step": r["ms_per_decode_step"],
+                                       "prefill_s": r["prefill_s"], "decode_steps": r["config"]["decode_steps"],
+                                       "decode_mode": r["decode_mode"]}
 
     out = {
         "metric": "routed queries/s at the 100M-token bank (router scoring + top-k + host gather, 18 layers)",

@@ -56,7 +56,8 @@ def build_service(cfg: MSAConfig, bank_tokens: int, seed: int = 0) -> MSAService
     return svc
 
 
-def main(argv=None):
+def main(argv=None, quiet: bool = False):
+    """Runs the workload and prints one JSON line (``quiet`` only returns the dict)."""
     ap = argparse.ArgumentParser()
     ap.add_argument("--bank-tokens", type=int, default=10_000_000)
     ap.add_argument("--batch", type=int, default=16)
@@ -110,7 +111,9 @@ def main(argv=None):
                       "kv_rows_last_router_layer": kv[:4]},
            "decode_mode": "eager" if args.eager else "hip graph replay", "graph_equals_eager": verified,
            "generated_shape": list(toks.shape)}
-    print(json.dumps(out), flush=True)
+    del model, svc, cache
+    if not quiet:
+        print(json.dumps(out), flush=True)
     return out
 
 

@@ -9,7 +9,6 @@
 
 namespace {
 
-constexpr int kAttnWaves = 4;
 constexpr int kMaxG = 8;
 
 template <typename T>
@@ -32,7 +31,7 @@ __device__ __forceinline__ int find_sample(const int32_t* cu_q, int B, int row) 
   return b;
 }
 
-template <typename T, int G>
+template <typename T, int G, int kAttnWaves>
 __global__ __launch_bounds__(kAttnWaves * 64) void attn_partial_kernel(
     const T* __restrict__ q, const int32_t* __restrict__ cu_q, const T* __restrict__ k, const T* __restrict__ v,
     const int64_t* __restrict__ kv_off, const int32_t* __restrict__ kv_len, int32_t B, int32_t Hq, int32_t Hkv,
@@ -47,8 +46,10 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_partial_kernel(
   const int sq = cu_q ? cu_q[b + 1] - q_first : 1;
   const int L = kv_len[b];
   const int visible = causal ? max(0, L - sq + (row - q_first) + 1) : L;
-  const int key0 = split * split_keys;
-  const int key1 = min(visible, key0 + split_keys);
+  // balanced splits of this sample's own length (the host only knows an upper bound of it)
+  const int per_split = split_keys > 0 ? split_keys : (L + n_split - 1) / n_split;
+  const int key0 = split * per_split;
+  const int key1 = min(visible, key0 + per_split);
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int slot = lane >> 4, j = lane & 15;
@@ -192,17 +193,19 @@ int launch_attn(const void* q, const int32_t* cu_q, const void* k, const void* v
   const int G = Hq / Hkv;
   dim3 grid((unsigned)total_q, (unsigned)Hkv, (unsigned)n_split);
   const float sl2 = scale * 1.4426950408889634f;
-#define MSA_ATTN_CASE(GG)                                                                                          \
+  // Wavefronts per workgroup: the VALU work grows with the group size, and one 8-wavefront workgroup per
+  // compute unit measured better for G >= 4 than two of 4 (61 vs 64 us on the decode shape).
+#define MSA_ATTN_CASE(GG, WW)                                                                                      \
   case GG:                                                                                                         \
-    attn_partial_kernel<T, GG><<<grid, kAttnWaves * 64, 0, st>>>(                                                  \
+    attn_partial_kernel<T, GG, WW><<<grid, WW * 64, 0, st>>>(                                                      \
         static_cast<const T*>(q), cu_q, static_cast<const T*>(k), static_cast<const T*>(v), kv_off, kv_len, B, Hq, \
-        Hkv, sl2, causal, n_split, plan.split_keys, part_ml, part_acc);                                                             \
+        Hkv, sl2, causal, n_split, 0, part_ml, part_acc);                                                          \
     break;
   switch (G) {
-    MSA_ATTN_CASE(1)
-    MSA_ATTN_CASE(2)
-    MSA_ATTN_CASE(4)
-    MSA_ATTN_CASE(8)
+    MSA_ATTN_CASE(1, 4)
+    MSA_ATTN_CASE(2, 4)
+    MSA_ATTN_CASE(4, 8)
+    MSA_ATTN_CASE(8, 8)
     default:
       msa_set_error("msa_sparse_attn: GQA group size %d unsupported (1, 2, 4, 8)", G);
       return MSA_EINVAL;
@@ -219,7 +222,9 @@ int launch_attn(const void* q, const int32_t* cu_q, const void* k, const void* v
 
 extern "C" size_t msa_attn_workspace_bytes(int32_t total_q, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_kv) {
   if (total_q <= 0 || Hq <= 0 || Hkv <= 0 || D <= 0 || max_kv <= 0) return 0;
-  const size_t n = (size_t)total_q * Hq * plan_splits(total_q, Hkv, max_kv).n_split;
+  // sized for whichever of the two kernels splits the keys further
+  const int splits = std::max(plan_splits(total_q, Hkv, max_kv).n_split, plan_splits_valu(total_q, Hkv, max_kv).n_split);
+  const size_t n = (size_t)total_q * Hq * splits;
   return align_up(n * 2 * sizeof(float), 256) + align_up(n * D * sizeof(float), 256);
 }
 
@@ -236,7 +241,8 @@ extern "C" int msa_sparse_attn(const void* q, const int32_t* cu_q, const void* k
   MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "msa_sparse_attn: bad dtype %d", dtype);
   MSA_REQUIRE(scale > 0.f, "msa_sparse_attn: scale must be positive");
   MSA_REQUIRE((int64_t)total_q * Hq < (int64_t)1 << 31 && total_q < 65536 * 32, "msa_sparse_attn: too many rows");
-  const SplitPlan plan = plan_splits(total_q, Hkv, max_kv);
+  const bool mfma = dtype == MSA_BF16 && max_sq >= 8;
+  const SplitPlan plan = mfma ? plan_splits(total_q, Hkv, max_kv) : plan_splits_valu(total_q, Hkv, max_kv);
   const int n_split = plan.n_split;
   MSA_REQUIRE(n_split <= 65535, "msa_sparse_attn: max_kv=%d too large", max_kv);
   const size_t need = msa_attn_workspace_bytes(total_q, Hq, Hkv, D, max_kv);
@@ -248,7 +254,7 @@ extern "C" int msa_sparse_attn(const void* q, const int32_t* cu_q, const void* k
   float* part_ml = static_cast<float*>(workspace);
   float* part_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + align_up(n * 2 * sizeof(float), 256));
   hipStream_t st = as_stream(stream);
-  if (dtype == MSA_BF16 && max_sq >= 8) {
+  if (mfma) {
     // bf16 query blocks: MFMA partial pass (K / V tiles through LDS) + the common combine; single rows
     // (decode) stay on the split-KV kernel below, which keeps more loads in flight per wavefront
     int rc = flash_attn_split_launch(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, plan, part_ml,

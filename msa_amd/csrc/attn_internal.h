@@ -13,13 +13,23 @@ struct SplitPlan {
   int n_split;
   int split_keys;
 };
-static inline SplitPlan plan_splits(int64_t total_q, int32_t Hkv, int32_t max_kv) {
+static inline SplitPlan plan_splits_for(int64_t total_q, int32_t Hkv, int32_t max_kv, int target) {
   const int64_t pairs = std::max<int64_t>(1, total_q * Hkv);
-  const int by_fill = (int)std::max<int64_t>(1, (1024 + pairs - 1) / pairs);
+  const int by_fill = (int)std::max<int64_t>(1, (target + pairs - 1) / pairs);
   const int by_size = std::max(1, (max_kv + kMinSplitKeys - 1) / kMinSplitKeys);
   const int n = std::min(by_fill, by_size);
   const int keys = ((max_kv + n - 1) / n + 63) / 64 * 64;
   return {(max_kv + keys - 1) / keys, keys};
+}
+// MFMA split kernel: about 1024 workgroups.
+static inline SplitPlan plan_splits(int64_t total_q, int32_t Hkv, int32_t max_kv) {
+  return plan_splits_for(total_q, Hkv, max_kv, 1024);
+}
+// VALU split kernel (decode): one workgroup per compute unit measured best (fewer, longer key streams); the
+// kernel itself divides each sample's own length evenly over n_split.
+static inline SplitPlan plan_splits_valu(int64_t total_q, int32_t Hkv, int32_t max_kv) {
+  static const int target = [] { const char* e = getenv("MSA_ATTN_WGS"); return e ? atoi(e) : 256; }();
+  return plan_splits_for(total_q, Hkv, max_kv, target);
 }
 
 // flash_attn.hip: bf16 partial pass over split `blockIdx.z` of the keys; writes un-normalised

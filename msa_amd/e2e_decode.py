@@ -99,7 +99,10 @@ def main(argv=None, quiet: bool = False):
         ref, _ = model.generate_greedy(ids, mask, doc_ids, args.verify_graph, use_graph=False)
         verified = bool(torch.equal(ref, toks[:, :args.verify_graph]))
         if not verified:
-            sys.exit("e2e_decode: graph replays and eager decoding produced different tokens")
+            diff = ref != toks[:, :args.verify_graph]
+            first = int(diff.any(dim=0).nonzero()[0])
+            sys.exit(f"e2e_decode: graph replays and eager decoding produced different tokens: first at step {first}, "
+                     f"{int(diff.any(dim=1).sum())} of {B} samples differ")
     last_router = svc.router_layer_ids[-1]
     kv = cache.cache_kwargs[last_router]["kv_lengths"].cpu().tolist()
     out = {"metric": "sparse decode tok/s (end to end, greedy)", "value": round(B * timings["decode_steps"] / timings["decode_s"], 1),

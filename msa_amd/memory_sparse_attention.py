@@ -249,7 +249,11 @@ class MemorySparseAttention(nn.Module):
                 max_sel = int(n_sel.max())
             if cache.meta.get("require_recall_topk", False):
                 ck["recall_topk"] = [{"topk_doc_ids": gids[i].tolist(), "score": scores[i].float().tolist()} for i in range(B)]
-        local_k, local_v, q_rows = k[valid], v[valid], q[valid]           # ragged [sum S_b, H, D]
+        dense = min(n_q_host) == S                                        # no padding anywhere: the ragged rows are views
+        if dense:
+            local_k, local_v, q_rows = k.reshape(B * S, Hkv, D), v.reshape(B * S, Hkv, D), q.reshape(B * S, Hq, D)
+        else:
+            local_k, local_v, q_rows = k[valid], v[valid], q[valid]       # ragged [sum S_b, H, D]
         cu_local = F.pad(n_q.cumsum(0), (1, 0)).to(torch.int32)
         max_kv = n_prefix + max_sel + max(n_q_host)                       # upper bound of any sample's context rows
         Lcap = max_kv + self.decode_reserve
@@ -257,8 +261,11 @@ class MemorySparseAttention(nn.Module):
         kv_off = torch.arange(B, dtype=torch.int64, device=dev) * Lcap
         out_rows = ops.sparse_attn(q_rows, kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), kv_off, kv_len, max_kv,
                                    cu_q=cu_local, max_sq=max(n_q_host), scale=self.scaling, causal=True)
-        attn = torch.zeros((B, S, Hq * D), device=dev, dtype=dtype)
-        attn[valid] = out_rows.view(-1, Hq * D)
+        if dense:
+            attn = out_rows.view(B, S, Hq * D)
+        else:
+            attn = torch.zeros((B, S, Hq * D), device=dev, dtype=dtype)
+            attn[valid] = out_rows.view(-1, Hq * D)
         ck.update({"compacked_key_cache": kc, "compacked_value_cache": vc, "kv_lengths": kv_len, "kv_offsets": kv_off,
                    "kv_capacity": Lcap})
         cache.record_kwargs(self.layer_idx, ck)

@@ -480,3 +480,43 @@ def test_flash_attention_blocks(ops, Hq, Hkv, causal):
     finally:
         ops.FLASH_MIN_ROWS = old
     assert cf.rel_err(out2.cpu(), want) < 1e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_by_hand_fixture_through_the_c_abi(ops, dtype):
+    """tests/golden/by_hand.json (numbers derived by hand on one-hot vectors) through the HIP path: exact in both
+    dtypes, since every operand and every result is a small dyadic number."""
+    say(f"by-hand fixture dtype={dtype}")
+    from tests.golden import by_hand
+    fx = by_hand.load()
+    q, mask, kr, dco = by_hand.tensors(fx, dtype)
+    bank = ops.Bank(1, dco.tolist(), [10, 20, 30], fx["Hkv"], fx["D"], dtype)
+    kr_dev = kr.cuda()
+    kh = torch.arange(6, dtype=torch.float32).view(6, 1, 1).expand(6, 2, 128).to(dtype).contiguous().pin_memory()
+    bank.set_layer(0, kr_dev, kh, kh)
+    cs = ops.chunk_scores(bank, 0, q.cuda(), mask.cuda(), "cosine", 1.0).cpu()
+    assert torch.equal(cs, torch.tensor(fx["chunk_scores_cosine"]))
+    sd = ops.chunk_scores(bank, 0, q.cuda(), mask.cuda(), "scaled_dot", fx["D"] ** -0.5).cpu()
+    assert torch.allclose(sd, torch.tensor(fx["chunk_scores_cosine"]) * fx["scaled_dot_factor"], rtol=1e-6)
+    for k, key in ((2, "top2"), (3, "top3")):
+        s, doc, gid = ops.route_topk(bank, 0, q.cuda(), mask.cuda(), "cosine", 1.0, k)
+        assert doc.cpu().tolist() == fx[key]                                  # the tie goes to the lower document id
+        assert gid.cpu().tolist() == [[10 * (d + 1) for d in row] for row in fx[key]]
+        want = torch.tensor(fx["doc_scores_cosine"]).gather(1, torch.tensor(fx[key]))
+        assert torch.equal(s.cpu(), want)
+    p = fx["pool"]
+    t = ops.chunk_table(p["doc_lens"], p["P"])
+    assert (t.chunk_start.cpu().tolist(), t.chunk_len.cpu().tolist(), t.chunk_doc.cpu().tolist()) == \
+        (p["chunk_start"], p["chunk_len"], p["chunk_doc"])
+    x = (torch.arange(sum(p["doc_lens"]), dtype=torch.float32) + 1).view(-1, 1, 1).expand(-1, 8, 128).to(dtype).contiguous().cuda()
+    pk, pv, pkr = ops.pool_chunks(x, x, x, t, normalize_kr=True)
+    assert torch.equal(pv[:, 0, 0].float().cpu(), torch.tensor(p["chunk_mean"]))
+    assert torch.allclose(pkr.float().cpu(), torch.full((3, 8, 128), p["normalized_element"]), rtol=TOL[dtype])
+    gth = fx["gather"]
+    sel = torch.tensor(gth["selected"], dtype=torch.int32)
+    mk, mv, cu = ops.gather_kv(bank, 0, sel, "cuda")
+    torch.cuda.synchronize()
+    assert cu.tolist() == gth["cu_sel"] and mk[:, 0, 0].float().cpu().tolist() == [float(c) for row in gth["chunks"] for c in row]
+    mk2, mv2, cu2 = ops.gather_kv_device(bank, 0, sel.cuda(), 8)
+    torch.cuda.synchronize()
+    assert cu2.cpu().tolist() == gth["cu_sel"] and torch.equal(mk2[:6].cpu(), mk.cpu())

@@ -316,3 +316,42 @@ def test_decode_step_reference_style_agrees():
         kk = torch.cat([ks[b], kn[b].transpose(0, 1)]); vv = torch.cat([vs[b], vn[b].transpose(0, 1)])
         want = cf.attention(q[b].transpose(0, 1), kk, vv)
         assert cf.rel_err(out[b].transpose(0, 1), want) < 1e-5
+
+
+def test_by_hand_fixture_pins_the_oracle():
+    """tests/golden/by_hand.json: numbers worked out by hand on one-hot vectors (masking, head mean, token max,
+    chunk max, tie order, pooling means, gather order, positions).  A wrong axis, sign, offset or tie rule fails."""
+    from tests.golden import by_hand
+    fx = by_hand.load()
+    q, mask, kr, dco = by_hand.tensors(fx)
+    cs = cf.chunk_scores(q, mask, kr, "cosine")
+    assert torch.allclose(cs, torch.tensor(fx["chunk_scores_cosine"], dtype=cs.dtype), atol=1e-12)
+    sd = cf.chunk_scores(q, mask, kr, "scaled_dot", scale=fx["D"] ** -0.5)
+    assert torch.allclose(sd, torch.tensor(fx["chunk_scores_cosine"], dtype=sd.dtype) * fx["scaled_dot_factor"], atol=1e-12)
+    ds = cf.doc_scores(cs, dco)
+    assert torch.allclose(ds, torch.tensor(fx["doc_scores_cosine"], dtype=ds.dtype), atol=1e-12)
+    assert cf.topk_docs(ds, 2)[1].tolist() == fx["top2"] and cf.topk_docs(ds, 3)[1].tolist() == fx["top3"]
+    # the reference's own op order gives the same numbers
+    qh = torch.nn.functional.normalize(q.permute(0, 2, 1, 3), p=2, dim=-1)
+    q5, m5 = rs.group_queries(qh, mask, fx["Hq"] // fx["Hkv"], -1.0)
+    chunks = np.diff(dco).tolist()
+    pool_ids = torch.repeat_interleave(torch.arange(1, len(chunks) + 1), torch.as_tensor(chunks))
+    s_ref, i_ref = rs.stage2_scores_topk(q5, m5, kr.transpose(0, 1).unsqueeze(0), pool_ids, chunks, 2)
+    assert torch.allclose(s_ref.double(), torch.tensor([[1.0, 0.5], [1.0, 0.5]], dtype=torch.float64), atol=1e-6)
+    assert (i_ref[:, 0] - 1).tolist() == [r[0] for r in fx["top2"]]          # 1-based pool ids; rank 0 has no tie
+    # pooling
+    p = fx["pool"]
+    _, off, cstart, clen, cdoc = cf.chunk_table(p["doc_lens"], p["P"])
+    assert (cstart.tolist(), clen.tolist(), cdoc.tolist(), off.tolist()) == (p["chunk_start"], p["chunk_len"], p["chunk_doc"],
+                                                                            p["doc_chunk_off"])
+    x = (torch.arange(sum(p["doc_lens"]), dtype=torch.float64) + 1).view(-1, 1, 1).expand(-1, 2, 128)
+    pooled = cf.pool_chunks(x, cstart, clen)
+    assert torch.allclose(pooled[:, 0, 0], torch.tensor(p["chunk_mean"], dtype=torch.float64), atol=1e-12)
+    assert torch.allclose(cf.l2_normalize(pooled), torch.full_like(pooled, p["normalized_element"]), atol=1e-12)
+    # gather order and positions
+    gth = fx["gather"]
+    bank = torch.arange(6, dtype=torch.float64).view(6, 1, 1).expand(6, 2, 128)
+    mk, _, cu, _ = cf.gather_selected(bank, bank, dco, torch.tensor(gth["selected"]))
+    assert cu.tolist() == gth["cu_sel"] and mk[:, 0, 0].tolist() == [float(c) for row in gth["chunks"] for c in row]
+    ps = fx["positions"]
+    assert cf.query_positions(ps["n_query"], ps["top_k"], ps["n_prefix"], ps["left_pad"]).tolist() == ps["position_ids"]

@@ -3,10 +3,10 @@
 // with M <= 16.  The weight matrix is read from HBM exactly once, which is the whole cost: per
 // decode step of a 36-layer model the projections stream ~8 GB.  The 16 rows of x are exactly one
 // 16x16x32 MFMA operand, so a wavefront multiplies 16 weight rows (one row group) at a time:
-//   lane (n = lane % 16, g = lane / 16), vector j = 0..3, loads the 16 bytes of weight row n at
-//   k = unit * 128 + 32 j + 8 g   (one load instruction covers 64 contiguous bytes of each of 16 rows),
-// and the same bytes of x row n.  The contraction order inside a 128-wide unit is permuted the same
-// way on both operands, which a dot product does not see.  A workgroup owns R row groups and splits
+//   lane (n = lane % 16, g = lane / 16), vector j = 0..J-1, loads the 16 bytes of weight row n at
+//   k = unit * 32 J + 32 j + 8 g   (one load instruction covers 64 contiguous bytes of each of 16 rows),
+// and the same bytes of x row n (J = 4, or 2 when the RMSNorm is folded in).  The contraction order
+// inside a unit is permuted the same way on both operands, which a dot product does not see.  A workgroup owns R row groups and splits
 // K over its wavefronts; partial sums meet in LDS and are added in wavefront order (deterministic).
 #include <algorithm>
 
@@ -210,7 +210,6 @@ extern "C" int msa_skinny_linear(const void* x, const void* w, const void* resid
   MSA_REQUIRE((((uintptr_t)x | (uintptr_t)w | (uintptr_t)norm_w) & 15) == 0, "msa_skinny_linear: x / w / norm_w must be 16-byte aligned");
   const int units = K / kUnit;
   MSA_REQUIRE(norm_w == nullptr || eps > 0.f, "msa_skinny_linear: folded RMSNorm needs eps > 0");
-  const int max_waves = kMaxWaves;
   hipStream_t st = as_stream(stream);
 
   // Wavefronts per workgroup: split K far enough that the launch has a few thousand wavefronts, and
@@ -223,14 +222,12 @@ extern "C" int msa_skinny_linear(const void* x, const void* w, const void* resid
   if (env_r == 1 && epilogue != kEpiSiluMul) R = 1;
   if (env_r == 2) R = 2;
   const int groups = (N + 16 * R - 1) / (16 * R);
-  int want = (int)std::min<int64_t>(max_waves, std::max<int64_t>(1, (4096 + groups - 1) / groups));
-  want = std::min(want, units);
-  const int least = 1;
-  want = std::max(want, least);
+  int want = (int)std::min<int64_t>(kMaxWaves, std::max<int64_t>(1, (4096 + groups - 1) / groups));
+  want = std::max(1, std::min(want, units));
   int waves = want;
-  for (int cand = want; cand >= std::max(least, want / 2); --cand)
+  for (int cand = want; cand >= std::max(1, want / 2); --cand)
     if (units % cand == 0) { waves = cand; break; }
-  if (env_waves > 0) waves = std::max(least, std::min(std::min(env_waves, max_waves), units));
+  if (env_waves > 0) waves = std::max(1, std::min(std::min(env_waves, kMaxWaves), units));
 
 #define MSA_LIN(R_, E_)                                                                              \
   (norm_w ? launch<R_, E_, true>(x, w, residual, norm_w, eps, y, M, N, K, waves, st)                 \
@@ -242,7 +239,7 @@ extern "C" int msa_skinny_linear(const void* x, const void* w, const void* resid
     case kEpiResidual * 8 + 2: return MSA_LIN(2, kEpiResidual);
     case kEpiSiluMul * 8 + 2: return MSA_LIN(2, kEpiSiluMul);
   }
+#undef MSA_LIN
   msa_set_error("msa_skinny_linear: no kernel for epilogue %d with %d row groups", epilogue, R);
   return MSA_EINVAL;
-#undef MSA_LIN
 }

@@ -101,24 +101,53 @@ __global__ void qk_norm_rope_kernel(const T* __restrict__ q, const T* __restrict
 }
 
 // One workgroup per row.  With `residual`: residual <- residual + x (stored in T), then normalised.
+// Eight elements per lane per step (16-byte accesses for bf16) when H is a multiple of 8 and every tensor is
+// 16-byte aligned (`vec`); the summed row is kept in registers between
+// the two passes when it fits (H <= 256 * 8 * kKeep), otherwise it is re-read from `residual` / `x`.
 template <typename T>
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, T* __restrict__ residual,
                                                       const T* __restrict__ w, int32_t H, float eps,
-                                                      T* __restrict__ out) {
+                                                      T* __restrict__ out, int32_t vec) {
+  constexpr int kKeep = 2;                       // steps of a row held in registers (H <= 4096)
   __shared__ float part[4];
   const int64_t row = blockIdx.x;
   const T* xr = x + row * H;
   T* rr = residual ? residual + row * H : nullptr;
+  T* orow = out + row * H;
+  float keep[kKeep][8];
   float ssq = 0.f;
-  for (int i = threadIdx.x; i < H; i += 256) {
-    float v;
-    if constexpr (sizeof(T) == 2) v = bf16_to_f32(xr[i]); else v = xr[i];
-    if (rr) {
-      float r;
-      if constexpr (sizeof(T) == 2) { r = bf16_to_f32(rr[i]); v = bf16_to_f32(f32_to_bf16(v + r)); rr[i] = f32_to_bf16(v); }
-      else { r = rr[i]; v = v + r; rr[i] = v; }
+  if (vec) {
+    int step = 0;
+    for (int i = threadIdx.x * 8; i < H; i += 256 * 8, ++step) {
+      float v[8];
+      load8g<T>(xr + i, v);
+      if (rr) {
+        float r[8];
+        load8g<T>(rr + i, r);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          v[e] += r[e];
+          if constexpr (sizeof(T) == 2) v[e] = bf16_to_f32(f32_to_bf16(v[e]));     // the residual stream is stored in T
+        }
+        store8g<T>(rr + i, v);
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) ssq += v[e] * v[e];
+      if (step < kKeep) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) keep[step][e] = v[e];
+      }
     }
-    ssq += v * v;
+  } else {
+    for (int i = threadIdx.x; i < H; i += 256) {
+      float v;
+      if constexpr (sizeof(T) == 2) v = bf16_to_f32(xr[i]); else v = xr[i];
+      if (rr) {
+        if constexpr (sizeof(T) == 2) { v = bf16_to_f32(f32_to_bf16(v + bf16_to_f32(rr[i]))); rr[i] = f32_to_bf16(v); }
+        else { v = v + rr[i]; rr[i] = v; }
+      }
+      ssq += v * v;
+    }
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) ssq += __shfl_xor(ssq, o);
@@ -126,18 +155,49 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, T
   __syncthreads();
   const float inv = rsqrtf((part[0] + part[1] + part[2] + part[3]) / (float)H + eps);
   const T* src = rr ? rr : xr;      // rr was written by this same thread for the same indices
-  for (int i = threadIdx.x; i < H; i += 256) {
-    float v, g;
-    if constexpr (sizeof(T) == 2) { v = bf16_to_f32(src[i]); g = bf16_to_f32(w[i]); out[row * H + i] = f32_to_bf16(v * inv * g); }
-    else { v = src[i]; g = w[i]; out[row * H + i] = v * inv * g; }
+  if (vec) {
+    int step = 0;
+    for (int i = threadIdx.x * 8; i < H; i += 256 * 8, ++step) {
+      float v[8], g[8];
+      if (step < kKeep) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = keep[step][e];
+      } else {
+        load8g<T>(src + i, v);
+      }
+      load8g<T>(w + i, g);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = v[e] * inv * g[e];
+      store8g<T>(orow + i, v);
+    }
+  } else {
+    for (int i = threadIdx.x; i < H; i += 256) {
+      float v, g;
+      if constexpr (sizeof(T) == 2) { v = bf16_to_f32(src[i]); g = bf16_to_f32(w[i]); orow[i] = f32_to_bf16(v * inv * g); }
+      else { v = src[i]; g = w[i]; orow[i] = v * inv * g; }
+    }
   }
 }
 
-// out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]
+// out[n, i] = silu(gate_up[n, i]) * gate_up[n, I + i]; eight elements per lane (16-byte accesses for bf16)
+// when I is a multiple of 8 and the tensors are 16-byte aligned (`vec`).
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gate_up, int64_t N, int32_t I, T* __restrict__ out) {
-  const int64_t total = N * I;
+__global__ void silu_mul_kernel(const T* __restrict__ gate_up, int64_t N, int32_t I, T* __restrict__ out, int32_t vec) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  if (vec) {
+    const int64_t per_row = I / 8, total = N * per_row;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
+      const int64_t n = idx / per_row, i = (idx % per_row) * 8;
+      float g[8], u[8];
+      load8g<T>(gate_up + n * 2 * I + i, g);
+      load8g<T>(gate_up + n * 2 * I + I + i, u);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) g[e] = g[e] / (1.0f + __expf(-g[e])) * u[e];
+      store8g<T>(out + n * I + i, g);
+    }
+    return;
+  }
+  const int64_t total = N * I;
   for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += stride) {
     const int64_t n = idx / I, i = idx % I;
     float g, u;
@@ -210,12 +270,13 @@ extern "C" int msa_rmsnorm(const void* x, void* residual, const void* weight, in
   MSA_REQUIRE(x && weight && out, "msa_rmsnorm: null pointer");
   MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "msa_rmsnorm: bad dtype %d", dtype);
   MSA_REQUIRE(N > 0 && N < (int64_t)1 << 31 && H > 0, "msa_rmsnorm: bad shape");
+  const int vec = (H & 7) == 0 && (((uintptr_t)x | (uintptr_t)residual | (uintptr_t)weight | (uintptr_t)out) & 15) == 0;
   if (dtype == MSA_BF16)
     rmsnorm_kernel<bf16_t><<<(unsigned)N, 256, 0, as_stream(stream)>>>((const bf16_t*)x, (bf16_t*)residual,
-                                                                       (const bf16_t*)weight, H, eps, (bf16_t*)out);
+                                                                       (const bf16_t*)weight, H, eps, (bf16_t*)out, vec);
   else
     rmsnorm_kernel<float><<<(unsigned)N, 256, 0, as_stream(stream)>>>((const float*)x, (float*)residual,
-                                                                      (const float*)weight, H, eps, (float*)out);
+                                                                      (const float*)weight, H, eps, (float*)out, vec);
   MSA_LAUNCH_CHECK();
   return MSA_OK;
 }
@@ -225,11 +286,13 @@ extern "C" int msa_silu_mul(const void* gate_up, int32_t dtype, int64_t N, int32
   MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "msa_silu_mul: bad dtype %d", dtype);
   MSA_REQUIRE(N > 0 && I > 0, "msa_silu_mul: bad shape");
   const int64_t total = N * I;
-  const int grid = (int)std::min<int64_t>((total + 255) / 256, 16384);
+  const int vec = (I & 7) == 0 && (((uintptr_t)gate_up | (uintptr_t)out) & 15) == 0;
+  const int64_t items = vec ? total / 8 : total;
+  const int grid = (int)std::min<int64_t>((items + 255) / 256, 16384);
   if (dtype == MSA_BF16)
-    silu_mul_kernel<bf16_t><<<grid, 256, 0, as_stream(stream)>>>((const bf16_t*)gate_up, N, I, (bf16_t*)out);
+    silu_mul_kernel<bf16_t><<<grid, 256, 0, as_stream(stream)>>>((const bf16_t*)gate_up, N, I, (bf16_t*)out, vec);
   else
-    silu_mul_kernel<float><<<grid, 256, 0, as_stream(stream)>>>((const float*)gate_up, N, I, (float*)out);
+    silu_mul_kernel<float><<<grid, 256, 0, as_stream(stream)>>>((const float*)gate_up, N, I, (float*)out, vec);
   MSA_LAUNCH_CHECK();
   return MSA_OK;
 }

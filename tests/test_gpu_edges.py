@@ -230,3 +230,28 @@ def test_cache_append_rows_ragged_and_clamped(ops):
             want_v[b, lens[b]:lens[b] + fit] = vn.to(dtype)[cu[b]:cu[b] + fit]
         assert torch.equal(kc.cpu(), want_k) and torch.equal(vc.cpu(), want_v)
         assert kv_len.cpu().tolist() == [5, 4, 10, 10]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("H", [8, 100, 2560, 5120, 9000])
+def test_rmsnorm_and_silu_mul_widths(ops, dtype, H):
+    """Row widths on and off the 8-element vector path, and rows longer than what the kernel keeps in registers."""
+    say(f"rmsnorm / silu_mul H={H} dtype={dtype}")
+    g = torch.Generator().manual_seed(H)
+    N, eps = 5, 1e-6
+    x, res = torch.randn((N, H), generator=g).to(dtype), torch.randn((N, H), generator=g).to(dtype)
+    w = (1 + 0.1 * torch.randn(H, generator=g)).to(dtype)
+    tol = 1e-2 if dtype == torch.bfloat16 else 1e-5
+
+    def ref(v):
+        v = v.double()
+        return v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps) * w.double()
+
+    assert cf.rel_err(ops.rmsnorm(x.cuda(), w.cuda(), eps).cpu(), ref(x)) < tol
+    res_dev = res.clone().cuda()
+    out = ops.rmsnorm(x.cuda(), w.cuda(), eps, residual=res_dev).cpu()
+    summed = (x.double() + res.double()).to(dtype)
+    assert torch.equal(res_dev.cpu(), summed) and cf.rel_err(out, ref(summed)) < tol
+    gu = torch.randn((N, 2 * H), generator=g).to(dtype)
+    want = torch.nn.functional.silu(gu[:, :H].double()) * gu[:, H:].double()
+    assert cf.rel_err(ops.silu_mul(gu.cuda()).cpu(), want) < tol

@@ -365,3 +365,48 @@ def test_injected_block_equals_token_by_token_decode(env):
     assert torch.equal(toks[:, :2], plain[:, :2])                           # identical until the injection
     grown = cache.cache_kwargs[1]["kv_lengths"].cpu() - c0.cache_kwargs[1]["kv_lengths"].cpu()
     assert grown.tolist() == [2, 0]                                         # 3 injected tokens replaced 1 generated one
+
+
+class _StubAttention(torch.nn.Module):
+    """Stands in for the attention block: a fixed linear map, so the decoder layer's own norm / residual / MLP
+    wiring can be compared between its fused-kernel path on the GPU and the plain torch path on the CPU."""
+
+    def __init__(self, hid, seed):
+        super().__init__()
+        g = torch.Generator().manual_seed(seed)
+        self.a = torch.nn.Parameter(torch.randn((hid, hid), generator=g) * hid ** -0.5)
+        self.layer_idx = 0
+
+    def forward(self, hidden_states, *args, **kwargs):
+        return hidden_states @ self.a.to(hidden_states.dtype), None
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_decoder_layer_glue_matches_plain_torch(env, dtype):
+    say(f"decoder layer: fused norm / residual / MLP kernels vs plain torch, dtype={dtype}")
+    M = env["model"]
+    torch.manual_seed(3)
+    layer = M.MSADecoderLayer(env["cfg"], 0)
+    layer.self_attn = _StubAttention(HID, 5)
+    with torch.no_grad():
+        for p in layer.parameters():
+            if p.dim() == 1:
+                p.copy_(1.0 + 0.1 * torch.randn(p.shape))
+    layer = layer.eval()
+    x = torch.randn((3, 7, HID), generator=torch.Generator().manual_seed(8))
+    with torch.no_grad():
+        want = layer.double()(x.double(), None, None, None, object())                 # CPU: the plain torch branch
+        got = layer.to(dtype).cuda()(x.to(dtype).cuda(), None, None, None, object(), position_ids=None)
+    assert cf.rel_err(got.cpu(), want) < (2e-2 if dtype == torch.bfloat16 else 1e-5)
+    # the weight-streaming MLP of the decode step against the same module's torch arithmetic
+    if dtype == torch.bfloat16:
+        h = torch.randn((5, HID), generator=torch.Generator().manual_seed(9)).bfloat16().cuda()
+        n2 = layer.post_attention_layernorm
+        with torch.no_grad():
+            got = layer.mlp.decode_rows(h, n2.weight, n2.variance_epsilon)
+            hd = h.double().cpu()
+            w = {k: v.double().cpu() for k, v in layer.state_dict().items()}
+            normed = hd * torch.rsqrt((hd * hd).mean(-1, keepdim=True) + n2.variance_epsilon) * w["post_attention_layernorm.weight"]
+            act = torch.nn.functional.silu(normed @ w["mlp.gate_proj.weight"].T) * (normed @ w["mlp.up_proj.weight"].T)
+            want = hd + act @ w["mlp.down_proj.weight"].T
+        assert cf.rel_err(got.cpu(), want) < 2e-2

@@ -1,4 +1,4 @@
-"""End-to-end sparse generation at Qwen3-4B shape (BASELINE configs[4]): random-init bf16 weights,
+"""End-to-end sparse generation at Qwen3-4B shape (the end-to-end benchmark configuration): random-init bf16 weights,
 36 layers, routing on the upper 18, a synthetic pooled memory bank, top-16 documents, a 4K-token
 local context per query, batch 16, greedy decoding.
 

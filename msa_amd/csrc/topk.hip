@@ -63,7 +63,13 @@ __global__ __launch_bounds__(kWaves * 64) void doc_topk_kernel(const uint32_t* _
     if (d < d_end) {
       const int c0 = doc_chunk_off[d], c1 = doc_chunk_off[d + 1];
       uint32_t m = 0;
-      for (int c = c0; c < c1; ++c) m = max(m, key[c]);
+      for (int c = c0; c < c1; c += 16) {          // 16 independent loads in flight per lane (clamped: duplicates are harmless)
+        uint32_t kv[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) kv[u] = key[min(c + u, c1 - 1)];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) m = max(m, kv[u]);
+      }
       v = ((uint64_t)m << 32) | (uint64_t)(0xffffffffu - (uint32_t)d);
     }
     v = wave_sort_desc(v, lane);

@@ -177,6 +177,26 @@ def extra_decode(dev):
             "attention_only_tok_per_s_36_layers": round(B / (36 * ms) * 1e3)}
 
 
+def extra_routing_10m(dev):
+    """configs[2]: router scoring + top-k on a 10M-token bank (about 156k chunks), batch 32 x 128 query tokens,
+    top-16, one routed layer per call (the 18 layers of a model cost 18 of these)."""
+    from msa_amd import ops
+    B, S = 32, 128
+    doc_chunks = [-(-n // P) for n in make_doc_lens(10_000_000, 2)]
+    off = np.concatenate([[0], np.cumsum(doc_chunks)])
+    bank = ops.Bank(1, off.tolist(), list(range(len(doc_chunks))), HKV, D, torch.bfloat16)
+    kr = build_kr_layer(int(off[-1]), 21, dev)
+    bank.set_layer(0, kr)
+    g = torch.Generator(device=dev).manual_seed(22)
+    q = torch.randn((B, S, HQ, D), generator=g, device=dev).to(torch.bfloat16)
+    ms = time_cuda(lambda: ops.route_topk(bank, 0, q, None, "cosine", 1.0, TOPK), 10)
+    fl = 2.0 * B * S * HKV * D * int(off[-1])
+    return {"workload": "configs[2]: 10M-token bank, B=32 x S=128, top-16, bf16, one layer",
+            "chunks": int(off[-1]), "docs": len(doc_chunks), "ms_per_layer": round(ms, 4),
+            "queries_per_s_18_layers": round(B / (18 * ms) * 1e3, 1), "TFLOP/s": round(fl / ms / 1e9, 1),
+            "frac_mfma_peak": round(fl / ms / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
+
+
 def extra_prefill_attention(dev):
     """Stage-2 prefill attention of the end-to-end shape: B=16 queries of 4096 tokens over
     [3 + 288 memory rows | the 4096 query tokens], causal, GQA 32/8, bf16 (MFMA flash kernel)."""
@@ -404,7 +424,7 @@ def main():
 
     extras = None
     if not args.no_extras:
-        extras = {"pooling": extra_pooling(dev), "decode_attention": extra_decode(dev),
+        extras = {"pooling": extra_pooling(dev), "routing_10M_bank": extra_routing_10m(dev), "decode_attention": extra_decode(dev),
                   "prefill_attention": extra_prefill_attention(dev)}
 
     cpu = None

@@ -9,6 +9,11 @@
 
 namespace {
 
+// 2^x by the bare hardware instruction: the library exp2f wraps it in a range fix-up for results below
+// 2^-126 (five more VALU operations per call); softmax arguments are <= 0 and such tails may flush to zero.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+
 constexpr int kMaxG = 8;
 
 template <typename T>
@@ -75,13 +80,13 @@ __device__ __forceinline__ void attend_keys(const T* __restrict__ k, const T* __
         mb = fmaxf(mb, s[u]);
       }
       // mb is finite here: the batch's first key is always valid
-      const float alpha = exp2f(m[h] - mb);
+      const float alpha = fast_exp2(m[h] - mb);
       float psum = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[h][i] *= alpha;
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
-        const float pu = exp2f(s[u] - mb);
+        const float pu = fast_exp2(s[u] - mb);
         psum += pu;
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[h][i] += pu * vx[u][i];
@@ -156,13 +161,13 @@ __device__ __forceinline__ void attend_keys_bf16(const bf16_t* __restrict__ k, c
       float mb = m[h];
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) mb = fmaxf(mb, s[h][u]);
-      const float alpha = exp2f(m[h] - mb);          // mb is finite: the batch's first key is always valid
+      const float alpha = fast_exp2(m[h] - mb);          // mb is finite: the batch's first key is always valid
       float psum = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[h][i] *= alpha;
 #pragma unroll
       for (int pr = 0; pr < kBatch / 2; ++pr) {
-        const float p0 = exp2f(s[h][2 * pr] - mb), p1 = exp2f(s[h][2 * pr + 1] - mb);
+        const float p0 = fast_exp2(s[h][2 * pr] - mb), p1 = fast_exp2(s[h][2 * pr + 1] - mb);
         psum += p0 + p1;
         const uint32_t pp = pack_pair_rne(p0, p1);
 #pragma unroll
@@ -239,7 +244,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_partial_kernel(
     for (int x = 16; x <= 32; x <<= 1) {
       const float mo = __shfl_xor(m[h], x), lo = __shfl_xor(l[h], x);
       const float mn = fmaxf(m[h], mo);
-      const float a = mn == -INFINITY ? 0.f : exp2f(m[h] - mn), bo = mn == -INFINITY ? 0.f : exp2f(mo - mn);
+      const float a = mn == -INFINITY ? 0.f : fast_exp2(m[h] - mn), bo = mn == -INFINITY ? 0.f : fast_exp2(mo - mn);
       l[h] = l[h] * a + lo * bo;
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[h][i] = acc[h][i] * a + __shfl_xor(acc[h][i], x) * bo;
@@ -265,7 +270,7 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_partial_kernel(
     float lt = 0.f, at = 0.f;
 #pragma unroll
     for (int w = 0; w < kAttnWaves; ++w) {
-      const float a = mn == -INFINITY ? 0.f : exp2f(sm_m[w][h] - mn);
+      const float a = mn == -INFINITY ? 0.f : fast_exp2(sm_m[w][h] - mn);
       lt += sm_l[w][h] * a;
       at += sm_acc[w][h][d] * a;
     }
@@ -287,7 +292,7 @@ __global__ __launch_bounds__(kHeadDim) void attn_combine_kernel(const float* __r
   float lt = 0.f, at = 0.f;
   for (int s = 0; s < n_split; ++s) {
     const float ms = part_ml[(rh * n_split + s) * 2];
-    const float a = ms == -INFINITY ? 0.f : exp2f(ms - mn);
+    const float a = ms == -INFINITY ? 0.f : fast_exp2(ms - mn);
     lt += part_ml[(rh * n_split + s) * 2 + 1] * a;
     at += part_acc[(rh * n_split + s) * kHeadDim + d] * a;
   }

@@ -16,6 +16,11 @@
 
 namespace {
 
+// 2^x by the bare hardware instruction: the library exp2f wraps it in a range fix-up for results below
+// 2^-126 (five more VALU operations per call); softmax arguments are <= 0 and such tails may flush to zero.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
 
@@ -181,7 +186,7 @@ __global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
     const bool grow = !none && mx > m + 6.0f;
     if (__any(grow)) {
       const float mref = none ? m : mx;
-      const float alpha = (none || m == -INFINITY) ? (m == -INFINITY ? 0.f : 1.f) : exp2f(m - mref);
+      const float alpha = (none || m == -INFINITY) ? (m == -INFINITY ? 0.f : 1.f) : fast_exp2(m - mref);
       l *= alpha;
 #pragma unroll
       for (int d = 0; d < 4; ++d)
@@ -195,7 +200,7 @@ __global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const float p = none ? 0.f : exp2f(s[rb][e] - m);
+        const float p = none ? 0.f : fast_exp2(s[rb][e] - m);
         psum += p;
         pf[rb][e >> 3][e & 7] = (__bf16)p;
       }

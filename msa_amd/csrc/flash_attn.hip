@@ -158,26 +158,26 @@ __global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
 
     // online softmax of this lane's column; element e of block rb is key 64 t + 32 rb + 8 (e / 4) + 4 half + e % 4
     const int key_base = t * kKeysPerTile + 4 * half;
-    float mx = m;
+    // (the maximum is taken over the raw dot products and scaled once: scale > 0; the scale itself is folded
+    //  into the exponent's argument with one fma per element further down)
+    float mx_raw = -INFINITY;
     if ((t + 1) * kKeysPerTile <= wave_min_limit) {    // interior tile: every key visible to every column
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          s[rb][e] *= scale_log2e;
-          mx = fmaxf(mx, s[rb][e]);
-        }
+        for (int e = 0; e < 16; ++e) mx_raw = fmaxf(mx_raw, s[rb][e]);
     } else {
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int key = key_base + 32 * rb + 8 * (e >> 2) + (e & 3);
-          const float x = key < limit ? s[rb][e] * scale_log2e : -INFINITY;
+          const float x = key < limit ? s[rb][e] : -INFINITY;
           s[rb][e] = x;
-          mx = fmaxf(mx, x);
+          mx_raw = fmaxf(mx_raw, x);
         }
     }
+    float mx = fmaxf(m, mx_raw * scale_log2e);
     mx = fmaxf(mx, __shfl_xor(mx, 32));
     const bool none = mx == -INFINITY;                 // nothing visible to this column so far
     // Lazy rescaling: keep the old reference maximum while the new one is at most 2^6 above it; the
@@ -194,13 +194,14 @@ __global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
         for (int e = 0; e < 16; ++e) o[d][e] *= alpha;
       m = mref;
     }
+    const float neg_m = none ? 0.f : -m;               // nothing visible yet: every score is -inf, keep the argument -inf
     float psum = 0.f;
     bf16x8_t pf[2][2];
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
       for (int e = 0; e < 16; ++e) {
-        const float p = none ? 0.f : fast_exp2(s[rb][e] - m);
+        const float p = fast_exp2(fmaf(s[rb][e], scale_log2e, neg_m));     // -inf (masked) -> 0
         psum += p;
         pf[rb][e >> 3][e & 7] = (__bf16)p;
       }

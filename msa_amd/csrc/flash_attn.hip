@@ -9,9 +9,16 @@
 //   O^T[128 dims x 32 cols] += V^T . P^T      (contraction over keys).
 // S^T's accumulator layout IS the B-operand layout of the second product (same lane, same
 // column), up to the order of keys inside a group of 16, which the V^T operand mirrors, so P never
-// leaves registers.  V is transposed on its way into LDS (16-bit stores into [dim][key] rows with
-// that key order, XOR-swizzled so the stores of a wavefront spread over all banks) and read back
-// as 16-byte operands.
+// leaves registers.  V goes into LDS as it lies in memory ([key][dim] rows, 16-byte stores) and the
+// V^T operand comes out of gfx950's transposing LDS read (ds_read_b64_tr_b16): sixteen lanes hand in
+// the sixteen 8-byte pieces of four key rows x 16 dims and lane j of them receives dim j of the four
+// keys, so the transpose costs no instruction and the key order is whatever rows the lanes name.
+//
+// The loop is software-pipelined inside the wavefront: the scores of tile t + 1 are produced in the
+// same straight-line block as the exponentials of tile t, and an explicit issue order (scheduling
+// groups) puts the LDS reads two products ahead of their use, so one wavefront keeps the matrix pipe,
+// the VALU and the LDS busy at once.  K and V are double-buffered out of phase (iteration t reads
+// K(t + 1) and V(t) and stores K(t + 2) and V(t + 1)), one barrier per tile.
 #include "attn_internal.h"
 
 namespace {
@@ -26,28 +33,52 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
 
 constexpr int kKeysPerTile = 64;
 constexpr int kTileStride = 2 * kHeadDim + 16;   // bytes per key row in LDS: 256 + 16 pad (conflict-free b128 reads)
-constexpr int kVtStride = 2 * kKeysPerTile + 16;  // bytes per dim row of the transposed V tile
-constexpr int kFlashWaves = 4;
+constexpr int kVStride = 2 * kHeadDim + 64;      // bytes per key row of the V tile: four consecutive keys x 64 bytes
+                                                  // (one transposing read of a half-wave) cover all 64 banks once
+constexpr int kStageBytes = kKeysPerTile * (kTileStride + kVStride);   // one K tile + one V tile
+constexpr int kWaves = 4;
+constexpr int kLdsBytes = 2 * kStageBytes;
 
-// Position of key (0..63) inside a V^T row: bits 2 and 3 swapped (the accumulator layout holds keys
-// {0-3, 8-11} in one half-wave and {4-7, 12-15} in the other), then XOR with a per-dim-group value.
-__device__ __forceinline__ int vt_pos(int key, int dim) {
-  const int p = (key & ~12) | ((key & 4) << 1) | ((key & 8) >> 1);
-  return p ^ ((dim >> 4) << 3);
+// max / sum of a value over the two half-waves (lane and lane ^ 32), by the half-wave swap instruction
+__device__ __forceinline__ float half_wave_max(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float half_wave_sum(float x) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float floatx2_t __attribute__((ext_vector_type(2)));
+// two floats -> packed bf16 pair, round to nearest even (one v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint32_t pack_pair(float lo, float hi) {
+  floatx2_t f = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
+}
+
+typedef short shortx4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) shortx4_t lds_shortx4_t;
+
+// Transposing LDS read of 16-bit elements: within each group of 16 lanes, lanes 4 r .. 4 r + 3 name the four
+// 8-byte pieces of row r (r = 0..3, 16 elements) and lane j receives element j of rows 0..3.
+__device__ __forceinline__ shortx4_t lds_read_tr16(const char* p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t*)(p));
 }
 
 // kSplit: blockIdx.z selects a range of split_keys keys; the un-normalised accumulators and the
 // (reference max, sum) pair of every column go to part_acc / part_ml for the combine kernel.
 template <int G, bool kSplit>
-__global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
+__global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
     const bf16_t* __restrict__ q, const int32_t* __restrict__ cu_q, const bf16_t* __restrict__ k,
     const bf16_t* __restrict__ v, const int64_t* __restrict__ kv_off, const int32_t* __restrict__ kv_len, int32_t B,
     int32_t Hq, int32_t Hkv, float scale_log2e, int32_t causal, bf16_t* __restrict__ out, int32_t n_split,
     int32_t split_keys, float* __restrict__ part_ml, float* __restrict__ part_acc) {
   constexpr int kTokPerWave = 32 / G;
-  constexpr int kTokPerBlock = kFlashWaves * kTokPerWave;
-  __shared__ __align__(16) char lds_k[kKeysPerTile * kTileStride];
-  __shared__ __align__(16) char lds_v[kHeadDim * kVtStride];
+  constexpr int kTokPerBlock = kWaves * kTokPerWave;
+  constexpr int kLoads = kKeysPerTile * 16 / (kWaves * 64);   // 16-byte pieces of a K (or V) tile per thread
+  extern __shared__ __align__(16) char lds[];                  // 2 x [K tile | V tile]
+  constexpr int kVOffset = kKeysPerTile * kTileStride;
 
   // which (sample, token block) is this workgroup?  B is small; the scan is uniform.
   int blk = blockIdx.x, b = 0;
@@ -104,85 +135,62 @@ __global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
 #pragma unroll
   for (int x = 32; x > 0; x >>= 1) wave_min_limit = min(wave_min_limit, __shfl_xor(wave_min_limit, x));
 
-  uint4 rk[4], rv[4];
-  auto gload = [&](int t) {
+  uint4 rk[kLoads], rv[kLoads];
+  // Tile loads through buffer resources rebuilt per tile (scalar work only): the extent covers the tile's valid
+  // keys, so rows past the last key read as zero in hardware and a thread's offset never changes.
+  const int row_bytes = row_elems * 2;
+  const int voff0 = (tid >> 4) * row_bytes + (tid & 15) * 16;
+  auto gload_one = [&](const bf16_t* src, uint4 (&r)[kLoads], int t) {
+    const int rows = min(kKeysPerTile, kmax - t * kKeysPerTile);
+    const char* at = reinterpret_cast<const char*>(src) + ((base + (int64_t)t * kKeysPerTile) * row_elems + g * kHeadDim) * 2;
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(at), 0, max(0, (rows - 1) * row_bytes + 2 * kHeadDim), 0x00020000);   // 0 when no row is left
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int vv = tid + i * kFlashWaves * 64;
-      const int key = t * kKeysPerTile + (vv >> 4), dvec = vv & 15;
-      if (key < kmax) {
-        const int64_t off = (base + key) * row_elems + g * kHeadDim + dvec * 8;
-        rk[i] = *reinterpret_cast<const uint4*>(k + off);
-        rv[i] = *reinterpret_cast<const uint4*>(v + off);
-      } else {
-        rk[i] = make_uint4(0, 0, 0, 0);
-        rv[i] = make_uint4(0, 0, 0, 0);
-      }
+    for (int i = 0; i < kLoads; ++i)
+      r[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff0 + i * (kWaves * 4) * row_bytes, 0, 0));
+  };
+  auto store_k = [&](int slot) {
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) {
+      const int vv = tid + i * kWaves * 64;
+      *reinterpret_cast<uint4*>(lds + slot * kStageBytes + (vv >> 4) * kTileStride + (vv & 15) * 16) = rk[i];
     }
   };
-  auto lstore = [&]() {
+  auto store_v = [&](int slot) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int vv = tid + i * kFlashWaves * 64;
-      const int at = (vv >> 4) * kTileStride + (vv & 15) * 16;
-      *reinterpret_cast<uint4*>(lds_k + at) = rk[i];
-      const int key = vv >> 4, d0 = (vv & 15) * 8;
-      const uint32_t w[4] = {rv[i].x, rv[i].y, rv[i].z, rv[i].w};
-#pragma unroll
-      for (int e = 0; e < 8; ++e)
-        *reinterpret_cast<bf16_t*>(lds_v + (d0 + e) * kVtStride + vt_pos(key, d0 + e) * 2) =
-            (bf16_t)(w[e >> 1] >> (16 * (e & 1)));
+    for (int i = 0; i < kLoads; ++i) {
+      const int vv = tid + i * kWaves * 64;
+      *reinterpret_cast<uint4*>(lds + slot * kStageBytes + kVOffset + (vv >> 4) * kVStride + (vv & 15) * 16) = rv[i];
     }
   };
+  const char* k_lane = lds + col * kTileStride + half * 16;
+  const char* v_lane = lds + kVOffset + (4 * half + ((lane & 15) >> 2)) * kVStride + (lane & 16) * 2 + (lane & 3) * 8;
 
-  if (first_tile < n_tiles) gload(first_tile);
-  for (int t = first_tile; t < n_tiles; ++t) {
-    __syncthreads();                 // everyone is done reading the previous tile
-    lstore();
-    __syncthreads();
-    if (t + 1 < n_tiles) gload(t + 1);
-
-    // S^T = K . Q^T for the tile's two blocks of 32 keys
-    floatx16_t s[2];
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) s[rb][e] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks)
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb) {
-        const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(lds_k + (rb * 32 + col) * kTileStride + ks * 32 + half * 16);
-        s[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], s[rb], 0, 0, 0);
-      }
-
-    // online softmax of this lane's column; element e of block rb is key 64 t + 32 rb + 8 (e / 4) + 4 half + e % 4
+  auto step = [&](int t, floatx16_t (&sc)[2], floatx16_t (&sn)[2]) {
+    const int slot = (t - first_tile) & 1;
+    // (A) mask, column maximum
     const int key_base = t * kKeysPerTile + 4 * half;
-    // (the maximum is taken over the raw dot products and scaled once: scale > 0; the scale itself is folded
-    //  into the exponent's argument with one fma per element further down)
     float mx_raw = -INFINITY;
-    if ((t + 1) * kKeysPerTile <= wave_min_limit) {    // interior tile: every key visible to every column
+    if ((t + 1) * kKeysPerTile <= wave_min_limit) {
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) mx_raw = fmaxf(mx_raw, s[rb][e]);
+        for (int e = 0; e < 16; ++e) mx_raw = fmaxf(mx_raw, sc[rb][e]);
     } else {
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
           const int key = key_base + 32 * rb + 8 * (e >> 2) + (e & 3);
-          const float x = key < limit ? s[rb][e] : -INFINITY;
-          s[rb][e] = x;
+          const float x = key < limit ? sc[rb][e] : -INFINITY;
+          sc[rb][e] = x;
           mx_raw = fmaxf(mx_raw, x);
         }
     }
     float mx = fmaxf(m, mx_raw * scale_log2e);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
-    const bool none = mx == -INFINITY;                 // nothing visible to this column so far
-    // Lazy rescaling: keep the old reference maximum while the new one is at most 2^6 above it; the
-    // probabilities are then at most 64 (exact in bf16's range) and the accumulators are untouched.
-    // The decision is wave-uniform so the 64 accumulator multiplies are skipped as a block.
+    mx = half_wave_max(mx);
+    const bool none = mx == -INFINITY;
+    // (B) lazy rescaling, as in the plain loop
     const bool grow = !none && mx > m + 6.0f;
     if (__any(grow)) {
       const float mref = none ? m : mx;
@@ -194,33 +202,119 @@ __global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
         for (int e = 0; e < 16; ++e) o[d][e] *= alpha;
       m = mref;
     }
-    const float neg_m = none ? 0.f : -m;               // nothing visible yet: every score is -inf, keep the argument -inf
+    const float neg_m = none ? 0.f : -m;
+    // (C) scores of tile t + 1 next to the exponentials of tile t (the K slot holds zeros past the last tile)
+    const char* kn = k_lane + (slot ^ 1) * kStageBytes;
     float psum = 0.f;
     bf16x8_t pf[2][2];
+    bf16x8_t kf[3][2];                      // K operands, fetched two steps ahead of their products
 #pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
+    for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-      for (int e = 0; e < 16; ++e) {
-        const float p = fast_exp2(fmaf(s[rb][e], scale_log2e, neg_m));     // -inf (masked) -> 0
-        psum += p;
-        pf[rb][e >> 3][e & 7] = (__bf16)p;
+      for (int rb = 0; rb < 2; ++rb)
+        kf[ks][rb] = *reinterpret_cast<const bf16x8_t*>(kn + rb * 32 * kTileStride + ks * 32);
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      if (ks + 2 < 8) {
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+          kf[(ks + 2) % 3][rb] = *reinterpret_cast<const bf16x8_t*>(kn + rb * 32 * kTileStride + (ks + 2) * 32);
       }
-    psum += __shfl_xor(psum, 32);
-    l += psum;
-
-    // O^T += V^T . P^T: the k slots of step (rb, j) are the keys this lane's P values belong to
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
+        if (ks == 0) {
+          floatx16_t z;
+#pragma unroll
+          for (int e = 0; e < 16; ++e) z[e] = 0.f;
+          sn[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0][rb], qf[0], z, 0, 0, 0);
+        } else {
+          sn[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks % 3][rb], qf[ks], sn[rb], 0, 0, 0);
+        }
+        // two of this tile's 32 probabilities per product
+        const int prb = ks >> 2, e0 = (ks & 3) * 4 + 2 * rb;
+        const float p0 = fast_exp2(fmaf(sc[prb][e0], scale_log2e, neg_m));
+        const float p1 = fast_exp2(fmaf(sc[prb][e0 + 1], scale_log2e, neg_m));
+        const uint32_t pk = pack_pair(p0, p1);
+        psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), psum, false);
+        pf[prb][e0 >> 3][e0 & 7] = __builtin_bit_cast(bf16x2_t, pk)[0];
+        pf[prb][e0 >> 3][(e0 & 7) + 1] = __builtin_bit_cast(bf16x2_t, pk)[1];
+      }
+    }
+    l += half_wave_sum(psum);
+    // (D) O^T += V^T . P^T from this tile's V slot; refill the slots that are free
+    const char* vt = v_lane + slot * kStageBytes;
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int d = 0; d < 4; ++d) {
-          const int dim = 32 * d + col;
-          const int pos = (32 * rb + 16 * j + 8 * half) ^ ((dim >> 4) << 3);      // 8 keys of this half, in slot order
-          const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(lds_v + dim * kVtStride + pos * 2);
+          const char* at = vt + (32 * rb + 16 * j) * kVStride + 64 * d;
+          const shortx4_t lo = lds_read_tr16(at), hi = lds_read_tr16(at + 8 * kVStride);
+          const bf16x8_t a = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
           o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[rb][j], o[d], 0, 0, 0);
         }
+    store_k(slot);           // K(t + 2): this slot's K was last read before the previous barrier
+    store_v(slot ^ 1);       // V(t + 1): that slot's V was last read before the previous barrier
+    gload_one(k, rk, t + 3);
+    gload_one(v, rv, t + 2);
+    // Issue order of the straight-line part above: every matrix product is followed by the LDS reads of operands
+    // two products ahead and by a share of the exponentials, so neither the reads' latency nor the VALU work
+    // leaves the matrix pipe idle; the tile stores and loads ride behind the last products.
+    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 12; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+      __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+    }
+    __syncthreads();
+  };
+
+  if (first_tile < n_tiles) {
+    gload_one(k, rk, first_tile);
+    gload_one(v, rv, first_tile);
+    store_k(0);
+    store_v(0);
+    gload_one(k, rk, first_tile + 1);
+    store_k(1);
+    gload_one(k, rk, first_tile + 2);
+    gload_one(v, rv, first_tile + 1);
+    __syncthreads();
+    floatx16_t s0[2], s1[2];
+#pragma unroll
+    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) s0[rb][e] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+      for (int rb = 0; rb < 2; ++rb) {
+        const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(k_lane + rb * 32 * kTileStride + ks * 32);
+        s0[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], s0[rb], 0, 0, 0);
       }
+    for (int t = first_tile; t < n_tiles; t += 2) {
+      step(t, s0, s1);
+      if (t + 1 < n_tiles) step(t + 1, s1, s0);
+    }
   }
 
   if constexpr (kSplit) {
@@ -250,6 +344,41 @@ __global__ __launch_bounds__(kFlashWaves * 64, 2) void flash_attn_kernel(
   }
 }
 
+template <int G, bool kSplit>
+int flash_launch_g(const void* q, const int32_t* cu_q, const void* k, const void* v, const int64_t* kv_off,
+                   const int32_t* kv_len, int32_t B, int32_t total_q, int32_t Hq, int32_t Hkv, float scale,
+                   int32_t causal, void* out, SplitPlan plan, float* part_ml, float* part_acc, hipStream_t st) {
+  constexpr int kTokPerBlock = kWaves * 32 / G;
+  const int64_t blocks = ((int64_t)total_q + kTokPerBlock - 1) / kTokPerBlock + B;   // upper bound over ragged samples
+  MSA_REQUIRE(blocks < (int64_t)1 << 31, "flash attention: too many query rows");
+  dim3 grid((unsigned)blocks, (unsigned)Hkv, kSplit ? (unsigned)plan.n_split : 1u);
+  auto kern = flash_attn_kernel<G, kSplit>;
+  static bool attr_set = false;            // two tiles of K and V exceed the default dynamic LDS limit
+  if (!attr_set) {
+    MSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kLdsBytes));
+    attr_set = true;
+  }
+  kern<<<grid, kWaves * 64, kLdsBytes, st>>>(static_cast<const bf16_t*>(q), cu_q, static_cast<const bf16_t*>(k),
+                                             static_cast<const bf16_t*>(v), kv_off, kv_len, B, Hq, Hkv,
+                                             scale * 1.4426950408889634f, causal, static_cast<bf16_t*>(out),
+                                             kSplit ? plan.n_split : 1, kSplit ? plan.split_keys : 0, part_ml, part_acc);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
+
+template <bool kSplit, typename... Args>
+int flash_launch(int G, Args... args) {
+  switch (G) {
+    case 1: return flash_launch_g<1, kSplit>(args...);
+    case 2: return flash_launch_g<2, kSplit>(args...);
+    case 4: return flash_launch_g<4, kSplit>(args...);
+    case 8: return flash_launch_g<8, kSplit>(args...);
+  }
+  msa_set_error("flash attention: GQA group size %d unsupported (1, 2, 4, 8)", G);
+  return MSA_EINVAL;
+}
+
 }  // namespace
 
 extern "C" int msa_flash_attn(const void* q, const int32_t* cu_q, const void* k, const void* v, const int64_t* kv_off,
@@ -263,54 +392,13 @@ extern "C" int msa_flash_attn(const void* q, const int32_t* cu_q, const void* k,
   MSA_REQUIRE(scale > 0.f, "msa_flash_attn: scale must be positive");
   const int G = Hq / Hkv;
   MSA_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, "msa_flash_attn: GQA group size %d unsupported (1, 2, 4, 8)", G);
-  const int tok_per_block = kFlashWaves * 32 / G;
-  const int64_t blocks = ((int64_t)total_q + tok_per_block - 1) / tok_per_block + B;   // upper bound over ragged samples
-  MSA_REQUIRE(blocks < (int64_t)1 << 31, "msa_flash_attn: too many query rows");
-  dim3 grid((unsigned)blocks, (unsigned)Hkv);
-  const float sl2 = scale * 1.4426950408889634f;
-  hipStream_t st = as_stream(stream);
-#define MSA_FLASH_CASE(GG)                                                                                        \
-  case GG:                                                                                                        \
-    flash_attn_kernel<GG, false><<<grid, kFlashWaves * 64, 0, st>>>(                                              \
-        static_cast<const bf16_t*>(q), cu_q, static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v), kv_off, \
-        kv_len, B, Hq, Hkv, sl2, causal, static_cast<bf16_t*>(out), 1, 0, nullptr, nullptr);                      \
-    break;
-  switch (G) {
-    MSA_FLASH_CASE(1)
-    MSA_FLASH_CASE(2)
-    MSA_FLASH_CASE(4)
-    MSA_FLASH_CASE(8)
-  }
-#undef MSA_FLASH_CASE
-  MSA_LAUNCH_CHECK();
-  return MSA_OK;
+  return flash_launch<false>(G, q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale,
+                             causal, out, SplitPlan{1, 0}, (float*)nullptr, (float*)nullptr, as_stream(stream));
 }
 
 int flash_attn_split_launch(const void* q, const int32_t* cu_q, const void* k, const void* v, const int64_t* kv_off,
                             const int32_t* kv_len, int32_t B, int32_t total_q, int32_t Hq, int32_t Hkv, float scale,
                             int32_t causal, SplitPlan plan, float* part_ml, float* part_acc, hipStream_t st) {
-  const int G = Hq / Hkv;
-  const int tok_per_block = kFlashWaves * 32 / G;
-  const int64_t blocks = ((int64_t)total_q + tok_per_block - 1) / tok_per_block + B;   // upper bound over ragged samples
-  MSA_REQUIRE(blocks < (int64_t)1 << 31, "msa_sparse_attn: too many query rows");
-  dim3 grid((unsigned)blocks, (unsigned)Hkv, (unsigned)plan.n_split);
-  const float sl2 = scale * 1.4426950408889634f;
-#define MSA_FLASH_SPLIT_CASE(GG)                                                                                  \
-  case GG:                                                                                                        \
-    flash_attn_kernel<GG, true><<<grid, kFlashWaves * 64, 0, st>>>(                                               \
-        static_cast<const bf16_t*>(q), cu_q, static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v), kv_off, \
-        kv_len, B, Hq, Hkv, sl2, causal, nullptr, plan.n_split, plan.split_keys, part_ml, part_acc);              \
-    break;
-  switch (G) {
-    MSA_FLASH_SPLIT_CASE(1)
-    MSA_FLASH_SPLIT_CASE(2)
-    MSA_FLASH_SPLIT_CASE(4)
-    MSA_FLASH_SPLIT_CASE(8)
-    default:
-      msa_set_error("msa_sparse_attn: GQA group size %d unsupported (1, 2, 4, 8)", G);
-      return MSA_EINVAL;
-  }
-#undef MSA_FLASH_SPLIT_CASE
-  MSA_LAUNCH_CHECK();
-  return MSA_OK;
+  return flash_launch<true>(Hq / Hkv, q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq,
+                            Hkv, scale, causal, (void*)nullptr, plan, part_ml, part_acc, st);
 }

@@ -255,3 +255,41 @@ def test_rmsnorm_and_silu_mul_widths(ops, dtype, H):
     gu = torch.randn((N, 2 * H), generator=g).to(dtype)
     want = torch.nn.functional.silu(gu[:, :H].double()) * gu[:, H:].double()
     assert cf.rel_err(ops.silu_mul(gu.cuda()).cpu(), want) < tol
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 8), (16, 2)])
+@pytest.mark.parametrize("causal", [True, False])
+def test_flash_kernel_through_the_c_abi(ops, Hq, Hkv, causal):
+    """msa_flash_attn called directly (the host wrapper only picks it for large batches): every tile count parity of
+    its two-tile pipeline (1, 2, 3, 4, 7, 16 tiles of 64 keys), a sample without keys, a causal sample with more
+    query rows than keys (the leading rows see nothing and come out as zeros), single-row and ragged query blocks."""
+    say(f"flash kernel direct Hq={Hq} Hkv={Hkv} causal={causal}")
+    from msa_amd import _lib
+    D = 128
+    sq = [130, 1, 33, 64, 200, 5, 7, 40]
+    L = [400, 70, 33, 1000, 200, 192, 0, 10]
+    cu_q = np.concatenate([[0], np.cumsum(sq)])
+    cu_kv = np.concatenate([[0], np.cumsum(L)])
+    q = _randn((int(cu_q[-1]), Hq, D), 300, torch.bfloat16)
+    k = _randn((int(cu_kv[-1]), Hkv, D), 301, torch.bfloat16)
+    v = _randn((int(cu_kv[-1]), Hkv, D), 302, torch.bfloat16)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    kv_off = torch.as_tensor(cu_kv[:-1], dtype=torch.int64).cuda()
+    kv_len = torch.as_tensor(L, dtype=torch.int32).cuda()
+    cu_q_dev = torch.as_tensor(cu_q, dtype=torch.int32).cuda()
+    out = torch.full_like(qd, float("nan"))
+    lib = _lib.load()
+    _lib.check(lib.msa_flash_attn(_lib.ptr(qd), _lib.ptr(cu_q_dev), _lib.ptr(kd), _lib.ptr(vd), _lib.ptr(kv_off),
+                                  _lib.ptr(kv_len), len(sq), int(cu_q[-1]), Hq, Hkv, D, D ** -0.5, int(causal),
+                                  _lib.ptr(out), torch.cuda.current_stream().cuda_stream), "msa_flash_attn")
+    torch.cuda.synchronize()
+    out = out.cpu()
+    assert not torch.isnan(out).any()
+    for b in range(len(sq)):
+        rows = slice(int(cu_q[b]), int(cu_q[b + 1]))
+        keys = slice(int(cu_kv[b]), int(cu_kv[b + 1]))
+        blind = sq[b] if L[b] == 0 else (max(0, sq[b] - L[b]) if causal else 0)     # leading rows that see no key
+        assert (out[rows][:blind] == 0).all()
+        if blind < sq[b]:
+            want = cf.attention(q[rows][blind:], k[keys], v[keys], causal=causal)
+            assert cf.rel_err(out[rows][blind:], want) < 1e-2, (b, sq[b], L[b])

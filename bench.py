@@ -32,7 +32,7 @@ HQ, HKV, D, P, TOPK = 32, 8, 128, 64, 16
 # Bytes past L2 per launch of the scoring kernel at the default workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a plain 1 GiB device copy
 # (FETCH_SIZE x2.0, WRITE_SIZE x1.0); see profiles/score_gemm_c4_100M_bank.txt.
-SCORE_TRAFFIC_DEFAULT_WORKLOAD = (2.0 * 4_904_568 + 1.0 * 122_269) * 1024
+SCORE_TRAFFIC_DEFAULT_WORKLOAD = (2.0 * 3_354_966 + 1.0 * 122_269) * 1024
 
 
 def log(msg):

@@ -9,6 +9,7 @@
 // inside a unit is permuted the same way on both operands, which a dot product does not see.  A workgroup owns R row groups and splits
 // K over its wavefronts; partial sums meet in LDS and are added in wavefront order (deterministic).
 #include <algorithm>
+#include <type_traits>
 
 #include "common.h"
 
@@ -46,7 +47,11 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_linear_kernel(
   constexpr int kUnitBytes = 64 * J;   // one unit = J vectors of 16 bytes per lane = 32 J elements of a row
   const int units = K / (32 * J);
   extern __shared__ __align__(16) float part[];   // [waves][R][64][4], then [waves][16] row sums of squares
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, waves = blockDim.x >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, waves = blockDim.x >> 6;
+  // the wavefront index as a scalar: every K offset below derives from it and rides in the scalar offset of the
+  // buffer loads, which must be provably uniform (a value the compiler takes for divergent costs a
+  // read-first-lane loop around every load)
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n_l = lane & 15, g = lane >> 4;
   const int n_base = blockIdx.x * (16 * R);
   const int64_t row_bytes = (int64_t)K * 2;
@@ -61,7 +66,8 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_linear_kernel(
   const int voff = n_l * (int)row_bytes + g * 16;
 
   // this wavefront's share of the K units
-  const int u0 = (int)((int64_t)units * wave / waves), u1 = (int)((int64_t)units * (wave + 1) / waves);
+  const int u0 = (int)((uint32_t)units * (uint32_t)wave / (uint32_t)waves);        // units * waves < 2^31: K is bounded by the host
+  const int u1 = (int)((uint32_t)units * (uint32_t)(wave + 1) / (uint32_t)waves);
 
   floatx4_t acc[R];
 #pragma unroll
@@ -179,6 +185,184 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_linear_kernel(
   }
 }
 
+// Streaming form for matrices with many row groups per compute unit (gate/up, LM head): a workgroup stays for the
+// whole launch.  Wavefront w owns the K slice [32 F w, 32 F (w + 1)) for every row group the workgroup visits and
+// keeps its x operands for that slice (with the RMSNorm weight folded in) in registers, so the activations are read
+// once per workgroup instead of once per row group, and far fewer workgroups have to be dispatched.  Work items are
+// pairs of row groups (32 weight rows; gate and up of the same 16 outputs for the silu epilogue), dealt round robin;
+// a step is one row group: its F weight vectors per lane are prefetched one step ahead, the partial sums meet in
+// a ring of four LDS buffers behind one barrier per step, and all threads share the work of adding them up (a fixed
+// tree) and storing the row group.  Launched with 16 wavefronts.
+template <int F, int kEpi, bool kNorm>
+__global__ __launch_bounds__(kMaxWaves * 64) void skinny_stream_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const bf16_t* __restrict__ residual,
+    const bf16_t* __restrict__ norm_w, float eps, bf16_t* __restrict__ y, int32_t M, int32_t N, int32_t K,
+    int64_t y_row_stride, int32_t n_items) {
+  extern __shared__ __align__(16) float part[];   // [4][waves][64][4] partial sums, then [waves][16] sums of squares
+  const int tid = threadIdx.x, lane = tid & 63, waves = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n_l = lane & 15, g = lane >> 4;
+  const int row_bytes = K * 2;
+  const int slice_off = wave * (F * 64);           // byte offset of this wavefront's K slice inside a row
+  const int voff = n_l * row_bytes + g * 16;
+  float* row_ssq = part + 4 * waves * 256;
+
+  // activations of the slice, once
+  const __amdgpu_buffer_rsrc_t rs_x = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(reinterpret_cast<const char*>(x)), 0, M * row_bytes, 0x00020000);
+  u32x4_t xf[F];
+#pragma unroll
+  for (int f = 0; f < F; ++f) xf[f] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, voff, slice_off + f * 64, 0);
+
+  // this workgroup's items: blockIdx.x, blockIdx.x + gridDim.x, ...; two steps (row groups) per item
+  const int my_items = n_items > (int)blockIdx.x ? (n_items - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+  const int n_steps = 2 * my_items;
+  auto group_of = [&](int s) { return 2 * ((int)blockIdx.x + (s >> 1) * (int)gridDim.x) + (s & 1); };
+  // Three register stages of weight operands, always indexed by compile-time constants: a step's loads are issued
+  // two steps ahead.  Every step issues its prefetch (an empty one past the end) and the step count is padded to a
+  // multiple of three, so the loop body is straight-line as far as memory instructions go and the wait counts the
+  // compiler derives are exact; with one stage less, the wait for a step's operands also covered the output store
+  // of the step before, i.e. a store round trip per step.
+  constexpr int kStages = 3;
+  u32x4_t fw[kStages][F];
+  auto load_w = [&](auto slot_tag, int s) {
+    constexpr int slot = decltype(slot_tag)::value;
+    const int gid = group_of(s);
+    // rows <= 0 for the missing second group of an odd tail and for the step past the last one (the prefetch is
+    // issued unconditionally so that the wait counts in the loop stay exact): an empty extent reads zeros and
+    // touches no memory.  The clamp compiles to a vector instruction; read-first-lane brings the extent back into a
+    // scalar register so that the descriptor stays scalar and the loads need no per-lane descriptor loop.
+    const int rows = s < n_steps ? min(16, N - gid * 16) : 0;
+    const int extent = __builtin_amdgcn_readfirstlane(max(0, rows) * row_bytes);
+    const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(reinterpret_cast<const char*>(w)) + (int64_t)gid * 16 * row_bytes, 0, extent, 0x00020000);
+#pragma unroll
+    for (int f = 0; f < F; ++f) fw[slot][f] = __builtin_amdgcn_raw_buffer_load_b128(rs_w, voff, slice_off + f * 64, 0);
+  };
+  load_w(std::integral_constant<int, 0>{}, 0);
+  load_w(std::integral_constant<int, 1>{}, 1);
+
+  if constexpr (kNorm) {
+    // RMSNorm folded in: the operand is bf16(x * norm_w); the row scale rsqrt(mean(x^2) + eps) commutes with the
+    // product and is applied to the fp32 sums when a row group is stored
+    const __amdgpu_buffer_rsrc_t rs_g = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(reinterpret_cast<const char*>(norm_w)), 0, row_bytes, 0x00020000);
+    float ssq = 0.f;
+#pragma unroll
+    for (int f = 0; f < F; ++f) {
+      const u32x4_t gf = __builtin_amdgcn_raw_buffer_load_b128(rs_g, g * 16, slice_off + f * 64, 0);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const float lo = bf16lo(xf[f][c]), hi = bf16hi(xf[f][c]);
+        ssq += lo * lo + hi * hi;
+        xf[f][c] = pack_rne(lo * bf16lo(gf[c]), hi * bf16hi(gf[c]));
+      }
+    }
+    ssq += __shfl_xor(ssq, 16);
+    ssq += __shfl_xor(ssq, 32);
+    if (g == 0) row_ssq[wave * 16 + n_l] = ssq;       // visible to everyone behind the first step's barrier
+  }
+
+  // Adding up a step's partial sums is shared by all 1024 threads, so that no wavefront falls behind the others at
+  // the next barrier: eight threads own a pair of neighbouring outputs (row o_m of x, columns o_n, o_n + 1 of the
+  // row group); each adds the partials of two wavefronts and the eight meet by three DPP exchanges (a fixed tree:
+  // results are reproducible).  A wavefront thus holds one output row of the group, and its store covers the row's
+  // 32 contiguous bytes in one instruction (a full memory sector; narrower pieces cost a read-modify-write).
+  const int pair = tid >> 3, sub = tid & 7;
+  const int o_m = pair >> 3, o_n = (pair & 7) * 2;
+  const int o_idx = ((o_m >> 2) * 16 + o_n) * 4 + (o_m & 3);          // float index of (o_m, o_n) in a partial row
+  float inv = 1.f;                                                  // RMSNorm scale of row o_m
+  bool have_inv = !kNorm;
+  auto sum_parts = [&](int s, float& v0, float& v1) {
+    const float* base = part + ((s & 3) * waves + 2 * sub) * 256 + o_idx;
+    v0 = base[0] + base[256];
+    v1 = base[4] + base[256 + 4];
+#pragma unroll
+    for (int x = 1; x < 8; x <<= 1) {
+      v0 += __shfl_xor(v0, x);
+      v1 += __shfl_xor(v1, x);
+    }
+  };
+  const bool pair_store = ((y_row_stride & 1) == 0) && ((reinterpret_cast<uintptr_t>(y) & 3) == 0);
+  auto store_pair = [&](int n, float a, float b) {          // columns n, n + 1 of row o_m
+    bf16_t* at = y + (int64_t)o_m * y_row_stride + n;
+    const int n_end = kEpi == kEpiSiluMul ? N / 2 : N;
+    if (pair_store && n + 1 < n_end) {
+      *reinterpret_cast<uint32_t*>(at) = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
+    } else {
+      if (n < n_end) at[0] = f32_to_bf16(a);
+      if (n + 1 < n_end) at[1] = f32_to_bf16(b);
+    }
+  };
+
+  auto step = [&](int s, auto slot_tag) {
+    constexpr int slot = decltype(slot_tag)::value;
+    load_w(std::integral_constant<int, (slot + 2) % kStages>{}, s + 2);
+    floatx4_t acc = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int f = 0; f < F; ++f)
+      acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_frag(xf[f]), as_frag(fw[slot][f]), acc, 0, 0, 0);
+    // acc[e] is y[m = 4 g + e][16 gid + n_l] over this wavefront's K slice
+    *reinterpret_cast<floatx4_t*>(part + ((s & 3) * waves + wave) * 256 + lane * 4) = acc;
+    __syncthreads();
+    if (s >= n_steps) return;                        // padding step
+    if (kEpi == kEpiSiluMul && !(s & 1)) return;     // gate rows: stored together with the up rows of the next step
+    if (!have_inv) {
+      float tot = 0.f;
+      for (int wv = 0; wv < waves; ++wv) tot += row_ssq[wv * 16 + o_m];
+      inv = rsqrtf(tot / (float)K + eps);
+      have_inv = true;
+    }
+    const int gid = group_of(s);
+    if constexpr (kEpi == kEpiSiluMul) {
+      // steps s - 1 and s are gate and up of the same 16 outputs
+      float g0, g1, u0, u1;
+      sum_parts(s - 1, g0, g1);
+      sum_parts(s, u0, u1);
+      if (sub != 0 || o_m >= M) return;
+      const float a0 = bf16_to_f32(f32_to_bf16(g0 * inv)), b0 = bf16_to_f32(f32_to_bf16(u0 * inv));
+      const float a1 = bf16_to_f32(f32_to_bf16(g1 * inv)), b1 = bf16_to_f32(f32_to_bf16(u1 * inv));
+      store_pair((gid >> 1) * 16 + o_n, a0 / (1.f + __expf(-a0)) * b0, a1 / (1.f + __expf(-a1)) * b1);
+    } else {
+      float v0, v1;
+      sum_parts(s, v0, v1);
+      const int n = gid * 16 + o_n;
+      if (sub != 0 || o_m >= M) return;
+      v0 *= inv;
+      v1 *= inv;
+      if (kEpi == kEpiResidual) {
+        const bf16_t* r = residual + (int64_t)o_m * y_row_stride + n;
+        if (n < N) v0 = bf16_to_f32(f32_to_bf16(v0)) + bf16_to_f32(r[0]);
+        if (n + 1 < N) v1 = bf16_to_f32(f32_to_bf16(v1)) + bf16_to_f32(r[1]);
+      }
+      store_pair(n, v0, v1);
+    }
+  };
+  for (int s = 0; s < n_steps; s += kStages) {
+    step(s, std::integral_constant<int, 0>{});
+    step(s + 1, std::integral_constant<int, 1>{});
+    step(s + 2, std::integral_constant<int, 2>{});
+  }
+}
+
+template <int F, int kEpi, bool kNorm>
+int launch_stream(const void* x, const void* w, const void* residual, const void* norm_w, float eps, void* y, int32_t M,
+                  int32_t N, int32_t K, int waves, int grid, int n_items, hipStream_t st) {
+  const size_t lds = (size_t)waves * (4 * 256 + 16) * sizeof(float);
+  const int64_t y_stride = kEpi == kEpiSiluMul ? N / 2 : N;
+  static bool attr_set = false;              // 16 wavefronts need 65 KB, just past the default dynamic LDS limit
+  if (!attr_set) {
+    MSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_stream_kernel<F, kEpi, kNorm>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, kMaxWaves * (4 * 256 + 16) * (int)sizeof(float)));
+    attr_set = true;
+  }
+  skinny_stream_kernel<F, kEpi, kNorm><<<grid, waves * 64, lds, st>>>(
+      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<const bf16_t*>(residual),
+      static_cast<const bf16_t*>(norm_w), eps, static_cast<bf16_t*>(y), M, N, K, y_stride, n_items);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
+
 template <int R, int kEpi, bool kNorm>
 int launch(const void* x, const void* w, const void* residual, const void* norm_w, float eps, void* y, int32_t M,
            int32_t N, int32_t K, int waves, hipStream_t st) {
@@ -211,6 +395,26 @@ extern "C" int msa_skinny_linear(const void* x, const void* w, const void* resid
   const int units = K / kUnit;
   MSA_REQUIRE(norm_w == nullptr || eps > 0.f, "msa_skinny_linear: folded RMSNorm needs eps > 0");
   hipStream_t st = as_stream(stream);
+
+  // Many row groups per compute unit and a K that 16 wavefronts split into 5 MFMA steps each (K = 2560): the
+  // streaming kernel, one workgroup per compute unit at most, an equal number of items (32 rows) each.
+  static const int env_stream = [] { const char* e = getenv("MSA_LINEAR_STREAM"); return e ? atoi(e) : 1; }();
+  if (K == 16 * 5 * 32 && env_stream != 0) {
+    const int n_items = (N + 31) / 32;
+    const int iters = (n_items + 255) / 256;
+    const int grid = (n_items + iters - 1) / iters;
+    if (iters >= 2) {                                // with one item per workgroup the plain kernel does the same work
+#define MSA_STREAM(E_)                                                                                              \
+  (norm_w ? launch_stream<5, E_, true>(x, w, residual, norm_w, eps, y, M, N, K, kMaxWaves, grid, n_items, st)       \
+          : launch_stream<5, E_, false>(x, w, residual, norm_w, eps, y, M, N, K, kMaxWaves, grid, n_items, st))
+      switch (epilogue) {
+        case kEpiPlain: return MSA_STREAM(kEpiPlain);
+        case kEpiResidual: return MSA_STREAM(kEpiResidual);
+        case kEpiSiluMul: return MSA_STREAM(kEpiSiluMul);
+      }
+#undef MSA_STREAM
+    }
+  }
 
   // Wavefronts per workgroup: split K far enough that the launch has a few thousand wavefronts, and
   // prefer a count that divides the K units so every wavefront streams the same number of bytes.

@@ -138,6 +138,7 @@ def test_error_codes(ops):
 # weight-streaming linear layer of the decode step
 # ---------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("M,N,K", [(1, 48, 128), (5, 500, 256), (16, 2560, 4096), (16, 6144, 2560), (7, 2560, 9728),
+                                   (16, 16400, 2560), (3, 8210, 2560), (16, 20000, 2560),
                                    (16, 20, 384)])
 def test_skinny_linear_plain_and_residual(ops, M, N, K):
     say(f"skinny_linear M={M} N={N} K={K}")
@@ -154,7 +155,7 @@ def test_skinny_linear_plain_and_residual(ops, M, N, K):
     assert torch.equal(ops.skinny_linear(x.cuda(), w.cuda()).cpu(), got)
 
 
-@pytest.mark.parametrize("M,I,K", [(16, 9728, 2560), (3, 64, 256), (16, 528, 1024)])
+@pytest.mark.parametrize("M,I,K", [(16, 9728, 2560), (3, 64, 256), (16, 528, 1024), (7, 8208, 2560), (16, 4112, 2560)])
 def test_skinny_linear_norm_and_silu_mul(ops, M, I, K):
     say(f"skinny_linear norm + silu-mul M={M} I={I} K={K}")
     g = torch.Generator().manual_seed(I + K)

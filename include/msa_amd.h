@@ -218,6 +218,17 @@ int msa_rmsnorm(const void* x, void* residual, const void* weight, int32_t dtype
                 int32_t H, float eps, void* out, void* stream);
 int msa_silu_mul(const void* gate_up, int32_t dtype, int64_t N, int32_t I, void* out, void* stream);
 
+/* Greedy sampling of a decode step in place of `logits.argmax(-1)` and the token bookkeeping that follows it
+ * in the generation loops (src/msa/generate.py:102-105, :190-259: next token = argmax of the last position, position
+ * += 1, token appended to the output): tok[b] = index of the largest of logits[b, 0..V) (the smallest index among
+ * equal values; a NaN with a clear sign bit ranks above +inf, as in torch.argmax); pos[b] += 1 if pos is given; if
+ * out / col are given, out[b, col[b]] = tok[b] when 0 <= col[b] < max_new, then col[b] += 1.  `scratch` holds
+ * B * 32 64-bit words.  Two launches, no host synchronisation, safe to capture in a HIP graph. */
+#define MSA_GREEDY_SCRATCH_WORDS_PER_ROW 32
+int msa_greedy_sample(const void* logits, int32_t dtype, int32_t B, int64_t V, void* scratch, int64_t* tok,
+                      int64_t* pos, int64_t* out, int64_t out_stride, int64_t* col, int32_t max_new,
+                      void* stream);
+
 /* Linear layer for the few rows of a decode step: y[M, N] = x[M, K] . w[N, K]^T, bf16, M <= 16,
  * K a multiple of 128, w in torch.nn.Linear layout (the F.linear calls behind q/k/v/o_proj and the MLP at
  * src/msa/memory_sparse_attention.py:125-127, 405 when one token per sample is decoded).  The weight matrix is

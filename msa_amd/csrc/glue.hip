@@ -208,6 +208,73 @@ __global__ void silu_mul_kernel(const T* __restrict__ gate_up, int64_t N, int32_
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Greedy sampling of a decode step: row-wise argmax of the logits and the token bookkeeping around it in two
+// launches (partial maxima over slices of a row, then one thread per row).  A candidate is the 64-bit key
+// (order-preserving bits of the value) << 32 | (0xffffffff - index): the largest key is the largest value and,
+// among equal values, the smallest index.
+// ------------------------------------------------------------------------------------------------
+constexpr int kArgmaxSplits = 32;
+
+template <typename T>
+__device__ __forceinline__ uint32_t sortable_bits(T v);
+template <>
+__device__ __forceinline__ uint32_t sortable_bits<bf16_t>(bf16_t v) {
+  const uint32_t b = (uint32_t)v << 16;
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+template <>
+__device__ __forceinline__ uint32_t sortable_bits<float>(float v) {
+  const uint32_t b = __float_as_uint(v);
+  return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const T* __restrict__ logits, int64_t V,
+                                                             unsigned long long* __restrict__ partial) {
+  const int row = blockIdx.x, split = blockIdx.y;
+  const int64_t per = (V + kArgmaxSplits - 1) / kArgmaxSplits;
+  const int64_t lo = split * per, hi = min(V, lo + per);
+  const T* x = logits + (int64_t)row * V;
+  unsigned long long best = 0;
+  for (int64_t i = lo + threadIdx.x; i < hi; i += blockDim.x) {
+    const unsigned long long cand = ((unsigned long long)sortable_bits<T>(x[i]) << 32) | (0xffffffffu - (uint32_t)i);
+    best = cand > best ? cand : best;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const unsigned long long other = __shfl_xor(best, off);
+    best = other > best ? other : best;
+  }
+  __shared__ unsigned long long wave_best[4];
+  if ((threadIdx.x & 63) == 0) wave_best[threadIdx.x >> 6] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) best = wave_best[w] > best ? wave_best[w] : best;
+    partial[(int64_t)row * kArgmaxSplits + split] = best;
+  }
+}
+
+__global__ void greedy_commit_kernel(const unsigned long long* __restrict__ partial, int32_t B, int64_t* __restrict__ tok,
+                                     int64_t* __restrict__ pos, int64_t* __restrict__ out, int64_t out_stride,
+                                     int64_t* __restrict__ col, int32_t max_new) {
+  const int b = blockIdx.x * blockDim.x + threadIdx.x;
+  if (b >= B) return;
+  unsigned long long best = 0;
+  for (int s = 0; s < kArgmaxSplits; ++s) {
+    const unsigned long long c = partial[(int64_t)b * kArgmaxSplits + s];
+    best = c > best ? c : best;
+  }
+  const int64_t idx = (int64_t)(0xffffffffu - (uint32_t)(best & 0xffffffffu));
+  tok[b] = idx;
+  if (pos) pos[b] += 1;
+  if (out) {
+    const int64_t c = col[b];
+    if (c >= 0 && c < max_new) out[(int64_t)b * out_stride + c] = idx;
+    col[b] = c + 1;
+  }
+}
+
 }  // namespace
 
 static int qk_norm_rope_launch(const char* who, const void* q, const void* k, const void* v, int64_t q_row_stride,
@@ -293,6 +360,29 @@ extern "C" int msa_silu_mul(const void* gate_up, int32_t dtype, int64_t N, int32
     silu_mul_kernel<bf16_t><<<grid, 256, 0, as_stream(stream)>>>((const bf16_t*)gate_up, N, I, (bf16_t*)out, vec);
   else
     silu_mul_kernel<float><<<grid, 256, 0, as_stream(stream)>>>((const float*)gate_up, N, I, (float*)out, vec);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
+
+extern "C" int msa_greedy_sample(const void* logits, int32_t dtype, int32_t B, int64_t V, void* scratch, int64_t* tok,
+                                 int64_t* pos, int64_t* out, int64_t out_stride, int64_t* col, int32_t max_new,
+                                 void* stream) {
+  MSA_REQUIRE(logits && scratch && tok, "msa_greedy_sample: null pointer");
+  MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "msa_greedy_sample: dtype %d", dtype);
+  MSA_REQUIRE(B > 0 && B <= 65535 && V > 0 && V < ((int64_t)1 << 32), "msa_greedy_sample: B=%d V=%lld", B, (long long)V);
+  MSA_REQUIRE((out == nullptr) == (col == nullptr), "msa_greedy_sample: out and col go together");
+  hipStream_t st = as_stream(stream);
+  dim3 grid((unsigned)B, kArgmaxSplits);
+  if (dtype == MSA_BF16) {
+    argmax_partial_kernel<bf16_t><<<grid, 256, 0, st>>>(static_cast<const bf16_t*>(logits), V,
+                                                        static_cast<unsigned long long*>(scratch));
+  } else {
+    argmax_partial_kernel<float><<<grid, 256, 0, st>>>(static_cast<const float*>(logits), V,
+                                                       static_cast<unsigned long long*>(scratch));
+  }
+  MSA_LAUNCH_CHECK();
+  greedy_commit_kernel<<<(B + 63) / 64, 64, 0, st>>>(static_cast<const unsigned long long*>(scratch), B, tok, pos, out,
+                                                     out_stride, col, max_new);
   MSA_LAUNCH_CHECK();
   return MSA_OK;
 }

@@ -183,6 +183,10 @@ class MSAForCausalLM(nn.Module):
         fold_head = (dev.type == "cuda" and self.lm_head.weight.dtype == torch.bfloat16 and B <= ops.SKINNY_MAX_ROWS
                      and cfg.hidden_size % 128 == 0 and self.lm_head.bias is None)
 
+        native_sample = (dev.type == "cuda" and tok_buf.is_contiguous() and pos_buf.is_contiguous()
+                         and pos_buf.dtype == torch.int64 and pos_buf.numel() == B)
+        sample_scratch = torch.empty(B * 32, dtype=torch.int64, device=dev) if native_sample else None
+
         def step():
             # everything is in-place on fixed buffers so the same launches can be replayed as a graph
             if fold_head:                          # final norm folded into the weight-streaming LM head
@@ -191,6 +195,9 @@ class MSAForCausalLM(nn.Module):
                                            eps=self.model.norm.variance_epsilon).view(B, 1, -1)
             else:
                 logits = self.lm_head(self.model(tok_buf, ones, pos_buf, cache, gen_ids))
+            if native_sample:                      # argmax + token bookkeeping in two small launches
+                ops.greedy_sample(logits.view(B, -1), tok_buf, pos_buf, out_buf, col, sample_scratch)
+                return
             new_tok = logits.argmax(-1)
             tok_buf.copy_(new_tok)
             pos_buf.add_(1)

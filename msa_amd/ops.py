@@ -382,6 +382,28 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def greedy_sample(logits: torch.Tensor, tok: torch.Tensor, pos: Optional[torch.Tensor] = None,
+                  out: Optional[torch.Tensor] = None, col: Optional[torch.Tensor] = None,
+                  scratch: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Row-wise argmax of ``logits [B, V]`` written to ``tok`` (int64, ``B`` elements) with the bookkeeping of a
+    greedy decode step done in place: ``pos += 1``; ``out[b, col[b]] = tok[b]``; ``col += 1``.  Returns ``tok``."""
+    _need_cuda(logits, tok, pos, out, col)
+    B, V = logits.shape
+    if not logits.is_contiguous() or tok.dtype != torch.int64 or tok.numel() != B:
+        raise ValueError("logits must be contiguous [B, V] and tok int64 with B elements")
+    for t in (pos, col):
+        if t is not None and (t.dtype != torch.int64 or t.numel() != B or not t.is_contiguous()):
+            raise ValueError("pos / col must be contiguous int64 with B elements")
+    if (out is None) != (col is None) or (out is not None and (out.dtype != torch.int64 or out.stride(-1) != 1)):
+        raise ValueError("out [B, max_new] int64 and col go together")
+    if scratch is None:
+        scratch = torch.empty(B * 32, dtype=torch.int64, device=logits.device)
+    check(_lib.load().msa_greedy_sample(ptr(logits), dtype_code(logits.dtype), B, V, ptr(scratch), ptr(tok), ptr(pos),
+                                        ptr(out), out.stride(0) if out is not None else 0, ptr(col),
+                                        out.shape[1] if out is not None else 0, _stream()), "msa_greedy_sample")
+    return tok
+
+
 SKINNY_MAX_ROWS = 16
 
 

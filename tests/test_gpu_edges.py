@@ -294,3 +294,33 @@ def test_flash_kernel_through_the_c_abi(ops, Hq, Hkv, causal):
         if blind < sq[b]:
             want = cf.attention(q[rows][blind:], k[keys], v[keys], causal=causal)
             assert cf.rel_err(out[rows][blind:], want) < 1e-2, (b, sq[b], L[b])
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("B,V", [(16, 151936), (3, 1000), (1, 31), (5, 65)])
+def test_greedy_sample_against_argmax(ops, dtype, B, V):
+    """Row-wise argmax + the token bookkeeping of a decode step; ties go to the smallest index (bf16 logits of this
+    width tie often), -inf rows and the write window of `out` are covered."""
+    say(f"greedy_sample B={B} V={V} dtype={dtype}")
+    g = torch.Generator().manual_seed(B * 7 + V)
+    logits = torch.randn((B, V), generator=g).to(dtype)
+    if V > 40:
+        logits[0, 7] = logits[0, 33] = 100.0                   # a planted tie: the first index wins
+        logits[B - 1] = float("-inf")
+        logits[B - 1, V - 1] = -5.0                            # a single finite value at the very end
+    want = torch.stack([torch.nonzero(r == r.max())[0, 0] for r in logits.float()])     # first index of the maximum
+    dev = logits.cuda()
+    tok = torch.full((B, 1), -1, dtype=torch.int64, device="cuda")
+    pos = torch.arange(B, dtype=torch.int64, device="cuda").view(B, 1) * 10
+    out = torch.full((B, 3), -7, dtype=torch.int64, device="cuda")
+    col = torch.ones((B, 1), dtype=torch.int64, device="cuda")
+    for step in range(3):                                      # the third call finds col == 3 == max_new: no write
+        ops.greedy_sample(dev, tok, pos, out, col)
+    torch.cuda.synchronize()
+    assert tok.view(-1).cpu().tolist() == want.tolist()
+    assert pos.view(-1).cpu().tolist() == [10 * b + 3 for b in range(B)]
+    assert col.view(-1).cpu().tolist() == [4] * B
+    assert out.cpu()[:, 0].tolist() == [-7] * B and out.cpu()[:, 1].tolist() == want.tolist() == out.cpu()[:, 2].tolist()
+    tok2 = torch.empty(B, dtype=torch.int64, device="cuda")
+    ops.greedy_sample(dev, tok2)                               # argmax only
+    assert tok2.cpu().tolist() == want.tolist()

@@ -214,6 +214,18 @@ int msa_qk_norm_rope_append(const void* q, const void* k, const void* v, int64_t
                             const float* rope_cos, const float* rope_sin, int32_t rope_rows,
                             int32_t dtype, int32_t B, int32_t Hq, int32_t Hkv, int32_t D, void* q_out,
                             void* kcache, void* vcache, int32_t Lcap, int32_t* kv_len, void* stream);
+/* The decode step of src/msa/memory_sparse_attention.py:361-405 from the fused projection output to the attention
+ * output in two launches: q / k RMSNorm + rotary (:129-133), the cache update (:372-379) and GQA attention over
+ * [cache | new token] (:389-399) for one new token per sample.  qkv rows are [Hq q heads | Hkv k heads | Hkv v heads]
+ * (bf16, row stride in elements); kcache / vcache are [B, Lcap, Hkv, D]; kv_len[b] rows are valid on entry and
+ * kv_len[b] + 1 on return (a full cache drops the new row and the token attends to the cache only).  Groups of 4 or
+ * 8 query heads per KV head.  Workspace: msa_attn_workspace_bytes(B, Hq, Hkv, D, Lcap).  Same results as
+ * msa_qk_norm_rope_append followed by msa_sparse_attn up to the order of the fp32 sums. */
+int msa_decode_attn_fused(const void* qkv, int64_t row_stride, const int64_t* positions, const void* q_norm_w,
+                          const void* k_norm_w, float eps, const float* rope_cos, const float* rope_sin,
+                          int32_t rope_rows, int32_t B, int32_t Hq, int32_t Hkv, int32_t D, void* kcache,
+                          void* vcache, int32_t Lcap, int32_t* kv_len, float scale, void* out, void* workspace,
+                          size_t workspace_bytes, void* stream);
 int msa_rmsnorm(const void* x, void* residual, const void* weight, int32_t dtype, int64_t N,
                 int32_t H, float eps, void* out, void* stream);
 int msa_silu_mul(const void* gate_up, int32_t dtype, int64_t N, int32_t I, void* out, void* stream);

@@ -288,13 +288,183 @@ __global__ __launch_bounds__(kAttnWaves * 64) void attn_partial_kernel(
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Decode step with the q / k RMSNorm, the rotary embedding and the cache append folded into the attention launch
+// (bf16, one new token per sample, groups of 4 or 8 query heads).  Row b of `qkv` is the fused projection output
+// [Hq q heads | Hkv k heads | Hkv v heads].  Every workgroup (sample, KV head, split) normalises and rotates the q
+// heads of its group (16 lanes per head, 8 dims per lane, the same arithmetic as the stand-alone kernel) and shares
+// them through LDS; the workgroup of the last split also prepares the new token's k / v row of its KV head, writes it
+// to the cache at [b][kv_len[b]] and feeds it to its running softmax as one more key.  kv_len is only read here: the
+// combine kernel that follows advances it.  A full cache drops the new row (and the token then does not see itself).
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float row16_ror8(float v) {  // value of the lane 8 places away in the 16-lane row
+  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
+}
+
+// RMSNorm over the head's 128 dims (fp32) times the norm weight, then half-split rotary with the table row
+// cos_row / sin_row; `src` and `w` point at this lane's 8 elements; returns them packed to bf16.
+__device__ __forceinline__ uint4 norm_rope_8(const bf16_t* src, const bf16_t* w, float eps, const float* cos_row,
+                                             const float* sin_row, int j) {
+  const uint4 xr = *reinterpret_cast<const uint4*>(src), wr = *reinterpret_cast<const uint4*>(w);
+  const uint32_t xs[4] = {xr.x, xr.y, xr.z, xr.w}, ws[4] = {wr.x, wr.y, wr.z, wr.w};
+  float x[8], wt[8];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    x[2 * c] = bf16lo(xs[c]); x[2 * c + 1] = bf16hi(xs[c]);
+    wt[2 * c] = bf16lo(ws[c]); wt[2 * c + 1] = bf16hi(ws[c]);
+  }
+  float ssq = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) ssq += x[i] * x[i];
+  const float inv = rsqrtf(row16_allsum(ssq) * (1.0f / kHeadDim) + eps);
+  const int f = 8 * (j & 7);                    // frequency index of this lane's first element
+  float out[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float y = x[i] * inv * wt[i];
+    const float other = row16_ror8(y);          // the paired dim (d + 64 for j < 8, d - 64 for j >= 8)
+    const float c = cos_row[f + i], sn = sin_row[f + i];
+    out[i] = j < 8 ? y * c - other * sn : y * c + other * sn;
+  }
+  uint4 r;
+  r.x = pack_bf16x2(out[0], out[1]); r.y = pack_bf16x2(out[2], out[3]);
+  r.z = pack_bf16x2(out[4], out[5]); r.w = pack_bf16x2(out[6], out[7]);
+  return r;
+}
+
+template <int G>
+__global__ __launch_bounds__(8 * 64) void attn_decode_fused_kernel(
+    const bf16_t* __restrict__ qkv, int64_t row_stride, int32_t Hq, int32_t Hkv, const int64_t* __restrict__ pos,
+    const bf16_t* __restrict__ qw, const bf16_t* __restrict__ kw, float eps, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t, int32_t rope_rows, bf16_t* __restrict__ kcache, bf16_t* __restrict__ vcache,
+    int32_t Lcap, const int32_t* __restrict__ kv_len, float scale_log2e, int32_t n_split,
+    float* __restrict__ part_ml, float* __restrict__ part_acc) {
+  constexpr int kW = 8;
+  __shared__ float sm_m[kW][G], sm_l[kW][G];
+  __shared__ float sm_acc[kW][G][kHeadDim];
+  __shared__ uint4 sm_q[G][16];
+
+  const int b = blockIdx.x, g = blockIdx.y, split = blockIdx.z;
+  const int L_old = kv_len[b];
+  const bool has_new = L_old < Lcap;
+  const int per_split = (L_old + n_split - 1) / n_split;
+  const int key0 = split * per_split;
+  const int key1 = min(L_old, key0 + per_split);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int slot = lane >> 4, j = lane & 15;
+  const int row_elems = Hkv * kHeadDim;
+  const int64_t p = min((int64_t)max((int64_t)0, pos[b]), (int64_t)rope_rows - 1);
+  const float* cos_row = cos_t + p * 64;
+  const float* sin_row = sin_t + p * 64;
+  const bf16_t* row = qkv + (int64_t)b * row_stride;
+
+  // q heads of the group: head 4 wave + slot (wavefront 0, and wavefront 1 when G = 8)
+  const int hq = wave * 4 + slot;
+  if (hq < G) sm_q[hq][j] = norm_rope_8(row + (int64_t)(g * G + hq) * kHeadDim + 8 * j, qw + 8 * j, eps, cos_row, sin_row, j);
+  // the new token's key / value of this KV head: the last wavefront's first key slot, in the last split only
+  const bool owner = split == n_split - 1 && wave == kW - 1 && slot == 0 && has_new;
+  uint4 k_new = make_uint4(0, 0, 0, 0), v_new = k_new;
+  if (owner) {
+    k_new = norm_rope_8(row + (int64_t)(Hq + g) * kHeadDim + 8 * j, kw + 8 * j, eps, cos_row, sin_row, j);
+    v_new = *reinterpret_cast<const uint4*>(row + (int64_t)(Hq + Hkv + g) * kHeadDim + 8 * j);
+    const int64_t at = (((int64_t)b * Lcap + L_old) * Hkv + g) * kHeadDim + 8 * j;
+    *reinterpret_cast<uint4*>(kcache + at) = k_new;
+    *reinterpret_cast<uint4*>(vcache + at) = v_new;
+  }
+  __syncthreads();
+
+  float m[G], l[G], acc[G][8];
+  uint32_t qp[G][4];
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+    m[h] = -INFINITY; l[h] = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[h][i] = 0.f;
+    const uint4 w = sm_q[h][j];
+    qp[h][0] = w.x; qp[h][1] = w.y; qp[h][2] = w.z; qp[h][3] = w.w;
+  }
+  const int64_t lane_off = (int64_t)b * Lcap * row_elems + g * kHeadDim + 8 * j;     // this lane's slice of key 0
+  attend_keys_bf16<G>(kcache, vcache, lane_off, row_elems, key0 + wave * 4 + slot, key1, kW * 4, qp, scale_log2e, m, l, acc);
+  if (owner) {
+    // one more key, straight from registers; the probability is rounded to bf16 as in the paired products above
+    const uint32_t vs[4] = {v_new.x, v_new.y, v_new.z, v_new.w};
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      float d = dot2_bf16(qp[h][0], k_new.x, 0.f);
+      d = dot2_bf16(qp[h][1], k_new.y, d);
+      d = dot2_bf16(qp[h][2], k_new.z, d);
+      d = dot2_bf16(qp[h][3], k_new.w, d);
+      const float sc = row16_allsum(d) * scale_log2e;
+      const float mb = fmaxf(m[h], sc);
+      const float alpha = fast_exp2(m[h] - mb), pr = fast_exp2(sc - mb);
+      const float prb = bf16lo(pack_pair_rne(pr, 0.f));
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        acc[h][2 * c] = acc[h][2 * c] * alpha + prb * bf16lo(vs[c]);
+        acc[h][2 * c + 1] = acc[h][2 * c + 1] * alpha + prb * bf16hi(vs[c]);
+      }
+      l[h] = l[h] * alpha + pr;
+      m[h] = mb;
+    }
+  }
+
+  // merge the 4 key slots of the wavefront (lanes differing in bits 4 and 5)
+#pragma unroll
+  for (int h = 0; h < G; ++h) {
+#pragma unroll
+    for (int x = 16; x <= 32; x <<= 1) {
+      const float mo = __shfl_xor(m[h], x), lo = __shfl_xor(l[h], x);
+      const float mn = fmaxf(m[h], mo);
+      const float a = mn == -INFINITY ? 0.f : fast_exp2(m[h] - mn), bo = mn == -INFINITY ? 0.f : fast_exp2(mo - mn);
+      l[h] = l[h] * a + lo * bo;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[h][i] = acc[h][i] * a + __shfl_xor(acc[h][i], x) * bo;
+      m[h] = mn;
+    }
+  }
+  if (slot == 0) {
+#pragma unroll
+    for (int h = 0; h < G; ++h) {
+      if (j == 0) { sm_m[wave][h] = m[h]; sm_l[wave][h] = l[h]; }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sm_acc[wave][h][8 * j + i] = acc[h][i];
+    }
+  }
+  __syncthreads();
+  for (int idx = tid; idx < G * kHeadDim; idx += kW * 64) {
+    const int h = idx / kHeadDim, d = idx % kHeadDim;
+    float mn = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kW; ++w) mn = fmaxf(mn, sm_m[w][h]);
+    float lt = 0.f, at = 0.f;
+#pragma unroll
+    for (int w = 0; w < kW; ++w) {
+      const float a = mn == -INFINITY ? 0.f : fast_exp2(sm_m[w][h] - mn);
+      lt += sm_l[w][h] * a;
+      at += sm_acc[w][h][d] * a;
+    }
+    const int64_t o = ((int64_t)b * Hq + g * G + h) * n_split + split;
+    part_acc[o * kHeadDim + d] = at;
+    if (d == 0) { part_ml[o * 2] = mn; part_ml[o * 2 + 1] = lt; }
+  }
+}
+
 // One workgroup of 128 threads per (query row, head): merge the splits and normalise.
+// With `bump_len` (decode step whose attention kernel appended the new token's K / V row itself) the workgroup of
+// head 0 of row b also advances bump_len[b], unless the cache was full and the row was dropped.
 template <typename T>
 __global__ __launch_bounds__(kHeadDim) void attn_combine_kernel(const float* __restrict__ part_ml,
                                                                 const float* __restrict__ part_acc, int32_t n_split,
-                                                                T* __restrict__ out) {
+                                                                T* __restrict__ out, int32_t* __restrict__ bump_len = nullptr,
+                                                                int32_t Lcap = 0, int32_t Hq = 1) {
   const int64_t rh = blockIdx.x;   // row * Hq + head
   const int d = threadIdx.x;
+  if (bump_len != nullptr && d == 0 && rh % Hq == 0) {
+    const int64_t b = rh / Hq;
+    const int32_t len = bump_len[b];
+    if (len < Lcap) bump_len[b] = len + 1;
+  }
   float mn = -INFINITY;
   for (int s = 0; s < n_split; ++s) mn = fmaxf(mn, part_ml[(rh * n_split + s) * 2]);
   float lt = 0.f, at = 0.f;
@@ -394,4 +564,45 @@ extern "C" int msa_sparse_attn(const void* q, const int32_t* cu_q, const void* k
                                part_acc, st);
   return launch_attn<float>(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, plan, out, part_ml,
                             part_acc, st);
+}
+
+extern "C" int msa_decode_attn_fused(const void* qkv, int64_t row_stride, const int64_t* positions, const void* q_norm_w,
+                                     const void* k_norm_w, float eps, const float* rope_cos, const float* rope_sin,
+                                     int32_t rope_rows, int32_t B, int32_t Hq, int32_t Hkv, int32_t D, void* kcache,
+                                     void* vcache, int32_t Lcap, int32_t* kv_len, float scale, void* out,
+                                     void* workspace, size_t workspace_bytes, void* stream) {
+  MSA_REQUIRE(qkv && positions && q_norm_w && k_norm_w && rope_cos && rope_sin && kcache && vcache && kv_len && out &&
+                  workspace, "msa_decode_attn_fused: null pointer");
+  MSA_REQUIRE(D == kHeadDim, "msa_decode_attn_fused: head dim %d unsupported (need %d)", D, kHeadDim);
+  MSA_REQUIRE(B > 0 && Hkv > 0 && Hkv <= 65535 && Hq % Hkv == 0 && (Hq / Hkv == 4 || Hq / Hkv == 8),
+              "msa_decode_attn_fused: B=%d Hq=%d Hkv=%d (groups of 4 or 8 query heads)", B, Hq, Hkv);
+  MSA_REQUIRE(row_stride >= (int64_t)(Hq + 2 * Hkv) * D && row_stride % 8 == 0, "msa_decode_attn_fused: bad row stride");
+  MSA_REQUIRE((((uintptr_t)qkv | (uintptr_t)q_norm_w | (uintptr_t)k_norm_w | (uintptr_t)kcache | (uintptr_t)vcache) & 15) == 0,
+              "msa_decode_attn_fused: pointers must be 16-byte aligned");
+  MSA_REQUIRE(Lcap > 0 && rope_rows > 0 && eps > 0.f && scale > 0.f, "msa_decode_attn_fused: bad scalar argument");
+  const SplitPlan plan = plan_splits_valu(B, Hkv, Lcap);
+  const int n_split = plan.n_split;
+  const size_t need = msa_attn_workspace_bytes(B, Hq, Hkv, D, Lcap);
+  if (need > workspace_bytes) {
+    msa_set_error("msa_decode_attn_fused: workspace of %zu bytes, need %zu", workspace_bytes, need);
+    return MSA_ESIZE;
+  }
+  const size_t n = (size_t)B * Hq * n_split;
+  float* part_ml = static_cast<float*>(workspace);
+  float* part_acc = reinterpret_cast<float*>(static_cast<char*>(workspace) + align_up(n * 2 * sizeof(float), 256));
+  hipStream_t st = as_stream(stream);
+  dim3 grid((unsigned)B, (unsigned)Hkv, (unsigned)n_split);
+  const float sl2 = scale * 1.4426950408889634f;
+#define MSA_FUSED_CASE(GG)                                                                                           \
+  attn_decode_fused_kernel<GG><<<grid, 8 * 64, 0, st>>>(                                                            \
+      static_cast<const bf16_t*>(qkv), row_stride, Hq, Hkv, positions, static_cast<const bf16_t*>(q_norm_w),         \
+      static_cast<const bf16_t*>(k_norm_w), eps, rope_cos, rope_sin, rope_rows, static_cast<bf16_t*>(kcache),        \
+      static_cast<bf16_t*>(vcache), Lcap, kv_len, sl2, n_split, part_ml, part_acc)
+  if (Hq / Hkv == 4) MSA_FUSED_CASE(4); else MSA_FUSED_CASE(8);
+#undef MSA_FUSED_CASE
+  MSA_LAUNCH_CHECK();
+  attn_combine_kernel<bf16_t><<<(unsigned)((int64_t)B * Hq), kHeadDim, 0, st>>>(part_ml, part_acc, n_split,
+                                                                                static_cast<bf16_t*>(out), kv_len, Lcap, Hq);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
 }

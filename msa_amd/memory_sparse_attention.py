@@ -148,10 +148,16 @@ class MemorySparseAttention(nn.Module):
             raise ValueError("compact KV cache not found: did prefill stage 2 run?")
         qkv = ops.skinny_linear(residual, self._fused_weight(residual.device), norm_weight=norm_weight, eps=eps)
         kc, vc, kv_len = ck["compacked_key_cache"], ck["compacked_value_cache"], ck["kv_lengths"]
-        q = ops.qk_norm_rope_append(qkv, Hq, Hkv, D, position_ids.reshape(-1), self.q_norm.weight, self.k_norm.weight,
-                                    self.q_norm.variance_epsilon, self._rope_tables(residual.device), kc, vc, kv_len)
-        out = ops.sparse_attn(q.view(B, Hq, D), kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), ck["kv_offsets"], kv_len,
-                              ck["kv_capacity"], scale=self.scaling, causal=True)
+        if Hq // Hkv in (4, 8) and kc.dim() == 4 and kc.is_contiguous() and vc.is_contiguous():
+            # q / k norm + rotary + cache append folded into the attention launch
+            out = ops.decode_attn_fused(qkv, Hq, Hkv, D, position_ids.reshape(-1), self.q_norm.weight, self.k_norm.weight,
+                                        self.q_norm.variance_epsilon, self._rope_tables(residual.device), kc, vc, kv_len,
+                                        scale=self.scaling)
+        else:
+            q = ops.qk_norm_rope_append(qkv, Hq, Hkv, D, position_ids.reshape(-1), self.q_norm.weight, self.k_norm.weight,
+                                        self.q_norm.variance_epsilon, self._rope_tables(residual.device), kc, vc, kv_len)
+            out = ops.sparse_attn(q.view(B, Hq, D), kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), ck["kv_offsets"], kv_len,
+                                  ck["kv_capacity"], scale=self.scaling, causal=True)
         return ops.skinny_linear(out.view(B, Hq * D), self.o_proj.weight, residual=residual)
 
     def forward_with_kvcache_for_batch_parrallel(self, hidden_states, doc_ids, attention_mask=None,

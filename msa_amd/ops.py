@@ -382,6 +382,33 @@ def silu_mul(gate_up: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def decode_attn_fused(qkv: torch.Tensor, Hq: int, Hkv: int, D: int, positions: torch.Tensor, q_norm_w, k_norm_w,
+                      eps: float, rope: Tuple[torch.Tensor, torch.Tensor], kcache: torch.Tensor, vcache: torch.Tensor,
+                      kv_len: torch.Tensor, scale: Optional[float] = None) -> torch.Tensor:
+    """One decode step from the fused projection output ``qkv [B, (Hq + 2 Hkv) D]`` (bf16) to the attention output
+    ``[B, Hq, D]``: q / k norm + rotary, in-place append of the new K / V row to ``kcache / vcache [B, Lcap, Hkv, D]``
+    at ``kv_len`` (advanced by one) and attention over ``[cache | new token]``, in two launches."""
+    _need_cuda(qkv, positions, q_norm_w, k_norm_w, rope[0], rope[1], kcache, vcache, kv_len)
+    B, W = qkv.shape
+    if qkv.dtype != torch.bfloat16 or W != (Hq + 2 * Hkv) * D or positions.dtype != torch.int64 or positions.numel() != B:
+        raise ValueError("qkv must be bf16 [B, (Hq + 2 Hkv) D] and positions int64 [B]")
+    if kcache.shape != vcache.shape or kcache.dim() != 4 or kcache.shape[0] != B or tuple(kcache.shape[2:]) != (Hkv, D) \
+            or kcache.dtype != torch.bfloat16 or kv_len.dtype != torch.int32 or kv_len.numel() != B:
+        raise ValueError("caches must be bf16 [B, Lcap, Hkv, D] and kv_len int32 [B]")
+    Lcap = kcache.shape[1]
+    lib = _lib.load()
+    need = lib.msa_attn_workspace_bytes(B, Hq, Hkv, D, Lcap)
+    ws = _attn_ws.get(qkv.device)
+    if ws is None or ws.numel() < need:
+        ws = _attn_ws[qkv.device] = torch.empty(need, dtype=torch.uint8, device=qkv.device)
+    out = torch.empty((B, Hq, D), dtype=qkv.dtype, device=qkv.device)
+    check(lib.msa_decode_attn_fused(ptr(qkv), W, ptr(positions), ptr(q_norm_w), ptr(k_norm_w), eps, ptr(rope[0]),
+                                    ptr(rope[1]), rope[0].shape[0], B, Hq, Hkv, D, ptr(kcache), ptr(vcache), Lcap,
+                                    ptr(kv_len), D ** -0.5 if scale is None else scale, ptr(out), ptr(ws), ws.numel(),
+                                    _stream()), "msa_decode_attn_fused")
+    return out
+
+
 def greedy_sample(logits: torch.Tensor, tok: torch.Tensor, pos: Optional[torch.Tensor] = None,
                   out: Optional[torch.Tensor] = None, col: Optional[torch.Tensor] = None,
                   scratch: Optional[torch.Tensor] = None) -> torch.Tensor:

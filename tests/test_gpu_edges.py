@@ -211,6 +211,40 @@ def test_qk_norm_rope_append_equals_separate_kernels(ops):
     assert torch.equal(kc2[2], kc0[2]) and not torch.equal(kc2[0, 0], kc0[0, 0])
 
 
+@pytest.mark.parametrize("Hq,Hkv", [(8, 2), (32, 8), (16, 2)])
+def test_decode_attn_fused_equals_the_separate_launches(ops, Hq, Hkv):
+    """q / k norm + rotary + cache append + attention in one call against msa_qk_norm_rope_append followed by
+    msa_sparse_attn: identical cache rows and lengths, outputs equal up to the order of the fp32 sums, including an
+    empty cache (the token sees only itself), a full cache (the row is dropped) and lengths around the batch of 4
+    keys and the split of the key range."""
+    say(f"decode_attn_fused Hq={Hq} Hkv={Hkv}")
+    D, Lcap = 128, 700
+    lens = [0, 1, 3, 4, 5, 699, 700, 257, 512, 31]
+    B = len(lens)
+    g = torch.Generator().manual_seed(Hq * 100 + Hkv)
+    qkv = torch.randn((B, (Hq + 2 * Hkv) * D), generator=g).bfloat16().cuda()
+    pos = torch.tensor([3, 700, 0, 41, 9, 1023, 5000, 77, 512, 30], dtype=torch.int64).cuda()   # 5000 clamps to the table
+    qw, kw = (1 + 0.1 * torch.randn(D, generator=g)).bfloat16().cuda(), (1 + 0.1 * torch.randn(D, generator=g)).bfloat16().cuda()
+    rope = ops.rope_tables(1024, D, 1e6, device="cuda")
+    kc0 = torch.randn((B, Lcap, Hkv, D), generator=g).bfloat16().cuda()
+    vc0 = torch.randn((B, Lcap, Hkv, D), generator=g).bfloat16().cuda()
+    kc1, vc1, l1 = kc0.clone(), vc0.clone(), torch.tensor(lens, dtype=torch.int32).cuda()
+    q = ops.qk_norm_rope_append(qkv, Hq, Hkv, D, pos, qw, kw, 1e-6, rope, kc1, vc1, l1)
+    kv_off = torch.arange(B, dtype=torch.int64, device="cuda") * Lcap
+    want = ops.sparse_attn(q, kc1.view(-1, Hkv, D), vc1.view(-1, Hkv, D), kv_off, l1, Lcap, causal=True)
+    kc2, vc2, l2 = kc0.clone(), vc0.clone(), torch.tensor(lens, dtype=torch.int32).cuda()
+    got = ops.decode_attn_fused(qkv, Hq, Hkv, D, pos, qw, kw, 1e-6, rope, kc2, vc2, l2)
+    torch.cuda.synchronize()
+    assert l2.cpu().tolist() == l1.cpu().tolist() == [min(n + 1, Lcap) for n in lens]
+    assert torch.equal(kc2, kc1) and torch.equal(vc2, vc1)
+    assert cf.rel_err(got.cpu(), want.cpu()) < 2e-3
+    # and against the oracle from the raw projection output (sample 5: a long row; sample 0: the token alone)
+    for b in (0, 5, 9):
+        n = int(l2[b])
+        ref = cf.attention(q[b:b + 1].cpu(), kc2[b, :n].cpu(), vc2[b, :n].cpu(), causal=True)
+        assert cf.rel_err(got[b:b + 1].cpu(), ref) < 1e-2
+
+
 def test_cache_append_rows_ragged_and_clamped(ops):
     say("cache_append_rows: ragged blocks, empty block, capacity clamp")
     B, Lcap, Hkv, D = 4, 10, 2, 128

@@ -393,7 +393,7 @@ def main():
     # ---- bandwidth-bound regime: one query (and fewer tokens) per scan of layer 0
     sweep = []
     if not args.no_sweep:
-        for b1, s1 in ((1, 16), (1, 64), (1, 128), (2, 128), (4, 128)):
+        for b1, s1 in ((1, 1), (1, 16), (1, 64), (1, 128), (2, 128), (4, 128)):
             q1 = qs[0][:b1, :s1].contiguous()
             sc = torch.empty((b1, TOPK), dtype=torch.float32, device=dev)
             dc = torch.empty((b1, TOPK), dtype=torch.int32, device=dev)

@@ -177,6 +177,47 @@ def extra_decode(dev):
             "attention_only_tok_per_s_36_layers": round(B / (36 * ms) * 1e3)}
 
 
+def extra_decode_projections(dev):
+    """configs[4] projection share: the four weight-streaming linears of a decode layer and the LM head at B=16
+    (Qwen3-4B shapes, bf16), each replayed from a HIP graph over distinct weight copies so that neither the Python
+    launch cost nor the Infinity Cache flatter the number (a launch inside the graph costs about 4 us whatever its
+    work, which is most of the small matrices' distance from the HBM peak)."""
+    from msa_amd import ops
+    M, H, I, V = 16, 2560, 9728, 151936
+    g = torch.Generator(device=dev).manual_seed(14)
+    shapes = [("qkv (norm folded)", 6144, H, "norm"), ("o_proj (+residual)", H, 4096, "res"),
+              ("gate/up (norm, silu-mul)", 2 * I, H, "silu"), ("down_proj (+residual)", H, I, "res"),
+              ("lm_head (norm folded)", V, H, "norm")]
+    out = {}
+    for name, N, K, kind in shapes:
+        copies = 2 if N * K * 2 > (300 << 20) else 10
+        ws = [(torch.randn((N, K), generator=g, device=dev) * K ** -0.5).to(torch.bfloat16) for _ in range(copies)]
+        x = torch.randn((M, K), generator=g, device=dev).to(torch.bfloat16)
+        nw = torch.ones((K,), device=dev, dtype=torch.bfloat16)
+        res = torch.zeros((M, N), device=dev, dtype=torch.bfloat16)
+
+        def run():
+            for w in ws:
+                if kind == "norm":
+                    ops.skinny_linear(x, w, norm_weight=nw, eps=1e-6)
+                elif kind == "silu":
+                    ops.skinny_linear(x, w, silu_mul=True, norm_weight=nw, eps=1e-6)
+                else:
+                    ops.skinny_linear(x, w, residual=res)
+        run()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            run()
+        us = time_cuda(graph.replay, 5) * 1e3 / copies
+        by = N * K * 2
+        out[name] = {"N": N, "K": K, "us": round(us, 2), "GB/s": round(by / us / 1e3, 1),
+                     "frac_hbm": round(by / us / 1e3 / HBM_PEAK_GBS, 4)}
+        del ws
+    return {"workload": "configs[4] projection share: weight-streaming linears of one decode layer + LM head, B=16, bf16",
+            "kernels": out}
+
+
 def extra_routing_10m(dev):
     """configs[2]: router scoring + top-k on a 10M-token bank (about 156k chunks), batch 32 x 128 query tokens,
     top-16, one routed layer per call (the 18 layers of a model cost 18 of these)."""
@@ -425,7 +466,7 @@ def main():
     extras = None
     if not args.no_extras:
         extras = {"pooling": extra_pooling(dev), "routing_10M_bank": extra_routing_10m(dev), "decode_attention": extra_decode(dev),
-                  "prefill_attention": extra_prefill_attention(dev)}
+                  "prefill_attention": extra_prefill_attention(dev), "decode_projections": extra_decode_projections(dev)}
 
     cpu = None
     if not args.no_cpu_baseline:

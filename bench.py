@@ -171,10 +171,29 @@ def extra_decode(dev):
         ops.sparse_attn(q, kc.view(-1, HKV, D), vc.view(-1, HKV, D), kv_off, kv_len, Lcap)
     ms = time_cuda(step, 20)
     by = 2 * B * (L + 12) * HKV * D * 2        # mean context over the 22 steps run
+    # the form the end-to-end decode uses: q/k norm + rotary + append + attention from the fused projection output,
+    # replayed from a HIP graph (no Python launch cost between the two kernels)
+    kv_len.fill_(L)
+    qkv = torch.randn((B, (HQ + 2 * HKV) * D), generator=g, device=dev).to(torch.bfloat16)
+    pos = torch.full((B,), L, dtype=torch.int64, device=dev)
+    nw = torch.ones((D,), device=dev, dtype=torch.bfloat16)
+    rope = ops.rope_tables(8192, D, 1e6, device=dev)
+
+    def fused():
+        ops.decode_attn_fused(qkv, HQ, HKV, D, pos, nw, nw, 1e-6, rope, kc, vc, kv_len)
+    fused()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fused()
+    ms_fused = time_cuda(graph.replay, 20)
     return {"workload": "configs[4] attention share: 1 layer-step, B=16, L=4388, GQA 32/8, bf16",
             "ms_per_layer_step": round(ms, 4), "GB/s": round(by / ms / 1e6, 1),
             "frac_hbm": round(by / ms / 1e6 / HBM_PEAK_GBS, 4),
-            "attention_only_tok_per_s_36_layers": round(B / (36 * ms) * 1e3)}
+            "attention_only_tok_per_s_36_layers": round(B / (36 * ms) * 1e3),
+            "fused_norm_rope_append_attention_in_graph": {"ms_per_layer_step": round(ms_fused, 4),
+                                                          "GB/s": round(by / ms_fused / 1e6, 1),
+                                                          "frac_hbm": round(by / ms_fused / 1e6 / HBM_PEAK_GBS, 4)}}
 
 
 def extra_decode_projections(dev):

@@ -256,6 +256,14 @@ int msa_greedy_sample(const void* logits, int32_t dtype, int32_t B, int64_t V, v
 int msa_skinny_linear(const void* x, const void* w, const void* residual, const void* norm_w, float eps,
                       int32_t epilogue, int32_t dtype, int32_t M, int32_t N, int32_t K, void* y,
                       void* stream);
+/* The same call with a scratch buffer of msa_skinny_linear_workspace_bytes(M, N, K) bytes (0 when the shape has
+ * no use for one): matrices with few rows and a long K (down_proj) are then cut into row blocks x K slices whose
+ * fp32 partial sums meet in the workspace and are added in K order by a second launch, which cuts the activation
+ * bytes every compute unit re-reads.  With a NULL or too small workspace it is msa_skinny_linear. */
+size_t msa_skinny_linear_workspace_bytes(int32_t M, int32_t N, int32_t K);
+int msa_skinny_linear_ws(const void* x, const void* w, const void* residual, const void* norm_w, float eps,
+                         int32_t epilogue, int32_t dtype, int32_t M, int32_t N, int32_t K, void* y,
+                         void* workspace, size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

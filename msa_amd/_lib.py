@@ -52,6 +52,8 @@ SIGNATURES = {
                                         _i32, _vp, _f32, _vp, _vp, _sz, _vp]),
     "msa_greedy_sample": (C.c_int, [_vp, _i32, _i32, _i64, _vp, _vp, _vp, _vp, _i64, _vp, _i32, _vp]),
     "msa_skinny_linear": (C.c_int, [_vp, _vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _vp, _vp]),
+    "msa_skinny_linear_workspace_bytes": (_sz, [_i32, _i32, _i32]),
+    "msa_skinny_linear_ws": (C.c_int, [_vp, _vp, _vp, _vp, _f32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _sz, _vp]),
     "msa_sparse_attn": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _f32,
                                   _i32, _vp, _vp, _sz, _vp]),
 }

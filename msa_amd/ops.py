@@ -432,6 +432,7 @@ def greedy_sample(logits: torch.Tensor, tok: torch.Tensor, pos: Optional[torch.T
 
 
 SKINNY_MAX_ROWS = 16
+_linear_ws = {}
 
 
 def interleave_gate_up(gate_w: torch.Tensor, up_w: torch.Tensor) -> torch.Tensor:
@@ -461,7 +462,13 @@ def skinny_linear(x: torch.Tensor, w: torch.Tensor, residual: Optional[torch.Ten
     epi = 2 if silu_mul else (1 if residual is not None else 0)
     if norm_weight is not None and (norm_weight.shape != (K,) or norm_weight.dtype != x.dtype or not norm_weight.is_contiguous()):
         raise ValueError("skinny_linear: norm_weight must be a contiguous [K] tensor of x's dtype")
-    check(_lib.load().msa_skinny_linear(ptr(x), ptr(w), ptr(residual) if residual is not None else None,
-                                        ptr(norm_weight) if norm_weight is not None else None, float(eps), epi,
-                                        dtype_code(x.dtype), M, N, K, ptr(out), _stream()), "msa_skinny_linear")
+    lib = _lib.load()
+    need = lib.msa_skinny_linear_workspace_bytes(M, N, K)
+    ws = _linear_ws.get(x.device)
+    if need and (ws is None or ws.numel() < need):
+        ws = _linear_ws[x.device] = torch.empty(need, dtype=torch.uint8, device=x.device)
+    check(lib.msa_skinny_linear_ws(ptr(x), ptr(w), ptr(residual) if residual is not None else None,
+                                   ptr(norm_weight) if norm_weight is not None else None, float(eps), epi,
+                                   dtype_code(x.dtype), M, N, K, ptr(out), ptr(ws) if need else None,
+                                   ws.numel() if need else 0, _stream()), "msa_skinny_linear_ws")
     return out

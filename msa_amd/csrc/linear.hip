@@ -364,26 +364,35 @@ int launch_stream(const void* x, const void* w, const void* residual, const void
 }
 
 // ------------------------------------------------------------------------------------------------
-// Tiled form for matrices with few rows and a long K (down_proj: 2560 x 9728).  With one 16-row group per workgroup
-// every workgroup re-reads all of x, as many bytes as its weights, and a compute unit moves only about 34 GB/s
-// whatever the source; here the matrix is cut both ways, workgroup (row block, K slice) owns `gpw` row groups (one per
-// wavefront) over kslice elements of K, so it reads 16 / (16 gpw) of its weight bytes in activations.  The x slice is
-// staged once in LDS in operand order; a wavefront streams its 16 weight rows of the slice (up to twenty loads in flight per lane)
-// and stores its fp32 partial block; `skinny_tile_reduce_kernel` adds the K slices in order and applies the epilogue.
+// Tiled form for matrices with few rows and a long K (down_proj: 2560 x 9728): the matrix is cut both ways,
+// workgroup (row block, K slice) owns `gpw` row groups (one per wavefront) over a slice of K.  A compute unit moves
+// only about 34 GB/s whatever the source, so what counts is the weight plus activation bytes per compute unit and
+// that all compute units take part: with one 16-row group per workgroup every workgroup re-reads all of x, as many
+// bytes as its weights, and 160 row groups leave 96 compute units idle; a tile of ten row groups over a sixteenth of
+// K reads a tenth of its weight bytes in activations and there are 256 of them.  The x slice is staged once in LDS
+// in operand order; a wavefront streams its 16 weight rows of the slice (up to twenty loads in flight per lane) and
+// stores its fp32 partial block; `skinny_tile_reduce_kernel` adds the K slices in order and applies the epilogue.
+// K slices are runs of 32-element MFMA steps, as even as the step count allows.  (The same cut measured slower than
+// the other forms for the gate/up and q/k/v matrices, which have rows enough: 29.7 vs 28.0 and 15.7 vs 12.8 us.)
 // ------------------------------------------------------------------------------------------------
 constexpr int kTileDepth = 20;      // weight vectors in flight per lane
+constexpr int kTileMaxSlices = 16;
 
 __global__ __launch_bounds__(kMaxWaves * 64) void skinny_tile_partial_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, float* __restrict__ part, int32_t M, int32_t N, int32_t K,
-    int32_t gpw, int32_t kslice) {
+    int32_t gpw) {
   extern __shared__ __align__(16) u32x4_t xs[];     // [steps padded to kTileDepth][64] x operands of the K slice
   const int tid = threadIdx.x, lane = tid & 63, waves = blockDim.x >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n_l = lane & 15, g = lane >> 4;
   const int row_bytes = K * 2;
-  const int rb = blockIdx.x, ks = blockIdx.y;
-  const int steps = kslice / 32, steps_pad = (steps + kTileDepth - 1) / kTileDepth * kTileDepth;
-  const int slice_off = ks * kslice * 2;
+  const int rb = blockIdx.x, ks = blockIdx.y, n_slices = gridDim.y;
+  const int steps_total = K / 32;
+  const int s0 = (int)((int64_t)steps_total * ks / n_slices), s1 = (int)((int64_t)steps_total * (ks + 1) / n_slices);
+  const int steps = s1 - s0;
+  const int steps_max = (steps_total + n_slices - 1) / n_slices;
+  const int steps_pad = (steps_max + kTileDepth - 1) / kTileDepth * kTileDepth;    // the host sizes LDS with this
+  const int slice_off = s0 * 64;
   const int voff = n_l * row_bytes + g * 16;
   const int groups = (N + 15) >> 4;
 
@@ -400,7 +409,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_tile_partial_kernel(
   const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(reinterpret_cast<const char*>(w)) + (int64_t)gid * 16 * row_bytes, 0, extent, 0x00020000);
   floatx4_t acc = floatx4_t{0.f, 0.f, 0.f, 0.f};
-  for (int f0 = 0; f0 < steps_pad; f0 += kTileDepth) {
+  for (int f0 = 0; f0 < steps; f0 += kTileDepth) {
     u32x4_t fw[kTileDepth];
 #pragma unroll
     for (int i = 0; i < kTileDepth; ++i) {
@@ -418,20 +427,20 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_tile_partial_kernel(
 
 // One thread per output element in the order the partial blocks are stored (row group, lane, accumulator element),
 // so the reads of every K slice are contiguous; all slices are loaded first and added in K order.
-constexpr int kTileSlices = 16;
 template <int kEpi>
 __global__ __launch_bounds__(256) void skinny_tile_reduce_kernel(const float* __restrict__ part,
                                                                  const bf16_t* __restrict__ residual,
-                                                                 bf16_t* __restrict__ y, int32_t M, int32_t N) {
+                                                                 bf16_t* __restrict__ y, int32_t M, int32_t N,
+                                                                 int32_t n_slices) {
   const int groups = (N + 15) >> 4;
-  const int t = blockIdx.x * blockDim.x + threadIdx.x;
+  const int t = blockIdx.x * blockDim.x + threadIdx.x;       // (row group, lane, element)
   if (t >= groups * 256) return;
-  float v[kTileSlices];
+  float v[kTileMaxSlices];
 #pragma unroll
-  for (int s = 0; s < kTileSlices; ++s) v[s] = part[(int64_t)s * groups * 256 + t];
+  for (int s = 0; s < kTileMaxSlices; ++s) v[s] = s < n_slices ? part[(int64_t)s * groups * 256 + t] : 0.f;
   float sum = 0.f;
 #pragma unroll
-  for (int s = 0; s < kTileSlices; ++s) sum += v[s];
+  for (int s = 0; s < kTileMaxSlices; ++s) sum += v[s];
   const int lane = (t >> 2) & 63;
   const int m = 4 * (lane >> 4) + (t & 3), n = 16 * (t >> 8) + (lane & 15);
   if (m >= M || n >= N) return;
@@ -439,25 +448,32 @@ __global__ __launch_bounds__(256) void skinny_tile_reduce_kernel(const float* __
   y[(int64_t)m * N + n] = f32_to_bf16(sum);
 }
 
-// The cut of the tiled form: 16 K slices when K allows it, row blocks of up to 16 groups; used when it takes at
-// least 8 us less per compute unit than the plain form at ~34 GB/s per compute unit (the second launch costs ~4 us).
+// The cut of the tiled form: up to 16 row groups per row block (fewer when the matrix has fewer than 256 groups), as
+// many K slices as keep the launch within one workgroup per compute unit (at most 16); used when it takes at least
+// 8 us less per compute unit than the plain form at ~34 GB/s (the second launch costs ~4 us).
 struct TilePlan {
-  int n_slices, kslice, gpw, row_blocks;
+  int n_slices, gpw, row_blocks;
   bool use;
 };
 TilePlan plan_tile(int32_t N, int32_t K) {
-  TilePlan t{0, 0, 0, 0, false};
+  TilePlan t{0, 0, 0, false};
   const int groups = (N + 15) / 16;
-  if (K % (16 * 32) != 0 || groups > 256) return t;
-  t.n_slices = kTileSlices;
-  t.kslice = K / 16;
+  const int steps = K / 32;
+  if (K % 32 != 0 || groups > 256) return t;
   t.gpw = std::min(kMaxWaves, (groups + 15) / 16);
   t.row_blocks = (groups + t.gpw - 1) / t.gpw;
-  if (t.row_blocks * t.n_slices > 256) return t;
-  const double plain_bytes = (16.0 + 16.0) * K * 2;                               // one row group + all of x
-  const double tiled_bytes = (16.0 * t.gpw + 16.0) * t.kslice * 2;
-  t.use = (plain_bytes - tiled_bytes) / 34e3 > 8.0;                               // bytes / (34 GB/s) in us
+  t.n_slices = std::min(std::min(kTileMaxSlices, steps), 256 / std::max(1, t.row_blocks));
+  if (t.n_slices < 2) return t;
+  static const int env_tile = [] { const char* e = getenv("MSA_LINEAR_TILE"); return e ? atoi(e) : 1; }();
+  if (env_tile == 0) return t;
+  const double plain_bytes = (16.0 + 16.0) * K * 2;                             // one row group + all of x
+  const double tiled_bytes = (16.0 * t.gpw + 16.0) * ((double)K / t.n_slices) * 2;
+  t.use = (plain_bytes - tiled_bytes) / 34e3 > 8.0;                             // bytes / (34 GB/s) in us
   return t;
+}
+
+size_t tile_workspace_bytes(const TilePlan& t, int32_t N) {
+  return (size_t)t.n_slices * ((N + 15) / 16) * 256 * sizeof(float);
 }
 
 template <int R, int kEpi, bool kNorm>
@@ -548,36 +564,35 @@ extern "C" int msa_skinny_linear(const void* x, const void* w, const void* resid
 extern "C" size_t msa_skinny_linear_workspace_bytes(int32_t M, int32_t N, int32_t K) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   const TilePlan t = plan_tile(N, K);
-  return t.use ? (size_t)t.n_slices * ((N + 15) / 16) * 256 * sizeof(float) : 0;
+  return t.use ? tile_workspace_bytes(t, N) : 0;
 }
 
 extern "C" int msa_skinny_linear_ws(const void* x, const void* w, const void* residual, const void* norm_w, float eps,
                                     int32_t epilogue, int32_t dtype, int32_t M, int32_t N, int32_t K, void* y,
                                     void* workspace, size_t workspace_bytes, void* stream) {
-  static const int env_tile = [] { const char* e = getenv("MSA_LINEAR_TILE"); return e ? atoi(e) : 1; }();
-  const TilePlan t = (N > 0 && K > 0) ? plan_tile(N, K) : TilePlan{0, 0, 0, 0, false};
-  const size_t need = t.use ? (size_t)t.n_slices * ((N + 15) / 16) * 256 * sizeof(float) : 0;
-  const bool tiled = env_tile != 0 && t.use && norm_w == nullptr && (epilogue == kEpiPlain || epilogue == kEpiResidual) &&
-                     workspace != nullptr && workspace_bytes >= need && dtype == MSA_BF16 && M > 0 && M <= 16 &&
-                     (int64_t)M * K * 2 < ((int64_t)1 << 31) && (int64_t)32 * K * 2 < ((int64_t)1 << 31);
-  if (!tiled) return msa_skinny_linear(x, w, residual, norm_w, eps, epilogue, dtype, M, N, K, y, stream);
-  MSA_REQUIRE(x && w && y, "msa_skinny_linear_ws: null pointer");
-  MSA_REQUIRE((epilogue == kEpiResidual) == (residual != nullptr), "msa_skinny_linear_ws: residual pointer and epilogue disagree");
-  MSA_REQUIRE((((uintptr_t)x | (uintptr_t)w | (uintptr_t)workspace) & 15) == 0, "msa_skinny_linear_ws: x / w / workspace must be 16-byte aligned");
+  const bool fits = x && w && y && dtype == MSA_BF16 && M > 0 && M <= 16 && N > 0 && K > 0 && K % kUnit == 0 &&
+                    norm_w == nullptr && (epilogue == kEpiPlain || epilogue == kEpiResidual) &&
+                    (epilogue == kEpiResidual) == (residual != nullptr) && (int64_t)M * K * 2 < ((int64_t)1 << 31) &&
+                    (int64_t)32 * K * 2 < ((int64_t)1 << 31) &&
+                    (((uintptr_t)x | (uintptr_t)w | (uintptr_t)workspace) & 15) == 0;
+  const TilePlan t = fits ? plan_tile(N, K) : TilePlan{0, 0, 0, false};
+  if (!fits || !t.use || workspace == nullptr || workspace_bytes < tile_workspace_bytes(t, N))
+    return msa_skinny_linear(x, w, residual, norm_w, eps, epilogue, dtype, M, N, K, y, stream);   // it reports bad arguments
   hipStream_t st = as_stream(stream);
-  const int steps_pad = (t.kslice / 32 + kTileDepth - 1) / kTileDepth * kTileDepth;
+  const int groups = (N + 15) / 16;
+  const int steps_max = (K / 32 + t.n_slices - 1) / t.n_slices;
+  const int steps_pad = (steps_max + kTileDepth - 1) / kTileDepth * kTileDepth;
   const size_t lds = (size_t)steps_pad * 64 * 16;
-  MSA_REQUIRE(lds <= 64 * 1024, "msa_skinny_linear_ws: K slice of %d elements does not fit LDS", t.kslice);
+  MSA_REQUIRE(lds <= 64 * 1024, "msa_skinny_linear_ws: a K slice of %d steps does not fit LDS", steps_max);
   float* part = static_cast<float*>(workspace);
   skinny_tile_partial_kernel<<<dim3(t.row_blocks, t.n_slices), t.gpw * 64, lds, st>>>(
-      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), part, M, N, K, t.gpw, t.kslice);
+      static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), part, M, N, K, t.gpw);
   MSA_LAUNCH_CHECK();
-  const int blocks = (N + 15) / 16;          // one block of 256 threads per row group
   if (epilogue == kEpiResidual)
-    skinny_tile_reduce_kernel<kEpiResidual><<<blocks, 256, 0, st>>>(part, static_cast<const bf16_t*>(residual),
-                                                                   static_cast<bf16_t*>(y), M, N);
+    skinny_tile_reduce_kernel<kEpiResidual><<<groups, 256, 0, st>>>(part, static_cast<const bf16_t*>(residual),
+                                                                   static_cast<bf16_t*>(y), M, N, t.n_slices);
   else
-    skinny_tile_reduce_kernel<kEpiPlain><<<blocks, 256, 0, st>>>(part, nullptr, static_cast<bf16_t*>(y), M, N);
+    skinny_tile_reduce_kernel<kEpiPlain><<<groups, 256, 0, st>>>(part, nullptr, static_cast<bf16_t*>(y), M, N, t.n_slices);
   MSA_LAUNCH_CHECK();
   return MSA_OK;
 }

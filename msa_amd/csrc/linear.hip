@@ -43,7 +43,7 @@ template <int R, int kEpi, bool kNorm, int J>
 __global__ __launch_bounds__(kMaxWaves * 64) void skinny_linear_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const bf16_t* __restrict__ residual,
     const bf16_t* __restrict__ norm_w, float eps, bf16_t* __restrict__ y, int32_t M, int32_t N, int32_t K,
-    int64_t y_row_stride) {
+    int64_t y_row_stride, int32_t rows_per_wg) {
   constexpr int kUnitBytes = 64 * J;   // one unit = J vectors of 16 bytes per lane = 32 J elements of a row
   const int units = K / (32 * J);
   extern __shared__ __align__(16) float part[];   // [waves][R][64][4], then [waves][16] row sums of squares
@@ -53,11 +53,13 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_linear_kernel(
   // read-first-lane loop around every load)
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n_l = lane & 15, g = lane >> 4;
-  const int n_base = blockIdx.x * (16 * R);
+  // a workgroup owns rows [n_base, n_base + rows_per_wg) of w, rows_per_wg <= 16 R (fewer than 16 R when the matrix
+  // has too few rows to give every compute unit a full set: the rows past it read as zero and are not stored)
+  const int n_base = blockIdx.x * rows_per_wg;
   const int64_t row_bytes = (int64_t)K * 2;
 
   // rows past N (weights) and past M (activations) read as zero through the buffer bounds
-  const int rows_w = min(16 * R, N - n_base);
+  const int rows_w = min(rows_per_wg, N - n_base);
   const __amdgpu_buffer_rsrc_t rs_w = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(reinterpret_cast<const char*>(w)) + (int64_t)n_base * row_bytes, 0, (int)(rows_w * row_bytes),
       0x00020000);
@@ -173,7 +175,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_linear_kernel(
     floatx4_t sum = floatx4_t{0.f, 0.f, 0.f, 0.f};
     for (int wv = 0; wv < waves; ++wv) sum += *reinterpret_cast<const floatx4_t*>(&part[((wv * R + r) * 64 + lane) * 4]);
     const int n = n_base + 16 * r + n_l;
-    if (n >= N) continue;
+    if (n >= N || 16 * r + n_l >= rows_per_wg) continue;
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int m = 4 * g + e;
@@ -478,14 +480,14 @@ size_t tile_workspace_bytes(const TilePlan& t, int32_t N) {
 
 template <int R, int kEpi, bool kNorm>
 int launch(const void* x, const void* w, const void* residual, const void* norm_w, float eps, void* y, int32_t M,
-           int32_t N, int32_t K, int waves, hipStream_t st) {
-  const int groups = (N + 16 * R - 1) / (16 * R);
+           int32_t N, int32_t K, int waves, int rows_per_wg, hipStream_t st) {
+  const int groups = (N + rows_per_wg - 1) / rows_per_wg;
   const size_t lds = (size_t)waves * (R * 256 + 16) * sizeof(float);
   const int64_t y_stride = kEpi == kEpiSiluMul ? N / 2 : N;
   // with the norm folded in a unit is 64 elements instead of 128: the extra fragments then fit 128 VGPRs
   skinny_linear_kernel<R, kEpi, kNorm, kNorm ? 2 : 4><<<groups, waves * 64, lds, st>>>(
       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<const bf16_t*>(residual),
-      static_cast<const bf16_t*>(norm_w), eps, static_cast<bf16_t*>(y), M, N, K, y_stride);
+      static_cast<const bf16_t*>(norm_w), eps, static_cast<bf16_t*>(y), M, N, K, y_stride, rows_per_wg);
   MSA_LAUNCH_CHECK();
   return MSA_OK;
 }
@@ -538,7 +540,16 @@ extern "C" int msa_skinny_linear(const void* x, const void* w, const void* resid
   int R = ((int64_t)N / 32 * kMaxWaves >= 3072 || epilogue == kEpiSiluMul) ? 2 : 1;
   if (env_r == 1 && epilogue != kEpiSiluMul) R = 1;
   if (env_r == 2) R = 2;
-  const int groups = (N + 16 * R - 1) / (16 * R);
+  // Rows per workgroup: 16 R, or fewer when that leaves compute units without a workgroup (a compute unit moves
+  // only ~34 GB/s, so 256 workgroups of 10 rows beat 160 of 16 on a 2560-row matrix); the silu epilogue needs whole
+  // gate / up groups.
+  static const int env_spread = [] { const char* e = getenv("MSA_LINEAR_SPREAD"); return e ? atoi(e) : 1; }();
+  int rows_per_wg = 16 * R;
+  if (env_spread != 0 && epilogue != kEpiSiluMul && (N + 16 * R - 1) / (16 * R) < 256) {
+    const int spread = std::max(8, (N + 255) / 256);
+    if (spread > 16 * (R - 1) && spread < 16 * R) rows_per_wg = spread;
+  }
+  const int groups = (N + rows_per_wg - 1) / rows_per_wg;
   int want = (int)std::min<int64_t>(kMaxWaves, std::max<int64_t>(1, (4096 + groups - 1) / groups));
   want = std::max(1, std::min(want, units));
   int waves = want;
@@ -547,8 +558,8 @@ extern "C" int msa_skinny_linear(const void* x, const void* w, const void* resid
   if (env_waves > 0) waves = std::max(1, std::min(std::min(env_waves, kMaxWaves), units));
 
 #define MSA_LIN(R_, E_)                                                                              \
-  (norm_w ? launch<R_, E_, true>(x, w, residual, norm_w, eps, y, M, N, K, waves, st)                 \
-          : launch<R_, E_, false>(x, w, residual, norm_w, eps, y, M, N, K, waves, st))
+  (norm_w ? launch<R_, E_, true>(x, w, residual, norm_w, eps, y, M, N, K, waves, rows_per_wg, st)    \
+          : launch<R_, E_, false>(x, w, residual, norm_w, eps, y, M, N, K, waves, rows_per_wg, st))
   switch (epilogue * 8 + R) {
     case kEpiPlain * 8 + 1: return MSA_LIN(1, kEpiPlain);
     case kEpiPlain * 8 + 2: return MSA_LIN(2, kEpiPlain);

@@ -4,6 +4,11 @@
 // owns d in [8j, 8j+8) and [64+8j, 64+8j+8) — the two halves the half-split rotary pairs — so the
 // optional RoPE on K needs no cross-lane traffic.  256 threads cover R = 256 / (H*8) token rows
 // per step, accumulate in fp32 registers, and fold the R partial rows through LDS at the end.
+// Each lane keeps two groups of rows in flight as raw 16-byte loads (16 KB per wavefront in bf16):
+// with one row per wait the kernel was bound by load latency at 0.65-0.68 of the HBM rate; the
+// two-group pipeline reaches 0.75.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -27,21 +32,35 @@ struct PoolArgs {
   int32_t rope_rows;
 };
 
-template <typename T>
-__device__ __forceinline__ void load8(const T* p, float (&x)[8]);
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
+// Eight consecutive elements of a row as they come from memory; converted to fp32 only when consumed,
+// so a wavefront can keep two groups of rows in flight without holding them as floats.
+template <typename T>
+struct Raw8;
 template <>
-__device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float (&x)[8]) {
-  const uint4 w = *reinterpret_cast<const uint4*>(p);
-  x[0] = bf16lo(w.x); x[1] = bf16hi(w.x); x[2] = bf16lo(w.y); x[3] = bf16hi(w.y);
-  x[4] = bf16lo(w.z); x[5] = bf16hi(w.z); x[6] = bf16lo(w.w); x[7] = bf16hi(w.w);
-}
+struct Raw8<bf16_t> {
+  u32x4_t w;
+  __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t rs, int voff, int soff) {
+    w = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff, 0);
+  }
+  __device__ __forceinline__ void unpack(float (&x)[8]) const {
+    x[0] = bf16lo(w.x); x[1] = bf16hi(w.x); x[2] = bf16lo(w.y); x[3] = bf16hi(w.y);
+    x[4] = bf16lo(w.z); x[5] = bf16hi(w.z); x[6] = bf16lo(w.w); x[7] = bf16hi(w.w);
+  }
+};
 template <>
-__device__ __forceinline__ void load8<float>(const float* p, float (&x)[8]) {
-  const float4 a = *reinterpret_cast<const float4*>(p);
-  const float4 b = *reinterpret_cast<const float4*>(p + 4);
-  x[0] = a.x; x[1] = a.y; x[2] = a.z; x[3] = a.w; x[4] = b.x; x[5] = b.y; x[6] = b.z; x[7] = b.w;
-}
+struct Raw8<float> {
+  u32x4_t a, b;
+  __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t rs, int voff, int soff) {
+    a = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff, 0);
+    b = __builtin_amdgcn_raw_buffer_load_b128(rs, voff + 16, soff, 0);
+  }
+  __device__ __forceinline__ void unpack(float (&x)[8]) const {
+    x[0] = __uint_as_float(a.x); x[1] = __uint_as_float(a.y); x[2] = __uint_as_float(a.z); x[3] = __uint_as_float(a.w);
+    x[4] = __uint_as_float(b.x); x[5] = __uint_as_float(b.y); x[6] = __uint_as_float(b.z); x[7] = __uint_as_float(b.w);
+  }
+};
 
 template <typename T>
 __device__ __forceinline__ void store8(T* p, const float (&x)[8]);
@@ -59,7 +78,7 @@ __device__ __forceinline__ void store8<float>(float* p, const float (&x)[8]) {
 }
 
 template <typename T>
-__global__ __launch_bounds__(kThreads) void pool_chunks_kernel(PoolArgs a) {
+__global__ __launch_bounds__(kThreads, 2) void pool_chunks_kernel(PoolArgs a) {
   __shared__ float fold[kThreads * 16];
 
   const int c = blockIdx.x;
@@ -69,16 +88,39 @@ __global__ __launch_bounds__(kThreads) void pool_chunks_kernel(PoolArgs a) {
   const bool rope = a.rope[slot] != 0;
 
   const int U = a.H * 8;          // lanes per token row
-  const int R = kThreads / U;     // token rows per step
+  const int R = kThreads / U;     // token rows per step (the host checks that U divides the workgroup)
   const int tid = threadIdx.x;
   const int r = tid / U, u = tid % U;
-  const bool active = r < R;
   const int h = u >> 3, j = u & 7;
   const int row_elems = a.H * kHeadDim;
   const int col_lo = h * kHeadDim + 8 * j, col_hi = col_lo + 64;
 
-  const int32_t t0 = a.chunk_start[c];
-  const int32_t len = a.chunk_len[c];
+  const int32_t t0 = __builtin_amdgcn_readfirstlane(a.chunk_start[c]);
+  const int32_t len = __builtin_amdgcn_readfirstlane(a.chunk_len[c]);
+
+  // Rows are fetched in groups of R * kRows through a buffer resource that spans exactly the group's
+  // valid rows: a row past the chunk's end (or past T) reads as zero without touching memory and adds
+  // nothing to the sums, so the loop needs no per-row predicate.  Two groups (A, B) alternate; the
+  // loads of one are in flight while the other is consumed.
+  constexpr int kRows = sizeof(T) == 2 ? 4 : 2;
+  const int row_bytes = row_elems * (int)sizeof(T);
+  const int group_rows = R * kRows;
+  const int voff = r * row_bytes + col_lo * (int)sizeof(T);
+  const int q_stride = R * row_bytes;
+  const int32_t rows_valid = (int32_t)min((int64_t)len, a.T - (int64_t)t0);
+  const char* chunk_base = reinterpret_cast<const char*>(in) + (int64_t)t0 * row_bytes;
+  Raw8<T> lo_a[kRows], hi_a[kRows], lo_b[kRows], hi_b[kRows];
+  auto issue = [&](Raw8<T>(&lo)[kRows], Raw8<T>(&hi)[kRows], int base) {
+    const int rows = max(0, min(rows_valid - base, group_rows));
+    const __amdgpu_buffer_rsrc_t group = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(chunk_base) + (int64_t)base * row_bytes, 0, rows * row_bytes, 0x00020000);
+#pragma unroll
+    for (int q = 0; q < kRows; ++q) {
+      lo[q].load(group, voff, q * q_stride);
+      hi[q].load(group, voff + 64 * (int)sizeof(T), q * q_stride);
+    }
+  };
+  issue(lo_a, hi_a, 0);
 
   float acc_lo[8], acc_hi[8];
 #pragma unroll
@@ -86,7 +128,7 @@ __global__ __launch_bounds__(kThreads) void pool_chunks_kernel(PoolArgs a) {
 
   // rotary state of this lane's 8 frequencies at its current token, advanced by R positions per step
   float rc[8], rs[8], sc[8], ss[8];
-  if (rope && active) {
+  if (rope) {
     const int32_t pos0 = t0 - a.doc_start[a.chunk_doc[c]] + r;
     const int32_t p = min(pos0, a.rope_rows - 1), st = min(R, a.rope_rows - 1);
 #pragma unroll
@@ -98,56 +140,50 @@ __global__ __launch_bounds__(kThreads) void pool_chunks_kernel(PoolArgs a) {
     }
   }
 
-  if (active) {
-    constexpr int kUnroll = 4;
-    for (int base = 0; base < len; base += R * kUnroll) {
-      float xl[kUnroll][8], xh[kUnroll][8];
-      bool ok[kUnroll];
+  auto consume = [&](auto rope_tag, const Raw8<T>(&lo)[kRows], const Raw8<T>(&hi)[kRows]) {
+    constexpr bool kRope = decltype(rope_tag)::value;
 #pragma unroll
-      for (int q = 0; q < kUnroll; ++q) {
-        const int off = base + q * R + r;
-        const int64_t t = (int64_t)t0 + off;
-        ok[q] = off < len && t < a.T;
-        if (ok[q]) {
-          const T* p = in + t * row_elems;
-          load8<T>(p + col_lo, xl[q]);
-          load8<T>(p + col_hi, xh[q]);
+    for (int q = 0; q < kRows; ++q) {
+      float xl[8], xh[8];
+      lo[q].unpack(xl);
+      hi[q].unpack(xh);
+      if constexpr (kRope) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          acc_lo[i] += xl[i] * rc[i] - xh[i] * rs[i];
+          acc_hi[i] += xh[i] * rc[i] + xl[i] * rs[i];
         }
-      }
 #pragma unroll
-      for (int q = 0; q < kUnroll; ++q) {
-        if (rope) {
-          if (ok[q]) {
+        for (int i = 0; i < 8; ++i) {   // advance the angle by R positions
+          const float nc = rc[i] * sc[i] - rs[i] * ss[i];
+          rs[i] = rs[i] * sc[i] + rc[i] * ss[i];
+          rc[i] = nc;
+        }
+      } else {
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
-              acc_lo[i] += xl[q][i] * rc[i] - xh[q][i] * rs[i];
-              acc_hi[i] += xh[q][i] * rc[i] + xl[q][i] * rs[i];
-            }
-          }
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {   // advance the angle by R positions
-            const float nc = rc[i] * sc[i] - rs[i] * ss[i];
-            rs[i] = rs[i] * sc[i] + rc[i] * ss[i];
-            rc[i] = nc;
-          }
-        } else if (ok[q]) {
-#pragma unroll
-          for (int i = 0; i < 8; ++i) {
-            acc_lo[i] += xl[q][i];
-            acc_hi[i] += xh[q][i];
-          }
+        for (int i = 0; i < 8; ++i) {
+          acc_lo[i] += xl[i];
+          acc_hi[i] += xh[i];
         }
       }
     }
-  }
+  };
+  auto stream = [&](auto rope_tag) {
+    for (int base = 0; base < rows_valid; base += 2 * group_rows) {
+      issue(lo_b, hi_b, base + group_rows);
+      consume(rope_tag, lo_a, hi_a);
+      issue(lo_a, hi_a, base + 2 * group_rows);   // empty once past the end
+      consume(rope_tag, lo_b, hi_b);
+    }
+  };
+  if (rope) stream(std::true_type{});
+  else stream(std::false_type{});
 
   // fold the R partial rows: fold[(r * U + u) * 16 + i]
-  if (active) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      fold[(r * U + u) * 16 + i] = acc_lo[i];
-      fold[(r * U + u) * 16 + 8 + i] = acc_hi[i];
-    }
+  for (int i = 0; i < 8; ++i) {
+    fold[(r * U + u) * 16 + i] = acc_lo[i];
+    fold[(r * U + u) * 16 + 8 + i] = acc_hi[i];
   }
   __syncthreads();
   if (tid < U) {

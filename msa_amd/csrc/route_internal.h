@@ -3,7 +3,10 @@
 #include "common.h"
 
 constexpr int kTopkMax = 64;          // width of every candidate list (one wavefront)
-constexpr int kTopkDocsPerBlock = 4096;
+#ifndef TOPK_DOCS
+#define TOPK_DOCS 2048
+#endif
+constexpr int kTopkDocsPerBlock = TOPK_DOCS;
 
 struct RouteWorkspace {
   int32_t S_pad;        // query tokens padded to a multiple of 32 (one MFMA row block never spans two queries)

@@ -36,29 +36,37 @@ __global__ void presum_queries_kernel(const TIn* __restrict__ q, const uint8_t* 
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
   if (valid) {
-    for (int hh = 0; hh < G; ++hh) {
-      const TIn* p = q + (((int64_t)b * S + s) * Hq + (g * G + hh)) * kHeadDim + 8 * j;
-      float x[8];
-      if constexpr (sizeof(TIn) == 2) {
-        const uint4 w = *reinterpret_cast<const uint4*>(p);
-        x[0] = bf16lo(w.x); x[1] = bf16hi(w.x); x[2] = bf16lo(w.y); x[3] = bf16hi(w.y);
-        x[4] = bf16lo(w.z); x[5] = bf16hi(w.z); x[6] = bf16lo(w.w); x[7] = bf16hi(w.w);
-      } else {
-        const float4 u = *reinterpret_cast<const float4*>(p);
-        const float4 v = *reinterpret_cast<const float4*>(p + 4);
-        x[0] = u.x; x[1] = u.y; x[2] = u.z; x[3] = u.w; x[4] = v.x; x[5] = v.y; x[6] = v.z; x[7] = v.w;
-      }
-      float inv = 1.f;
-      if (normalize) {
-        float ssq = 0.f;
+    const TIn* p0 = q + (((int64_t)b * S + s) * Hq + g * G) * kHeadDim + 8 * j;
+    for (int h0 = 0; h0 < G; h0 += 4) {          // four heads' loads in flight before the first is normalised
+      float x[4][8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) ssq += x[i] * x[i];
-        ssq += __shfl_xor(ssq, 1); ssq += __shfl_xor(ssq, 2);     // the 16 lanes of one group
-        ssq += __shfl_xor(ssq, 4); ssq += __shfl_xor(ssq, 8);
-        inv = 1.0f / fmaxf(sqrtf(ssq), 1e-12f);
+      for (int u = 0; u < 4; ++u) {
+        const TIn* p = p0 + (int64_t)min(h0 + u, G - 1) * kHeadDim;
+        if constexpr (sizeof(TIn) == 2) {
+          const uint4 w = *reinterpret_cast<const uint4*>(p);
+          x[u][0] = bf16lo(w.x); x[u][1] = bf16hi(w.x); x[u][2] = bf16lo(w.y); x[u][3] = bf16hi(w.y);
+          x[u][4] = bf16lo(w.z); x[u][5] = bf16hi(w.z); x[u][6] = bf16lo(w.w); x[u][7] = bf16hi(w.w);
+        } else {
+          const float4 lo = *reinterpret_cast<const float4*>(p);
+          const float4 hi = *reinterpret_cast<const float4*>(p + 4);
+          x[u][0] = lo.x; x[u][1] = lo.y; x[u][2] = lo.z; x[u][3] = lo.w;
+          x[u][4] = hi.x; x[u][5] = hi.y; x[u][6] = hi.z; x[u][7] = hi.w;
+        }
       }
 #pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] += x[i] * inv;
+      for (int u = 0; u < 4; ++u) {
+        float inv = h0 + u < G ? 1.f : 0.f;      // a clamped repeat of the last head adds nothing
+        if (normalize) {
+          float ssq = 0.f;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) ssq += x[u][i] * x[u][i];
+          ssq += __shfl_xor(ssq, 1); ssq += __shfl_xor(ssq, 2);     // the 16 lanes of one group
+          ssq += __shfl_xor(ssq, 4); ssq += __shfl_xor(ssq, 8);
+          inv *= 1.0f / fmaxf(sqrtf(ssq), 1e-12f);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] += x[u][i] * inv;
+      }
     }
   }
   TOut* o = qs + ((int64_t)row * Hkv + g) * kHeadDim + 8 * j;
@@ -119,7 +127,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     const uint32_t* __restrict__ row_bits,  // [ceil(M_alloc / 32)] scored-row bitmask
     uint32_t* __restrict__ chunk_key,    // [B, C]
     int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t tiles_m, int32_t tiles_n,
-    int32_t m_group) {
+    int32_t m_group, int32_t exclusive) {
   constexpr int kThreads = WAVES_M * WAVES_N * 64;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -250,6 +258,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   k_tile(std::false_type{}, k_tiles - 1);
 
   // Epilogue.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of its 32x32 block.
+  // `exclusive`: every query's rows lie inside one wavefront's tile, so each (query, chunk) key has a single
+  // writer, which stores it (0 for a query without a scored token) into a plane nobody cleared.  Otherwise
+  // several wavefronts or workgroups hold parts of a query and combine through atomicMax on a zeroed plane.
+  const int n_queries = M_rows / (blocks_per_query * 32);
+  auto emit = [&](int q, int n, float run, bool any) {
+    if (half != 0 || n >= C || q >= n_queries) return;
+    uint32_t* dst = &chunk_key[(int64_t)q * C + n];
+    if (exclusive) *dst = any ? f32_to_key(run) : 0u;
+    else if (any) atomicMax(dst, f32_to_key(run));
+  };
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
     const int n = n0 + wn * WN + j * 32 + l32;
@@ -262,7 +280,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
       const int qid = blk / blocks_per_query;
       const uint32_t bits = row_bits[blk];               // 0 for blocks past M_rows (buffer is padded)
       if (qid != run_q) {
-        if (any && half == 0 && n < C) atomicMax(&chunk_key[(int64_t)run_q * C + n], f32_to_key(run));
+        if (run_q >= 0) emit(run_q, n, run, any);
         run = -INFINITY; any = false; run_q = qid;
       }
       if (bits != 0) {
@@ -277,7 +295,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
         any = true;
       }
     }
-    if (any && half == 0 && n < C) atomicMax(&chunk_key[(int64_t)run_q * C + n], f32_to_key(run));
+    emit(run_q, n, run, any);
   }
 }
 
@@ -301,7 +319,12 @@ struct KernelTimer {
 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
 int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* chunk_key, int32_t M_rows,
-                int32_t C, int32_t K, int32_t blocks_per_query, hipStream_t st) {
+                int32_t C, int32_t K, int32_t blocks_per_query, int32_t exclusive, hipStream_t st) {
+  if (exclusive && (BM / WAVES_M) % (blocks_per_query * 32) != 0) {
+    msa_set_error("score_gemm: single-writer epilogue asked for %d-row queries on %d-row wavefront tiles",
+                  blocks_per_query * 32, BM / WAVES_M);
+    return MSA_EINVAL;
+  }
   const int tiles_m = (M_rows + BM - 1) / BM, tiles_n = (C + BN - 1) / BN;
   const int m_group = tiles_m;   // all M tiles of a K_r tile adjacent: measured best (groups of 1, 2, 4 lose 2-14 %)
   const int grid = 8 * ((tiles_n + 7) / 8) * tiles_m;
@@ -316,7 +339,8 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
   const bool timed = g_timer.n < g_timer.cap;
   if (timed) MSA_HIP(hipEventRecord(g_timer.start[g_timer.n], st));
   kern<<<grid, WAVES_M * WAVES_N * 64, lds, st>>>(static_cast<const T*>(qs), static_cast<const T*>(kr), row_bits,
-                                                  chunk_key, M_rows, C, K, blocks_per_query, tiles_m, tiles_n, m_group);
+                                                  chunk_key, M_rows, C, K, blocks_per_query, tiles_m, tiles_n, m_group,
+                                                  exclusive);
   MSA_LAUNCH_CHECK();
   if (timed) {
     MSA_HIP(hipEventRecord(g_timer.stop[g_timer.n], st));
@@ -416,11 +440,24 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
   void* qs = ws + w.off_qs;
   uint32_t* row_bits = reinterpret_cast<uint32_t*>(ws + w.off_row_bits);
   uint32_t* chunk_key = reinterpret_cast<uint32_t*>(ws + w.off_chunk_key);
-  const int64_t m_alloc = ((int64_t)w.M_rows + 255) / 256 * 256;
+  // Tile choice by query rows: small M is HBM-bound (narrow M tile, more workgroups in flight),
+  // large M is MFMA-bound (256 x 256 tile, 8 wavefronts).  MSA_SCORE_TILE overrides for tuning.
+  // wave_rows[v] = rows of one wavefront's tile in variant v (BM / WAVES_M).
+  static const int wave_rows[10] = {32, 64, 128, 64, 64, 64, 64, 32, 128, 64};
+  const char* ev = getenv("MSA_SCORE_TILE");
+  const int variant = ev ? atoi(ev) : (w.M_rows <= 64 ? 0 : w.M_rows <= 128 ? 6 : 2);
+  if (bank->dtype == MSA_BF16 && (variant < 0 || variant > 9)) {
+    msa_set_error("MSA_SCORE_TILE=%d unknown", variant);
+    return MSA_EINVAL;
+  }
+  // A query whose rows fit one wavefront's tile has a single writer per chunk key: the kernel stores
+  // and the key plane needs no clearing (at the 100M-token bank the plane is 103 MB per launch).
+  const int32_t exclusive = (bank->dtype == MSA_BF16 ? wave_rows[variant] : 64) % w.S_pad == 0 ? 1 : 0;
 
-  // row masks and chunk keys start at zero (both live in one contiguous span of the workspace)
-  const int64_t zero_words = (int64_t)((w.off_cand - w.off_row_bits) / sizeof(uint32_t));
-  (void)m_alloc;
+  // row masks start at zero; so do the chunk keys when wavefronts combine through atomicMax (both live in one
+  // contiguous span of the workspace)
+  const int64_t zero_words =
+      (int64_t)(((exclusive ? w.off_chunk_key : w.off_cand) - w.off_row_bits) / sizeof(uint32_t));
   fill_u32_kernel<<<(int)std::min<int64_t>((zero_words + 1023) / 1024, 4096), 256, 0, st>>>(row_bits, zero_words, 0u);
   MSA_LAUNCH_CHECK();
 
@@ -440,13 +477,9 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
   const int32_t bpq = w.S_pad / 32;
   int rc;
   if (bank->dtype == MSA_BF16) {
-    // Tile choice by query rows: small M is HBM-bound (narrow M tile, more workgroups in flight),
-    // large M is MFMA-bound (256 x 256 tile, 8 wavefronts).  MSA_SCORE_TILE overrides for tuning.
-    const char* ev = getenv("MSA_SCORE_TILE");
-    const int variant = ev ? atoi(ev) : (w.M_rows <= 64 ? 0 : w.M_rows <= 128 ? 6 : 2);
 #define MSA_GEMM(BM_, BN_, WM_, WN_)                                                                              \
   launch_gemm<bf16_t, BM_, BN_, WM_, WN_>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C, \
-                                          K, bpq, st)
+                                          K, bpq, exclusive, st)
     switch (variant) {
       case 0: rc = MSA_GEMM(64, 128, 2, 2); break;
       case 1: rc = MSA_GEMM(128, 256, 2, 4); break;
@@ -463,7 +496,7 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
 #undef MSA_GEMM
   } else {
     rc = launch_gemm<float, 128, 128, 2, 2>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C, K,
-                                            bpq, st);
+                                            bpq, exclusive, st);
   }
   if (rc != MSA_OK) return rc;
   *layout_out = w;

@@ -32,7 +32,7 @@ HQ, HKV, D, P, TOPK = 32, 8, 128, 64, 16
 # Bytes past L2 per launch of the scoring kernel at the default workload, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a plain 1 GiB device copy
 # (FETCH_SIZE x2.0, WRITE_SIZE x1.0); see profiles/score_gemm_c4_100M_bank.txt.
-SCORE_TRAFFIC_DEFAULT_WORKLOAD = (2.0 * 3_354_966 + 1.0 * 122_269) * 1024
+SCORE_TRAFFIC_DEFAULT_WORKLOAD = (2.0 * 3_374_335 + 1.0 * 156_209) * 1024
 
 
 def log(msg):
@@ -382,6 +382,8 @@ def main():
                                             gv[li & 1].data_ptr(), cap_chunks, cu_dev[li].data_ptr(), gws.data_ptr(),
                                             gws.numel(), side.cuda_stream), "msa_gather_kv_device")
 
+    pending = [None]                  # layer whose selected K / V have not been fetched yet
+
     def step():
         if args.gather == "device":
             for li in range(L):
@@ -390,18 +392,25 @@ def main():
             return
         for li in range(L):
             route(li)                      # layer li is being scored ...
-            if li > 0:
-                gather(li - 1)             # ... while layer li-1's K / V come over from the host
-        gather(L - 1)
+            if pending[0] is not None:
+                gather(pending[0])         # ... while the previous layer's K / V come over from the host (the last
+            pending[0] = li                # layer's under the first scan of the next batch)
+
+    def drain():                           # the last batch's last layer has no scan left to hide under
+        if pending[0] is not None:
+            gather(pending[0])
+            pending[0] = None
 
     for _ in range(args.warmup):
         step()
+    drain()
     torch.cuda.synchronize()
     _lib.check(lib.msa_profile_enable(args.steps * L), "msa_profile_enable")
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
+    drain()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_buf = (C.c_float * (args.steps * L))()

@@ -358,3 +358,67 @@ def test_greedy_sample_against_argmax(ops, dtype, B, V):
     tok2 = torch.empty(B, dtype=torch.int64, device="cuda")
     ops.greedy_sample(dev, tok2)                               # argmax only
     assert tok2.cpu().tolist() == want.tolist()
+
+
+@pytest.mark.parametrize("B,S", [(16, 128), (4, 64), (3, 96), (2, 200), (1, 128), (5, 32), (9, 1)])
+def test_score_epilogue_forms_on_a_dirty_workspace(ops, B, S):
+    """Queries that fit one wavefront's tile are stored by a single writer into a key plane nobody cleared; the others
+    combine through atomicMax on a cleared plane.  Both must give the oracle's scores whatever the workspace held
+    before, and a query without a scored token must come back as -inf everywhere."""
+    say(f"epilogue forms B={B} S={S}")
+    bank, kr, dco, _ = _bank(ops, [3, 1, 7, 2, 9, 4, 1, 1, 12] * 41, 8, torch.bfloat16, 900 + B)
+    q = _randn((B, S, 32, 128), 901 + S, torch.bfloat16)
+    mask = torch.ones(B, S, dtype=torch.bool)
+    mask[0, S // 2 + 1:] = False
+    if B > 1:
+        mask[B - 1] = False
+    bank.workspace(B, S, 32, 16, "cuda").fill_(0xFF)
+    got = ops.chunk_scores(bank, 0, q.cuda(), mask.cuda()).cpu()
+    want = cf.chunk_scores(q, mask, kr, "cosine")
+    live = mask.any(dim=1)
+    assert cf.rel_err(got[live], want[live]) < 1e-2
+    assert torch.isinf(got[~live]).all() and (got[~live] < 0).all()
+    bank.workspace(B, S, 32, 16, "cuda").fill_(0xFF)
+    s, d, _ = ops.route_topk(bank, 0, q.cuda(), mask.cuda(), "cosine", 1.0, 16)
+    ds = cf.doc_scores(want, dco)
+    assert not cf.topk_acceptable(ds[live], d.cpu().long()[live], 16)
+    assert torch.isinf(s.cpu()[~live]).all()
+
+
+@pytest.mark.parametrize("topk", [1, 16, 64])
+def test_topk_windows_long_documents_and_filtering(ops, topk):
+    """Documents longer than the top-k kernel's LDS window (2044 keys) among one-chunk documents, more documents
+    than one workgroup's block, and planted winners at both ends of the bank: ids and order must be exact."""
+    say(f"top-k windows topk={topk}")
+    rng = np.random.default_rng(11)
+    doc_chunks = [1] * 3000 + [5000] + list(rng.integers(1, 40, size=2500)) + [2045, 2044, 4089] + [1] * 700
+    bank, kr, dco, dev = _bank(ops, doc_chunks, 8, torch.bfloat16, 930)
+    n_docs = len(doc_chunks)
+    B, S = 3, 8
+    q = _randn((B, S, 32, 128), 931, torch.bfloat16)
+    # plant winners: the last chunk of a chosen document becomes the direction one query token has after the
+    # pre-sum over each group's heads, scaled down by rank (6 % steps, far above bf16 noise); every query gets its
+    # own documents, spread over both ends of the bank and the long documents
+    edge = [0, 2999, 3000, 3001, n_docs - 1, n_docs - 702, n_docs - 703, 4000, 1, 2998, 3100, n_docs - 2,
+            n_docs - 701, n_docs - 704, 4001, 2, 2997, 3500, n_docs - 3, n_docs - 700, 3200, 4002, 3, 2996]
+    assert len(set(edge)) == len(edge) and doc_chunks[n_docs - 702] == 2044 and doc_chunks[3000] == 5000
+    n_win = max(1, min(8, topk))
+    qf = cf.l2_normalize(q.double())
+    for b in range(B):
+        for r, dsel in enumerate(edge[b::B][:n_win]):
+            c = int(dco[dsel + 1]) - 1
+            v = qf[b, r % S].view(8, 4, 128).mean(dim=1)                   # [Hkv, D]
+            kr[c] = (cf.l2_normalize(v) * (1.0 - 0.06 * r)).to(torch.bfloat16)
+    dev.copy_(kr.cuda())
+    s, d, _ = ops.route_topk(bank, 0, q.cuda(), None, "cosine", 1.0, topk)
+    ds = cf.doc_scores(cf.chunk_scores(q, torch.ones(B, S, dtype=torch.bool), kr, "cosine"), dco)
+    assert not cf.topk_acceptable(ds, d.cpu().long(), topk)
+    ws, wi = cf.topk_docs(ds, topk)
+    assert cf.rel_err(s.cpu(), ws) < 1e-2
+    sc = s.cpu()
+    assert (sc[:, :-1] >= sc[:, 1:]).all()
+    # clear winners (gap above the rest far larger than bf16 noise) must match the oracle id for id, in order
+    got = d.cpu().long()[:, :n_win]
+    assert torch.equal(got, wi[:, :n_win]), (got, wi[:, :n_win])
+    for b in range(B):
+        assert sorted(got[b].tolist()) == sorted(edge[b::B][:n_win])

@@ -120,7 +120,9 @@ struct Mma<float> {
 };
 
 // Workgroup tile BM x BN, WAVES_M x WAVES_N wavefronts, each owning TM x TN blocks of 32 x 32.
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
+// kDeep: two register sets of global loads in flight (two K tiles ahead of the one being multiplied) for the
+// HBM-bound shapes, where one tile's MFMA work is shorter than a load's latency.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool kDeep = false>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     const T* __restrict__ qs,            // [M_rows, K]  pre-summed queries, M_rows = B * S_pad
     const T* __restrict__ kr,            // [C, K]
@@ -168,31 +170,39 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
       const_cast<char*>(gb) + (int64_t)n0 * row_bytes_g, 0, (int)(rows_b * row_bytes_g), 0x00020000);
   const int voff = (tid >> 3) * (int)row_bytes_g + (tid & 7) * 16;
   const int vec_stride = (kThreads / 8) * (int)row_bytes_g;     // rows between a thread's vectors
-  u32x4_t ra[kVecA], rb[kVecB];
+  constexpr int kSets = kDeep ? 2 : 1;
+  u32x4_t ra[kSets][kVecA], rb[kSets][kVecB];
   // K_r streams through once per M tile group while the query matrix is re-read by every workgroup of an XCD: the
   // non-temporal hint on the K_r loads keeps the queries in the 4 MiB L2 (traffic past L2 9.9 -> 6.9 GB per launch
   // at the 100M-token bank, 1.5 % faster).
   constexpr int kStreamHint = 2;
-  auto load_tile = [&](int kt) {
+  constexpr int kPastEnd = 0x40000000;   // vector offset beyond any tile's extent: the load returns zeros, no traffic
+  const int k_tiles = (int)(row_bytes_g / kRowBytes);
+  auto load_tile = [&](auto set_tag, int kt) {
+    constexpr int set = decltype(set_tag)::value;
+    const int vo = kt < k_tiles ? voff : kPastEnd;   // a tile past the row is never fetched (keeps the loop branch-free)
 #pragma unroll
     for (int i = 0; i < kVecA; ++i)
-      ra[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, voff + i * vec_stride, kt * kRowBytes, 0);
+      ra[set][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, vo + i * vec_stride, kt * kRowBytes, 0);
 #pragma unroll
     for (int i = 0; i < kVecB; ++i)
-      rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, voff + i * vec_stride, kt * kRowBytes, kStreamHint);
+      rb[set][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo + i * vec_stride, kt * kRowBytes, kStreamHint);
   };
-  auto store_tile = [&](int buf) {
+  auto store_tile = [&](auto set_tag, int buf) {
+    constexpr int set = decltype(set_tag)::value;
 #pragma unroll
     for (int i = 0; i < kVecA; ++i) {
       const int v = tid + i * kThreads, r = v >> 3, c = v & 7;
-      *reinterpret_cast<u32x4_t*>(lds + buf * kBufBytes + r * kRowStride + c * 16) = ra[i];
+      *reinterpret_cast<u32x4_t*>(lds + buf * kBufBytes + r * kRowStride + c * 16) = ra[set][i];
     }
 #pragma unroll
     for (int i = 0; i < kVecB; ++i) {
       const int v = tid + i * kThreads, r = v >> 3, c = v & 7;
-      *reinterpret_cast<u32x4_t*>(lds + buf * kBufBytes + (BM + r) * kRowStride + c * 16) = rb[i];
+      *reinterpret_cast<u32x4_t*>(lds + buf * kBufBytes + (BM + r) * kRowStride + c * 16) = rb[set][i];
     }
   };
+  typedef std::integral_constant<int, 0> Set0;
+  typedef std::integral_constant<int, kSets - 1> Set1;
 
   floatx16_t acc[TM][TN];
 #pragma unroll
@@ -212,7 +222,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   // barrier of iteration kt-1; the writes of tile kt+1 are complete at the barrier of iteration kt.
   typedef typename Mma<T>::Frag Frag;
   constexpr int kSub = Mma<T>::kSub;
-  const int k_tiles = (int)(row_bytes_g / kRowBytes);
   const int a_row = (wm * WM + l32) * kRowStride, b_row = (BM + wn * WN + l32) * kRowStride;
   Frag fa[2][TM], fb[2][TN];
   auto load_frags = [&](int buf, int sub, int slot) {
@@ -225,8 +234,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   };
 
   // One K tile out of LDS buffer `buf`; kMore says a next tile exists (the steady-state loop is
-  // compiled without that condition so the wait counters around the barrier stay exact).
-  auto k_tile = [&](auto more_tag, int kt) {
+  // compiled without that condition so the wait counters around the barrier stay exact).  `set_tag` names the
+  // register set that holds tile kt+1 and takes the next global loads.
+  auto k_tile = [&](auto more_tag, auto set_tag, int kt) {
     constexpr bool kMore = decltype(more_tag)::value;
     const int buf = kt & 1;
 #pragma unroll
@@ -239,8 +249,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
         __builtin_amdgcn_sched_barrier(0);   // keep the last sub-step's MFMAs behind these reads
       }
       if (sub == 1 && kMore) {
-        store_tile(buf ^ 1);
-        if (kt + 2 < k_tiles) load_tile(kt + 2);
+        store_tile(set_tag, buf ^ 1);
+        if constexpr (kDeep) {
+          __builtin_amdgcn_sched_barrier(0);   // the refill reuses the registers the stores above read
+          load_tile(set_tag, kt + 3);
+        } else if (kt + 2 < k_tiles) {
+          load_tile(set_tag, kt + 2);
+        }
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
@@ -249,13 +264,34 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     }
   };
 
-  load_tile(0);
-  store_tile(0);
-  if (k_tiles > 1) load_tile(1);
-  __syncthreads();
-  load_frags(0, 0, 0);
-  for (int kt = 0; kt + 1 < k_tiles; ++kt) k_tile(std::true_type{}, kt);
-  k_tile(std::false_type{}, k_tiles - 1);
+  if constexpr (kDeep) {
+    // tile t travels in register set (t & 1): iteration kt stores tile kt+1 and refills its set with tile kt+3
+    load_tile(Set0{}, 0);
+    store_tile(Set0{}, 0);
+    load_tile(Set1{}, 1);
+    load_tile(Set0{}, 2);
+    __syncthreads();
+    load_frags(0, 0, 0);
+    int kt = 0;
+    for (; kt + 2 < k_tiles; kt += 2) {
+      k_tile(std::true_type{}, Set1{}, kt);
+      k_tile(std::true_type{}, Set0{}, kt + 1);
+    }
+    if (kt + 1 < k_tiles) {
+      k_tile(std::true_type{}, Set1{}, kt);
+      k_tile(std::false_type{}, Set0{}, kt + 1);
+    } else {
+      k_tile(std::false_type{}, Set1{}, kt);
+    }
+  } else {
+    load_tile(Set0{}, 0);
+    store_tile(Set0{}, 0);
+    if (k_tiles > 1) load_tile(Set0{}, 1);
+    __syncthreads();
+    load_frags(0, 0, 0);
+    for (int kt = 0; kt + 1 < k_tiles; ++kt) k_tile(std::true_type{}, Set0{}, kt);
+    k_tile(std::false_type{}, Set0{}, k_tiles - 1);
+  }
 
   // Epilogue.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of its 32x32 block.
   // `exclusive`: every query's rows lie inside one wavefront's tile, so each (query, chunk) key has a single
@@ -319,7 +355,7 @@ struct KernelTimer {
   int n = 0;
 } g_timer;
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N>
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool kDeep = false>
 int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* chunk_key, int32_t M_rows,
                 int32_t C, int32_t K, int32_t blocks_per_query, int32_t exclusive, hipStream_t st) {
   if (exclusive && (BM / WAVES_M) % (blocks_per_query * 32) != 0) {
@@ -331,7 +367,7 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
   const int m_group = tiles_m;   // all M tiles of a K_r tile adjacent: measured best (groups of 1, 2, 4 lose 2-14 %)
   const int grid = 8 * ((tiles_n + 7) / 8) * tiles_m;
   const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
-  auto kern = score_gemm_kernel<T, BM, BN, WAVES_M, WAVES_N>;
+  auto kern = score_gemm_kernel<T, BM, BN, WAVES_M, WAVES_N, kDeep>;
   static bool attr_set = false;
   if (!attr_set) {
     MSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -442,13 +478,15 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
   void* qs = ws + w.off_qs;
   uint32_t* row_bits = reinterpret_cast<uint32_t*>(ws + w.off_row_bits);
   uint32_t* chunk_key = reinterpret_cast<uint32_t*>(ws + w.off_chunk_key);
-  // Tile choice by query rows: small M is HBM-bound (narrow M tile, more workgroups in flight),
-  // large M is MFMA-bound (256 x 256 tile, 8 wavefronts).  MSA_SCORE_TILE overrides for tuning.
+  // Tile choice by query rows: small M is HBM-bound (narrow M tile, more workgroups in flight, two K tiles of
+  // global loads ahead: 3 % faster than one at 16-64 rows; at 128 rows the deeper prefetch measured slower and
+  // the wider tiles spill with it), large M is MFMA-bound (256 x 256 tile, 8 wavefronts).  MSA_SCORE_TILE
+  // overrides for tuning.
   // wave_rows[v] = rows of one wavefront's tile in variant v (BM / WAVES_M).
-  static const int wave_rows[10] = {32, 64, 128, 64, 64, 64, 64, 32, 128, 64};
+  static const int wave_rows[11] = {32, 64, 128, 64, 64, 64, 64, 32, 128, 64, 32};
   const char* ev = getenv("MSA_SCORE_TILE");
-  const int variant = ev ? atoi(ev) : (w.M_rows <= 64 ? 0 : w.M_rows <= 128 ? 6 : 2);
-  if (bank->dtype == MSA_BF16 && (variant < 0 || variant > 9)) {
+  const int variant = ev ? atoi(ev) : (w.M_rows <= 64 ? 10 : w.M_rows <= 128 ? 6 : 2);
+  if (bank->dtype == MSA_BF16 && (variant < 0 || variant > 10)) {
     msa_set_error("MSA_SCORE_TILE=%d unknown", variant);
     return MSA_EINVAL;
   }
@@ -485,6 +523,9 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
 #define MSA_GEMM(BM_, BN_, WM_, WN_)                                                                              \
   launch_gemm<bf16_t, BM_, BN_, WM_, WN_>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C, \
                                           K, bpq, exclusive, st)
+#define MSA_GEMM_DEEP(BM_, BN_, WM_, WN_)                                                                 \
+  launch_gemm<bf16_t, BM_, BN_, WM_, WN_, true>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows,   \
+                                                (int32_t)bank->C, K, bpq, exclusive, st)
     switch (variant) {
       case 0: rc = MSA_GEMM(64, 128, 2, 2); break;
       case 1: rc = MSA_GEMM(128, 256, 2, 4); break;
@@ -496,9 +537,11 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
       case 7: rc = MSA_GEMM(128, 256, 4, 2); break;
       case 8: rc = MSA_GEMM(128, 256, 1, 8); break;
       case 9: rc = MSA_GEMM(128, 192, 2, 2); break;
+      case 10: rc = MSA_GEMM_DEEP(64, 128, 2, 2); break;
       default: msa_set_error("MSA_SCORE_TILE=%d unknown", variant); return MSA_EINVAL;
     }
 #undef MSA_GEMM
+#undef MSA_GEMM_DEEP
   } else {
     rc = launch_gemm<float, 128, 128, 2, 2>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C, K,
                                             bpq, exclusive, st);

@@ -422,3 +422,17 @@ def test_topk_windows_long_documents_and_filtering(ops, topk):
     assert torch.equal(got, wi[:, :n_win]), (got, wi[:, :n_win])
     for b in range(B):
         assert sorted(got[b].tolist()) == sorted(edge[b::B][:n_win])
+
+
+@pytest.mark.parametrize("Hq,Hkv", [(4, 1), (8, 2), (32, 8), (24, 3)])
+@pytest.mark.parametrize("B,S", [(1, 40), (2, 20), (1, 5)])
+def test_scores_at_most_64_query_rows(ops, Hq, Hkv, B, S):
+    """The narrow tile with two K tiles of loads in flight: even and odd K-tile counts (Hkv * 128 / 64), a bank that
+    is not a multiple of the tile, masked tokens."""
+    say(f"narrow tile Hq={Hq} Hkv={Hkv} B={B} S={S}")
+    bank, kr, dco, _ = _bank(ops, [3, 1, 7, 2, 9, 4, 5] * 53, Hkv, torch.bfloat16, 950 + Hkv)
+    q = _randn((B, S, Hq, 128), 951 + S, torch.bfloat16)
+    mask = torch.ones(B, S, dtype=torch.bool)
+    mask[0, ::3] = False
+    got = ops.chunk_scores(bank, 0, q.cuda(), mask.cuda())
+    assert cf.rel_err(got.cpu(), cf.chunk_scores(q, mask, kr, "cosine")) < 1e-2

@@ -148,7 +148,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   const int rem = within % per_group;
   const int tile_n = (blockIdx.x % 8) * n_per_xcd + rem / m_group;
   const int tile_m = (within / per_group) * m_group + rem % m_group;
-  if (tile_n >= tiles_n) return;
+  if (tile_n >= tiles_n || tile_m >= tiles_m) return;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -364,8 +364,16 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
     return MSA_EINVAL;
   }
   const int tiles_m = (M_rows + BM - 1) / BM, tiles_n = (C + BN - 1) / BN;
-  const int m_group = tiles_m;   // all M tiles of a K_r tile adjacent: measured best (groups of 1, 2, 4 lose 2-14 %)
-  const int grid = 8 * ((tiles_n + 7) / 8) * tiles_m;
+  // M tiles are walked in groups of 8 per K_r tile: a group's query rows (4 MiB in bf16) are what an XCD's L2
+  // holds.  At 8 M tiles that is all of them (groups of 1, 2, 4 lose 2-14 % there); with 16 M tiles groups of 8
+  // measured 1.4 % faster than one group, with 256 (a 64k-row prefill batch) 4 %.  MSA_SCORE_MGROUP overrides.
+  int m_group = std::min(tiles_m, 8);
+  if (const char* mg = getenv("MSA_SCORE_MGROUP")) {
+    const int v = atoi(mg);
+    if (v > 0) m_group = std::min(v, tiles_m);
+  }
+  const int m_groups = (tiles_m + m_group - 1) / m_group;
+  const int grid = 8 * ((tiles_n + 7) / 8) * m_groups * m_group;
   const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
   auto kern = score_gemm_kernel<T, BM, BN, WAVES_M, WAVES_N, kDeep>;
   static bool attr_set = false;

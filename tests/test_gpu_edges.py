@@ -360,7 +360,7 @@ def test_greedy_sample_against_argmax(ops, dtype, B, V):
     assert tok2.cpu().tolist() == want.tolist()
 
 
-@pytest.mark.parametrize("B,S", [(16, 128), (4, 64), (3, 96), (2, 200), (1, 128), (5, 32), (9, 1)])
+@pytest.mark.parametrize("B,S", [(16, 128), (4, 64), (3, 96), (2, 200), (1, 128), (5, 32), (9, 1), (20, 128)])
 def test_score_epilogue_forms_on_a_dirty_workspace(ops, B, S):
     """Queries that fit one wavefront's tile are stored by a single writer into a key plane nobody cleared; the others
     combine through atomicMax on a cleared plane.  Both must give the oracle's scores whatever the workspace held

@@ -245,7 +245,8 @@ int msa_greedy_sample(const void* logits, int32_t dtype, int32_t B, int64_t V, v
  * K a multiple of 128, w in torch.nn.Linear layout (the F.linear calls behind q/k/v/o_proj and the MLP at
  * src/msa/memory_sparse_attention.py:125-127, 405 when one token per sample is decoded).  The weight matrix is
  * streamed from HBM once.  epilogue 0: plain; 1: y = residual + bf16(x w^T) (residual [M, N]); 2: w holds
- * alternating 16-row groups of gate and up rows (N = 2 I) and y[M, I] = silu(gate) * up, both products rounded
+ * alternating 8-row groups of gate and up rows (rows 16 i .. 16 i + 7 are gate rows 8 i .. 8 i + 7, the next eight
+ * the same up rows; N = 2 I, I a multiple of 8) and y[M, I] = silu(gate) * up, both products rounded
  * to bf16 first as the unfused sequence does.  With norm_w [K] the RMSNorm in front of the projection is folded
  * in: the operand is bf16(x * rsqrt(mean(x^2) + eps) * norm_w) (input_layernorm / post_attention_layernorm of
  * src/msa/model.py's decoder layer).  Partial sums are added in a fixed order: results are

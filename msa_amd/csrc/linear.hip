@@ -152,20 +152,21 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_linear_kernel(
     }
   }
   if (kEpi == kEpiSiluMul) {
-    // row groups alternate gate, up: group 2i holds gate rows [16 i, 16 i + 16), group 2i+1 the same up rows
-    for (int r = 2 * wave; r < R; r += 2 * waves) {
-      floatx4_t gate = floatx4_t{0.f, 0.f, 0.f, 0.f}, up = gate;
-      for (int wv = 0; wv < waves; ++wv) {
-        gate += *reinterpret_cast<const floatx4_t*>(&part[((wv * R + r) * 64 + lane) * 4]);
-        up += *reinterpret_cast<const floatx4_t*>(&part[((wv * R + r + 1) * 64 + lane) * 4]);
-      }
-      const int n = ((n_base + 16 * r) >> 1) + n_l;    // output column: a pair of groups folds into one
-      if (n_base + 16 * (r + 1) + n_l >= N) continue;
+    // every 16-row group holds gate rows [8 i, 8 i + 8) in its first half and the same up rows in its second: a
+    // lane with n_l < 8 has the gate sum and takes the up sum from the lane 8 further on
+    for (int r = wave; r < R; r += waves) {
+      floatx4_t sum = floatx4_t{0.f, 0.f, 0.f, 0.f};
+      for (int wv = 0; wv < waves; ++wv) sum += *reinterpret_cast<const floatx4_t*>(&part[((wv * R + r) * 64 + lane) * 4]);
+      floatx4_t up;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) up[e] = __shfl_xor(sum[e], 8);
+      const int n = ((n_base + 16 * r) >> 1) + n_l;    // output column: a group of 16 rows folds into 8 outputs
+      if (n_l >= 8 || n_base + 16 * r + 8 + n_l >= N) continue;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int m = 4 * g + e;
         if (m >= M) continue;
-        const float a = bf16_to_f32(f32_to_bf16(gate[e] * inv[e])), b = bf16_to_f32(f32_to_bf16(up[e] * inv[e]));
+        const float a = bf16_to_f32(f32_to_bf16(sum[e] * inv[e])), b = bf16_to_f32(f32_to_bf16(up[e] * inv[e]));
         y[(int64_t)m * y_row_stride + n] = f32_to_bf16(a / (1.f + __expf(-a)) * b);
       }
     }
@@ -191,7 +192,8 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_linear_kernel(
 // whole launch.  Wavefront w owns the K slice [32 F w, 32 F (w + 1)) for every row group the workgroup visits and
 // keeps its x operands for that slice (with the RMSNorm weight folded in) in registers, so the activations are read
 // once per workgroup instead of once per row group, and far fewer workgroups have to be dispatched.  Work items are
-// pairs of row groups (32 weight rows; gate and up of the same 16 outputs for the silu epilogue), dealt round robin;
+// pairs of row groups (32 weight rows), or single row groups for the silu epilogue (8 gate rows and the same 8 up
+// rows: the finer grain matters because a launch lasts as long as its busiest compute unit), dealt round robin;
 // a step is one row group: its F weight vectors per lane are prefetched one step ahead, the partial sums meet in
 // a ring of four LDS buffers behind one barrier per step, and all threads share the work of adding them up (a fixed
 // tree) and storing the row group.  Launched with 16 wavefronts.
@@ -216,10 +218,14 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_stream_kernel(
 #pragma unroll
   for (int f = 0; f < F; ++f) xf[f] = __builtin_amdgcn_raw_buffer_load_b128(rs_x, voff, slice_off + f * 64, 0);
 
-  // this workgroup's items: blockIdx.x, blockIdx.x + gridDim.x, ...; two steps (row groups) per item
+  // this workgroup's items: blockIdx.x, blockIdx.x + gridDim.x, ...; an item is a pair of row groups (two steps), or
+  // a single row group for the silu epilogue, whose groups are complete in themselves (8 gate rows + 8 up rows)
+  constexpr int kPer = kEpi == kEpiSiluMul ? 1 : 2;
   const int my_items = n_items > (int)blockIdx.x ? (n_items - (int)blockIdx.x + (int)gridDim.x - 1) / (int)gridDim.x : 0;
-  const int n_steps = 2 * my_items;
-  auto group_of = [&](int s) { return 2 * ((int)blockIdx.x + (s >> 1) * (int)gridDim.x) + (s & 1); };
+  const int n_steps = kPer * my_items;
+  auto group_of = [&](int s) {
+    return kPer == 1 ? (int)blockIdx.x + s * (int)gridDim.x : 2 * ((int)blockIdx.x + (s >> 1) * (int)gridDim.x) + (s & 1);
+  };
   // Three register stages of weight operands, always indexed by compile-time constants: a step's loads are issued
   // two steps ahead.  Every step issues its prefetch (an empty one past the end) and the step count is padded to a
   // multiple of three, so the loop body is straight-line as far as memory instructions go and the wait counts the
@@ -308,7 +314,6 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_stream_kernel(
     *reinterpret_cast<floatx4_t*>(part + ((s & 3) * waves + wave) * 256 + lane * 4) = acc;
     __syncthreads();
     if (s >= n_steps) return;                        // padding step
-    if (kEpi == kEpiSiluMul && !(s & 1)) return;     // gate rows: stored together with the up rows of the next step
     if (!have_inv) {
       float tot = 0.f;
       for (int wv = 0; wv < waves; ++wv) tot += row_ssq[wv * 16 + o_m];
@@ -317,14 +322,14 @@ __global__ __launch_bounds__(kMaxWaves * 64) void skinny_stream_kernel(
     }
     const int gid = group_of(s);
     if constexpr (kEpi == kEpiSiluMul) {
-      // steps s - 1 and s are gate and up of the same 16 outputs
-      float g0, g1, u0, u1;
-      sum_parts(s - 1, g0, g1);
-      sum_parts(s, u0, u1);
-      if (sub != 0 || o_m >= M) return;
+      // columns 0..7 of the group are gate rows, 8..15 the same up rows: the lanes 32 further on hold the up pair
+      float g0, g1;
+      sum_parts(s, g0, g1);
+      const float u0 = __shfl_xor(g0, 32), u1 = __shfl_xor(g1, 32);
+      if (sub != 0 || o_m >= M || o_n >= 8) return;
       const float a0 = bf16_to_f32(f32_to_bf16(g0 * inv)), b0 = bf16_to_f32(f32_to_bf16(u0 * inv));
       const float a1 = bf16_to_f32(f32_to_bf16(g1 * inv)), b1 = bf16_to_f32(f32_to_bf16(u1 * inv));
-      store_pair((gid >> 1) * 16 + o_n, a0 / (1.f + __expf(-a0)) * b0, a1 / (1.f + __expf(-a1)) * b1);
+      store_pair(gid * 8 + o_n, a0 / (1.f + __expf(-a0)) * b0, a1 / (1.f + __expf(-a1)) * b1);
     } else {
       float v0, v1;
       sum_parts(s, v0, v1);
@@ -505,7 +510,7 @@ extern "C" int msa_skinny_linear(const void* x, const void* w, const void* resid
               "msa_skinny_linear: K=%d too large", K);
   MSA_REQUIRE(epilogue >= kEpiPlain && epilogue <= kEpiSiluMul, "msa_skinny_linear: epilogue %d", epilogue);
   MSA_REQUIRE((epilogue == kEpiResidual) == (residual != nullptr), "msa_skinny_linear: residual pointer and epilogue disagree");
-  MSA_REQUIRE(epilogue != kEpiSiluMul || N % 32 == 0, "msa_skinny_linear: silu-mul needs N %% 32 == 0");
+  MSA_REQUIRE(epilogue != kEpiSiluMul || N % 16 == 0, "msa_skinny_linear: silu-mul needs N %% 16 == 0");
   MSA_REQUIRE((((uintptr_t)x | (uintptr_t)w | (uintptr_t)norm_w) & 15) == 0, "msa_skinny_linear: x / w / norm_w must be 16-byte aligned");
   const int units = K / kUnit;
   MSA_REQUIRE(norm_w == nullptr || eps > 0.f, "msa_skinny_linear: folded RMSNorm needs eps > 0");
@@ -515,7 +520,7 @@ extern "C" int msa_skinny_linear(const void* x, const void* w, const void* resid
   // streaming kernel, one workgroup per compute unit at most, an equal number of items (32 rows) each.
   static const int env_stream = [] { const char* e = getenv("MSA_LINEAR_STREAM"); return e ? atoi(e) : 1; }();
   if (K == 16 * 5 * 32 && env_stream != 0) {
-    const int n_items = (N + 31) / 32;
+    const int n_items = epilogue == kEpiSiluMul ? N / 16 : (N + 31) / 32;
     const int iters = (n_items + 255) / 256;
     const int grid = (n_items + iters - 1) / iters;
     if (iters >= 2) {                                // with one item per workgroup the plain kernel does the same work

@@ -436,12 +436,13 @@ _linear_ws = {}
 
 
 def interleave_gate_up(gate_w: torch.Tensor, up_w: torch.Tensor) -> torch.Tensor:
-    """``[2 I, K]`` weight with alternating 16-row groups of gate and up rows: the layout the silu-mul epilogue
-    of ``skinny_linear`` expects (``I`` a multiple of 16)."""
+    """``[2 I, K]`` weight with alternating 8-row groups of gate and up rows (rows ``16 i .. 16 i + 7`` are gate
+    rows ``8 i .. 8 i + 7``, the next 8 the same up rows): the layout the silu-mul epilogue of ``skinny_linear``
+    expects (``I`` a multiple of 8)."""
     I, K = gate_w.shape
-    if I % 16 or up_w.shape != gate_w.shape:
-        raise ValueError("gate / up weights must be [I, K] with I a multiple of 16")
-    return torch.stack([gate_w.view(I // 16, 16, K), up_w.view(I // 16, 16, K)], dim=1).reshape(2 * I, K).contiguous()
+    if I % 8 or up_w.shape != gate_w.shape:
+        raise ValueError("gate / up weights must be [I, K] with I a multiple of 8")
+    return torch.stack([gate_w.view(I // 8, 8, K), up_w.view(I // 8, 8, K)], dim=1).reshape(2 * I, K).contiguous()
 
 
 def skinny_linear(x: torch.Tensor, w: torch.Tensor, residual: Optional[torch.Tensor] = None,

@@ -155,7 +155,8 @@ def test_skinny_linear_plain_and_residual(ops, M, N, K):
     assert torch.equal(ops.skinny_linear(x.cuda(), w.cuda()).cpu(), got)
 
 
-@pytest.mark.parametrize("M,I,K", [(16, 9728, 2560), (3, 64, 256), (16, 528, 1024), (7, 8208, 2560), (16, 4112, 2560)])
+@pytest.mark.parametrize("M,I,K", [(16, 9728, 2560), (3, 64, 256), (16, 528, 1024), (7, 8208, 2560), (16, 4112, 2560),
+                                   (16, 4104, 2560), (5, 8, 128), (16, 2056, 2560)])
 def test_skinny_linear_norm_and_silu_mul(ops, M, I, K):
     say(f"skinny_linear norm + silu-mul M={M} I={I} K={K}")
     g = torch.Generator().manual_seed(I + K)
@@ -172,7 +173,7 @@ def test_skinny_linear_norm_and_silu_mul(ops, M, I, K):
     assert cf.rel_err(got, want) < 1e-2
     # and with the silu-mul epilogue over interleaved gate / up row groups
     wi = ops.interleave_gate_up(gate.cuda(), up.cuda())
-    assert wi.shape == (2 * I, K) and torch.equal(wi[:16].cpu(), gate[:16]) and torch.equal(wi[16:32].cpu(), up[:16])
+    assert wi.shape == (2 * I, K) and torch.equal(wi[:8].cpu(), gate[:8]) and torch.equal(wi[8:16].cpu(), up[:8])
     a, b = (normed @ gate.double().T).bfloat16().double(), (normed @ up.double().T).bfloat16().double()
     got = ops.skinny_linear(x.cuda(), wi, silu_mul=True, norm_weight=nw.cuda(), eps=eps).cpu()
     assert got.shape == (M, I) and cf.rel_err(got, torch.nn.functional.silu(a) * b) < 1.5e-2

@@ -515,7 +515,7 @@ def main():
         extras["e2e_sparse_decode"] = {"workload": r["config"]["workload"] + ", 10M-token bank, B=16, 4K context, greedy",
                                        "tokens_per_s": r["value"], "ms_per_decode_step": r["ms_per_decode_step"],
                                        "prefill_s": r["prefill_s"], "decode_steps": r["config"]["decode_steps"],
-                                       "decode_mode": r["decode_mode"]}
+                                       "decode_mode": r["decode_mode"], "stage1_encode": r["stage1_encode"]}
 
     out = {
         "metric": "routed queries/s at the 100M-token bank (router scoring + top-k + host gather, 18 layers)",

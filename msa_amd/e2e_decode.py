@@ -19,9 +19,9 @@ import numpy as np
 import torch
 
 from .config import GenerateConfig, MemoryConfig, ModelConfig, MSAConfig
-from .model import MSAForCausalLM
+from .model import MSAForCausalLM, encode_block
 from .msa_service import MSAService
-from .prefill import Document, num_chunks
+from .prefill import Document, num_chunks, prepare_block_inputs
 
 
 def build_service(cfg: MSAConfig, bank_tokens: int, seed: int = 0) -> MSAService:
@@ -56,6 +56,28 @@ def build_service(cfg: MSAConfig, bank_tokens: int, seed: int = 0) -> MSAService
     return svc
 
 
+def time_stage1(model: MSAForCausalLM, cfg: MSAConfig, tokens: int, seed: int = 1) -> dict:
+    """Stage 1 (encode) of one packed block of ragged documents, lengths U[256, 2048]: document-wise causal attention
+    and the pooled K / V / K_r of every layer.  Returns the second run's time (the first pays allocator warm-up)."""
+    dev = next(model.parameters()).device
+    g = np.random.default_rng(seed)
+    docs, left = [], tokens
+    while left > 0:
+        n = min(int(g.integers(256, 2049)), left)
+        docs.append(Document(doc_id=len(docs), input_ids=g.integers(0, cfg.vocab_size, size=n).tolist()))
+        left -= n
+    blk = prepare_block_inputs(docs, [1, 2, 3], cfg.msa_config.pooling_kernel_size)
+    dt = 0.0
+    for _ in range(2):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        cache = encode_block(model, blk, dev)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        del cache
+    return {"block_tokens": tokens, "documents": len(docs), "seconds": round(dt, 4), "tokens_per_s": round(tokens / dt)}
+
+
 def main(argv=None, quiet: bool = False):
     """Runs the workload and prints one JSON line (``quiet`` only returns the dict)."""
     ap = argparse.ArgumentParser()
@@ -64,6 +86,8 @@ def main(argv=None, quiet: bool = False):
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--steps", type=int, default=256)
     ap.add_argument("--layers", type=int, default=36)
+    ap.add_argument("--encode-tokens", type=int, default=32768,
+                    help="also time stage 1 (encode) on one packed block of this many tokens; 0 skips it")
     ap.add_argument("--eager", action="store_true", help="do not capture the decode step as a HIP graph")
     ap.add_argument("--verify-graph", type=int, default=0, metavar="N",
                     help="also decode N steps eagerly and require identical tokens from the graph replays")
@@ -85,6 +109,7 @@ def main(argv=None, quiet: bool = False):
         layer.self_attn.decode_reserve = args.steps + 8
     torch.cuda.synchronize()
     setup_s = time.perf_counter() - t0
+    stage1 = time_stage1(model, cfg, args.encode_tokens) if args.encode_tokens > 0 else None
     g = torch.Generator(device=dev).manual_seed(3)
     B, S = args.batch, args.context
     ids = torch.randint(0, cfg.vocab_size, (B, S), generator=g, device=dev)
@@ -112,6 +137,7 @@ def main(argv=None, quiet: bool = False):
                       "layers": args.layers, "bank_tokens": args.bank_tokens, "batch": B, "context_tokens": S,
                       "decode_steps": args.steps, "top_k": cfg.msa_config.top_k_docs,
                       "kv_rows_last_router_layer": kv[:4]},
+           "stage1_encode": stage1,
            "decode_mode": "eager" if args.eager else "hip graph replay", "graph_equals_eager": verified,
            "generated_shape": list(toks.shape)}
     del model, svc, cache

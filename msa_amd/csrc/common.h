@@ -2,6 +2,8 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stdint.h>
 #include <stdio.h>
 
@@ -28,6 +30,16 @@ void msa_set_error(const char* fmt, ...);
   } while (0)
 
 #define MSA_LAUNCH_CHECK() MSA_HIP(hipGetLastError())
+
+// A kernel that needs more dynamic LDS than the default limit gets its limit raised before its first launch, once
+// per process whatever the number of host threads (the library drives one device per process).  `done` is the
+// per-kernel flag of the call site.
+static inline hipError_t raise_dynamic_lds_limit(std::atomic<int>& done, const void* kernel, int bytes) {
+  if (done.load(std::memory_order_acquire)) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess) done.store(1, std::memory_order_release);   // two threads racing here set the same value twice
+  return e;
+}
 
 typedef uint16_t bf16_t;  // raw bf16 bits
 

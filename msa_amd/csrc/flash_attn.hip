@@ -353,12 +353,8 @@ int flash_launch_g(const void* q, const int32_t* cu_q, const void* k, const void
   MSA_REQUIRE(blocks < (int64_t)1 << 31, "flash attention: too many query rows");
   dim3 grid((unsigned)blocks, (unsigned)Hkv, kSplit ? (unsigned)plan.n_split : 1u);
   auto kern = flash_attn_kernel<G, kSplit>;
-  static bool attr_set = false;            // two tiles of K and V exceed the default dynamic LDS limit
-  if (!attr_set) {
-    MSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                kLdsBytes));
-    attr_set = true;
-  }
+  static std::atomic<int> lds_limit_raised{0};   // two tiles of K and V exceed the default dynamic LDS limit
+  MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(kern), kLdsBytes));
   kern<<<grid, kWaves * 64, kLdsBytes, st>>>(static_cast<const bf16_t*>(q), cu_q, static_cast<const bf16_t*>(k),
                                              static_cast<const bf16_t*>(v), kv_off, kv_len, B, Hq, Hkv,
                                              scale * 1.4426950408889634f, causal, static_cast<bf16_t*>(out),

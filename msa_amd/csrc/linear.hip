@@ -357,12 +357,9 @@ int launch_stream(const void* x, const void* w, const void* residual, const void
                   int32_t N, int32_t K, int waves, int grid, int n_items, hipStream_t st) {
   const size_t lds = (size_t)waves * (4 * 256 + 16) * sizeof(float);
   const int64_t y_stride = kEpi == kEpiSiluMul ? N / 2 : N;
-  static bool attr_set = false;              // 16 wavefronts need 65 KB, just past the default dynamic LDS limit
-  if (!attr_set) {
-    MSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_stream_kernel<F, kEpi, kNorm>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, kMaxWaves * (4 * 256 + 16) * (int)sizeof(float)));
-    attr_set = true;
-  }
+  static std::atomic<int> lds_limit_raised{0};   // 16 wavefronts need 65 KB, just past the default dynamic LDS limit
+  MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(skinny_stream_kernel<F, kEpi, kNorm>),
+                                  kMaxWaves * (4 * 256 + 16) * (int)sizeof(float)));
   skinny_stream_kernel<F, kEpi, kNorm><<<grid, waves * 64, lds, st>>>(
       static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), static_cast<const bf16_t*>(residual),
       static_cast<const bf16_t*>(norm_w), eps, static_cast<bf16_t*>(y), M, N, K, y_stride, n_items);

@@ -376,12 +376,8 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
   const int grid = 8 * ((tiles_n + 7) / 8) * m_groups * m_group;
   const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
   auto kern = score_gemm_kernel<T, BM, BN, WAVES_M, WAVES_N, kDeep>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    MSA_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)lds));
-    attr_set = true;
-  }
+  static std::atomic<int> lds_limit_raised{0};
+  MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(kern), (int)lds));
   const bool timed = g_timer.n < g_timer.cap;
   if (timed) MSA_HIP(hipEventRecord(g_timer.start[g_timer.n], st));
   kern<<<grid, WAVES_M * WAVES_N * 64, lds, st>>>(static_cast<const T*>(qs), static_cast<const T*>(kr), row_bits,

@@ -89,12 +89,18 @@ __global__ void qk_norm_rope_kernel(const T* __restrict__ q, const T* __restrict
   const float inv = rsqrtf(row16_sum(ssq) * (1.0f / kHeadDim) + eps);
   const int64_t p = min((int64_t)max((int64_t)0, pos[n]), (int64_t)rope_rows - 1);
   const int f = 8 * (j & 7);                    // frequency index of this lane's first element
+  // lanes j and j ^ 8 need the same eight cosines and sines: the lower lane fetches the cosines, the upper one the
+  // sines, and they swap (the table reads were four of a lane's seven memory instructions)
+  const float* tab = (j < 8 ? cos_t : sin_t) + p * 64 + f;
+  const float4 t0 = *reinterpret_cast<const float4*>(tab), t1 = *reinterpret_cast<const float4*>(tab + 4);
+  const float mine[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
   float out[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const float y = x[i] * inv * w[i];
     const float other = row16_ror8(y);          // the paired dim (d + 64 for j < 8, d - 64 for j >= 8)
-    const float c = cos_t[p * 64 + f + i], s = sin_t[p * 64 + f + i];
+    const float theirs = row16_ror8(mine[i]);
+    const float c = j < 8 ? mine[i] : theirs, s = j < 8 ? theirs : mine[i];
     out[i] = j < 8 ? y * c - other * s : y * c + other * s;
   }
   if (is_q || keep_kv) store8g<T>(dst + 8 * j, out);
@@ -288,6 +294,7 @@ static int qk_norm_rope_launch(const char* who, const void* q, const void* k, co
   MSA_REQUIRE(D == kHeadDim, "%s: head dim %d unsupported (need %d)", who, D, kHeadDim);
   MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "%s: bad dtype %d", who, dtype);
   MSA_REQUIRE(N > 0 && N < (int64_t)1 << 31, "%s: N=%lld out of range", who, (long long)N);
+  MSA_REQUIRE((((uintptr_t)rope_cos | (uintptr_t)rope_sin) & 15) == 0, "%s: rotary tables must be 16-byte aligned", who);
   MSA_REQUIRE((v == nullptr) == (v_out == nullptr), "%s: v and v_out go together", who);
   const int heads = Hq + Hkv + (v ? Hkv : 0);
   MSA_REQUIRE(Hq > 0 && Hkv > 0 && heads * 16 <= 1024, "%s: Hq=%d Hkv=%d unsupported", who, Hq, Hkv);

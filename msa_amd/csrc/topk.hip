@@ -8,10 +8,7 @@
 
 namespace {
 
-#ifndef TOPK_WAVES
-#define TOPK_WAVES 4
-#endif
-constexpr int kWaves = TOPK_WAVES;
+constexpr int kWaves = 4;
 
 __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int m) {
   return (uint64_t)__shfl_xor((unsigned long long)v, m);

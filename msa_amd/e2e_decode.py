@@ -88,6 +88,7 @@ def main(argv=None, quiet: bool = False):
     ap.add_argument("--layers", type=int, default=36)
     ap.add_argument("--encode-tokens", type=int, default=32768,
                     help="also time stage 1 (encode) on one packed block of this many tokens; 0 skips it")
+    ap.add_argument("--encode-only", action="store_true", help="time stage 1 (encode) and stop: no bank, no decode")
     ap.add_argument("--eager", action="store_true", help="do not capture the decode step as a HIP graph")
     ap.add_argument("--verify-graph", type=int, default=0, metavar="N",
                     help="also decode N steps eagerly and require identical tokens from the graph replays")
@@ -103,6 +104,14 @@ def main(argv=None, quiet: bool = False):
     with torch.device(dev):
         model = MSAForCausalLM(cfg).to(torch.bfloat16)
     model.init_random_(0.02, seed=0).eval()
+    if args.encode_only:
+        out = {"metric": "stage-1 encode tokens/s (one packed block)", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic",
+               "config": {"workload": "Qwen3-4B shape, random init, ragged documents U[256, 2048]", "layers": args.layers},
+               **time_stage1(model, cfg, max(args.encode_tokens, 1024))}
+        out["value"] = out["tokens_per_s"]
+        if not quiet:
+            print(json.dumps(out), flush=True)
+        return out
     svc = build_service(cfg, args.bank_tokens)
     svc.setup_memory_client(model)
     for layer in model.model.layers:

@@ -311,6 +311,9 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
         const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(k_lane + rb * 32 * kTileStride + ks * 32);
         s0[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], s0[rb], 0, 0, 0);
       }
+    // the first step overwrites K slot 0 (with tile first + 2) before its own barrier: every wavefront must have
+    // finished the reads of slot 0 above before any wavefront gets there
+    __syncthreads();
     for (int t = first_tile; t < n_tiles; t += 2) {
       step(t, s0, s1);
       if (t + 1 < n_tiles) step(t + 1, s1, s0);

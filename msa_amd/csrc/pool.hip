@@ -116,8 +116,9 @@ __global__ __launch_bounds__(kThreads, 2) void pool_chunks_kernel(PoolArgs a) {
         const_cast<char*>(chunk_base) + (int64_t)base * row_bytes, 0, rows * row_bytes, 0x00020000);
 #pragma unroll
     for (int q = 0; q < kRows; ++q) {
-      lo[q].load(group, voff, q * q_stride);
-      hi[q].load(group, voff + 64 * (int)sizeof(T), q * q_stride);
+      // the row displacement rides in the vector offset, the operand the range check is defined on
+      lo[q].load(group, voff + q * q_stride, 0);
+      hi[q].load(group, voff + q * q_stride + 64 * (int)sizeof(T), 0);
     }
   };
   issue(lo_a, hi_a, 0);

@@ -131,11 +131,32 @@ class MemorySparseAttention(nn.Module):
         return self._qkv_weight
 
     def _rope_tables(self, device):
-        rows = min(self.config.max_position_embeddings, 32768)
+        # one row per position the configuration allows; positions beyond it are refused where they are made
+        # (check_positions), not clamped in the kernels
+        rows = int(self.config.max_position_embeddings)
         key = (device, rows, float(self.config.rope_theta))
         if key not in _ROPE_TABLES:
             _ROPE_TABLES[key] = ops.rope_tables(rows, self.head_dim, self.config.rope_theta, device=device)
         return _ROPE_TABLES[key]
+
+    def check_positions(self, last_position: int) -> None:
+        """Raises when a position would fall outside the rotary tables (the reference computes cos / sin for any
+        position; here they are tabulated up to ``max_position_embeddings``)."""
+        rows = int(self.config.max_position_embeddings)
+        if last_position >= rows:
+            raise ValueError(f"position {last_position} is beyond max_position_embeddings = {rows}")
+
+    @staticmethod
+    def _claim_rows(ck: dict, n_new: int) -> None:
+        """Books ``n_new`` more rows per sample against the free rows behind the stage-2 context; raises instead
+        of letting the append kernels drop rows (the reference grows its cache without limit, :372-373)."""
+        left = ck.get("rows_free")
+        if left is None:
+            return
+        if n_new > left:
+            raise RuntimeError(f"compact KV cache is full: {n_new} new rows per sample, {left} free "
+                               f"(raise decode_reserve before stage 2)")
+        ck["rows_free"] = left - n_new
 
     def decode_rows(self, residual, norm_weight, eps, position_ids, cache):
         """The decode step of :meth:`_generate` on the residual stream ``[B, hidden]`` (B <= 16, bf16) with the
@@ -146,6 +167,7 @@ class MemorySparseAttention(nn.Module):
         ck = cache.cache_kwargs[self.layer_idx]
         if "compacked_key_cache" not in ck:
             raise ValueError("compact KV cache not found: did prefill stage 2 run?")
+        self._claim_rows(ck, 1)
         qkv = ops.skinny_linear(residual, self._fused_weight(residual.device), norm_weight=norm_weight, eps=eps)
         kc, vc, kv_len = ck["compacked_key_cache"], ck["compacked_value_cache"], ck["kv_lengths"]
         if Hq // Hkv in (4, 8) and kc.dim() == 4 and kc.is_contiguous() and vc.is_contiguous():
@@ -246,7 +268,8 @@ class MemorySparseAttention(nn.Module):
                 # native client: routing, gather plan and host->device gather are enqueued without any host sync
                 mem_k, mem_v, cu_sel, scores, gids = self.memory_client.doc_query_device(rq.contiguous(), query_mask,
                                                                                          self.layer_idx, fused)
-                max_sel = self.top_k_docs * self.memory_client.bank.max_doc_chunks
+                # the same k the client sized its gather buffers from (its own top-k setting, not this layer's)
+                max_sel = gids.shape[1] * self.memory_client.bank.max_doc_chunks
             else:
                 mem_k, mem_v, scores, n_sel, gids = self.memory_client.doc_query(rq.transpose(1, 2), query_mask,
                                                                                  self.layer_idx)
@@ -273,7 +296,7 @@ class MemorySparseAttention(nn.Module):
             attn = torch.zeros((B, S, Hq * D), device=dev, dtype=dtype)
             attn[valid] = out_rows.view(-1, Hq * D)
         ck.update({"compacked_key_cache": kc, "compacked_value_cache": vc, "kv_lengths": kv_len, "kv_offsets": kv_off,
-                   "kv_capacity": Lcap})
+                   "kv_capacity": Lcap, "rows_free": self.decode_reserve})
         cache.record_kwargs(self.layer_idx, ck)
         return self.o_proj(attn), None
 
@@ -296,14 +319,14 @@ class MemorySparseAttention(nn.Module):
             if n_host is None or len(n_host) != B:
                 n_host = n_new.tolist()
             cu_new = F.pad(n_new.cumsum(0), (1, 0)).to(torch.int32)
+            self._claim_rows(ck, max(n_host))
             ops.cache_append_rows(k[valid], v[valid], cu_new, max(n_host), kc, vc, kv_len)
             rows = ops.sparse_attn(q[valid], kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), ck["kv_offsets"], kv_len,
                                    ck["kv_capacity"], cu_q=cu_new, max_sq=max(n_host), scale=self.scaling, causal=True)
             attn = torch.zeros((B, S, Hq * D), device=q.device, dtype=q.dtype)
             attn[valid] = rows.view(-1, Hq * D)
             return self.o_proj(attn), None
-        # capacity is the caller's job (rows behind the context: decode_reserve); a full cache drops the
-        # new row inside the kernel instead of writing out of bounds
+        self._claim_rows(ck, 1)
         ops.cache_append(k[:, 0].contiguous(), v[:, 0].contiguous(), kc, vc, kv_len)
         out = ops.sparse_attn(q[:, 0].contiguous(), kc.view(-1, Hkv, D), vc.view(-1, Hkv, D), ck["kv_offsets"], kv_len,
                               ck["kv_capacity"], scale=self.scaling, causal=True)

@@ -98,6 +98,10 @@ class MSAModel(nn.Module):
         h = self.embed_tokens(input_ids)
         if past_key_values is not None and attention_mask is not None and input_ids.shape[1] > 1:
             past_key_values.meta["q_lens_host"] = attention_mask.sum(dim=1).tolist()   # one sync per forward, not per layer
+            if h.is_cuda and position_ids is not None:
+                # blocks of tokens (stage 1, stage 2, injected blocks) check their positions against the rotary
+                # tables here; single-token decode steps are checked once by the generation loops
+                self.layers[0].self_attn.check_positions(int(position_ids.max()))
         if h.is_cuda:
             for layer in self.layers:
                 h = layer(h, doc_ids, attention_mask, None, past_key_values, position_ids=position_ids)
@@ -154,6 +158,7 @@ class MSAForCausalLM(nn.Module):
             cache.record_kwargs(i, {"stage": "prefill_stage2"})
         n_valid = attention_mask.sum(dim=1).tolist()
         pos = torch.tensor([query_position_ids(n, k, 3, S - n) for n in n_valid], dtype=torch.long, device=input_ids.device)
+        self.model.layers[0].self_attn.check_positions(3 + k + max(n_valid) - 1 + max_new_tokens)
         if timings is not None:
             import time
             torch.cuda.synchronize()
@@ -252,10 +257,22 @@ def generate_interleaved(model: "MSAForCausalLM", input_ids, attention_mask, doc
     for i in range(cfg.num_hidden_layers):
         cache.cache_kwargs[i]["stage"] = "generate"
     last_pos = pos[:, -1].clone()                             # position of the last token each sample has fed
+    last_pos_bound = 3 + k + max(n_valid) - 1                 # host-side bound of the same
+    attn0 = model.model.layers[0].self_attn
+    rows_free = min(layer.self_attn.decode_reserve for layer in model.model.layers)
     out = [tok]
     for step in range(1, max_new_tokens):
         blocks = inject(step, torch.cat(out, dim=1)) if inject is not None else None
         blocks = [list(b) if b else [int(t)] for b, t in zip(blocks, tok[:, 0].tolist())] if blocks is not None else None
+        # every sample's compact cache has decode_reserve free rows behind its stage-2 context: a step that would
+        # not fit is refused here, before any kernel could drop rows
+        widest = 1 if blocks is None else max(len(b) for b in blocks)
+        if widest > rows_free:
+            raise RuntimeError(f"step {step} appends {widest} rows per sample but only {rows_free} of the "
+                               f"decode_reserve rows are left; raise decode_reserve on the layers before stage 2")
+        rows_free -= widest
+        last_pos_bound += widest
+        attn0.check_positions(last_pos_bound)
         if blocks is None or all(len(b) == 1 for b in blocks):
             ids = tok if blocks is None else torch.tensor(blocks, dtype=torch.long, device=dev)
             p = (last_pos + 1).unsqueeze(1)

@@ -12,7 +12,7 @@
  *   - pointers are DEVICE pointers unless the name ends in `_host`;
  *   - `stream` is a hipStream_t passed as void* (NULL = the null stream); all work is
  *     enqueued on it and nothing synchronises unless stated;
- *   - only msa_bank_create allocates device memory (two small tables); every other entry point
+ *   - only msa_bank_create allocates device memory (three index tables); every other entry point
  *     takes its scratch as `workspace`, sized by the matching *_workspace_bytes() function;
  *   - activations are token-major [T, H, D]; pooled tensors and the bank are chunk-major
  *     [C, Hkv, D]; document indices are 0-based in bank order; D must be 128;
@@ -97,9 +97,14 @@ int msa_bank_destroy(msa_bank* bank);
  *   msa_chunk_scores writes chunk_scores[B, C] fp32 (-inf where a query has no scored token).
  *   msa_route_topk writes scores_out[B, topk] (descending; ties by lower document index),
  *   doc_out[B, topk] (0-based, -1 past the number of documents) and doc_global_out[B, topk]
- *   (doc_global_id[doc], -1 likewise).  topk <= 64. */
+ *   (doc_global_id[doc], -1 likewise).  topk <= 64.  The max over a document's chunks (:789-792,
+ *   :817-820) is taken in the scoring kernel's epilogue, so routing never writes a per-chunk plane.
+ *   msa_route_workspace_bytes covers both calls (it holds the [B, C] plane of msa_chunk_scores);
+ *   msa_route_topk alone needs only msa_route_topk_workspace_bytes. */
 size_t msa_route_workspace_bytes(int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D,
                                  int64_t C, int64_t n_docs, int32_t topk);
+size_t msa_route_topk_workspace_bytes(int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D,
+                                      int64_t n_docs, int32_t topk);
 int msa_chunk_scores(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8,
                      int32_t B, int32_t S, int32_t Hq, int32_t mode, float scale,
                      float* chunk_scores, void* workspace, size_t workspace_bytes, void* stream);
@@ -124,7 +129,9 @@ int msa_profile_collect(float* ms_host, int32_t cap, int32_t* n_out);
  *   ascending bank order, each once.  msa_gather_plan fills cu_sel_host[B+1] (prefix sums of
  *   selected chunk counts).  msa_gather_kv enqueues one hipMemcpyAsync per contiguous document
  *   run and tensor on `copy_stream` into k_out / v_out [cu_sel[B], Hkv, D]; the caller orders
- *   consumers after the stream (event or synchronise). */
+ *   consumers after the stream (event or synchronise).  A document selected by several samples is
+ *   read from the host once (the batch-wide unique() of :1214); the other samples' rows are
+ *   device-to-device copies of the first on the same stream. */
 int msa_gather_plan(const msa_bank* bank, const int32_t* doc_sel_host, int32_t B, int32_t k,
                     int64_t* cu_sel_host);
 int msa_gather_kv(const msa_bank* bank, int32_t layer, const int32_t* doc_sel_host, int32_t B,
@@ -134,8 +141,9 @@ int msa_gather_kv(const msa_bank* bank, int32_t layer, const int32_t* doc_sel_ho
 /* Device-side variant of the same gather: the selection stays on the device (doc_sel[B, k] int32, e.g. msa_route_topk's
  * doc_out; -1 or out-of-range entries are skipped), a planning kernel sorts / de-duplicates it per sample and writes
  * cu_sel[B+1] (device int32), and a copy kernel reads the rows straight from the pinned host bank.  Nothing
- * synchronises and nothing is copied to the host; rows past out_capacity_chunks are dropped, so size the outputs for
- * B * k * (largest document's chunks).  k <= 64. */
+ * synchronises and nothing is copied to the host; rows past out_capacity_chunks are dropped and cu_sel stops at that
+ * capacity, so size the outputs for B * k * (largest document's chunks).  While B * k <= 2048 a document selected by
+ * several samples is read from the host once and copied on the device for the others.  k <= 64. */
 size_t msa_gather_device_workspace_bytes(int32_t B, int32_t k);
 int msa_gather_kv_device(const msa_bank* bank, int32_t layer, const int32_t* doc_sel, int32_t B,
                          int32_t k, void* k_out, void* v_out, int64_t out_capacity_chunks,

@@ -1,7 +1,10 @@
-// Gather of the selected documents' pooled K / V from pinned host memory (host code only).
+// Gather of the selected documents' pooled K / V from pinned host memory.
 // A document's chunks are contiguous rows of the chunk-major bank, so every document — and every
 // run of bank-adjacent documents — is one hipMemcpyAsync per tensor on the caller's copy stream.
+// A document picked by several samples of the batch crosses the host link once: later samples copy its
+// rows from the first sample's segment on the device (the batch-wide unique() of src/msa_service.py:1214).
 #include <algorithm>
+#include <unordered_map>
 #include <vector>
 
 #include "common.h"
@@ -72,13 +75,31 @@ extern "C" int msa_gather_kv(const msa_bank* bank, int32_t layer, const int32_t*
   MSA_REQUIRE(total == 0 || (k_out && v_out), "msa_gather_kv: null output");
 
   int64_t out_row = 0;
+  std::unordered_map<int32_t, int64_t> first_row;        // document -> output row of its first copy in this batch
   for (int32_t b = 0; b < B; ++b) {
     sample_docs(bank, doc_sel_host + (int64_t)b * k, k, docs);
     size_t i = 0;
     while (i < docs.size()) {
-      size_t j = i;
-      while (j + 1 < docs.size() && docs[j + 1] == docs[j] + 1) ++j;   // bank-adjacent documents: one run
-      const int64_t c0 = bank->doc_chunk_off_host[docs[i]], c1 = bank->doc_chunk_off_host[docs[j] + 1];
+      const int64_t c0 = bank->doc_chunk_off_host[docs[i]];
+      auto seen = first_row.find(docs[i]);
+      if (seen != first_row.end()) {                     // fetched for an earlier sample: device-to-device
+        const int64_t n = bank->doc_chunk_off_host[docs[i] + 1] - c0;
+        const size_t bytes = (size_t)n * row_bytes;
+        MSA_HIP(hipMemcpyAsync(kdst + out_row * row_bytes, kdst + seen->second * row_bytes, bytes,
+                               hipMemcpyDeviceToDevice, st));
+        MSA_HIP(hipMemcpyAsync(vdst + out_row * row_bytes, vdst + seen->second * row_bytes, bytes,
+                               hipMemcpyDeviceToDevice, st));
+        out_row += n;
+        ++i;
+        continue;
+      }
+      size_t j = i;                                      // bank-adjacent documents not seen before: one run
+      first_row.emplace(docs[i], out_row);
+      while (j + 1 < docs.size() && docs[j + 1] == docs[j] + 1 && first_row.find(docs[j + 1]) == first_row.end()) {
+        ++j;
+        first_row.emplace(docs[j], out_row + (bank->doc_chunk_off_host[docs[j]] - c0));
+      }
+      const int64_t c1 = bank->doc_chunk_off_host[docs[j] + 1];
       const size_t bytes = (size_t)(c1 - c0) * row_bytes;
       MSA_HIP(hipMemcpyAsync(kdst + out_row * row_bytes, ksrc + c0 * row_bytes, bytes, hipMemcpyHostToDevice, st));
       MSA_HIP(hipMemcpyAsync(vdst + out_row * row_bytes, vsrc + c0 * row_bytes, bytes, hipMemcpyHostToDevice, st));
@@ -93,23 +114,32 @@ extern "C" int msa_gather_kv(const msa_bank* bank, int32_t layer, const int32_t*
 // Device-side gather: no ids on the host, no per-document copies.  A one-workgroup planning
 // kernel sorts and de-duplicates each sample's selection (one wavefront per sample, bitonic
 // network over the <= 64 picks), prefix-sums the chunk counts into cu_sel and emits one
-// (source chunk, rows, destination row) entry per kept document; a copy kernel then pulls the
-// rows straight out of the pinned host bank (the pointers are device-visible) with 16-byte loads.
+// (source chunk, rows, destination row, device source row) entry per kept document; a copy kernel
+// then pulls the rows straight out of the pinned host bank (the pointers are device-visible) with
+// 16-byte loads.  A document that an earlier sample of the batch also picked is not read from the host
+// again: its entry names the earlier copy's rows and a second launch copies them on the device.
 // ------------------------------------------------------------------------------------------
 namespace {
 
 constexpr int kPlanWaves = 4;
+constexpr int kPlanInts = 4;            // ints per plan entry
+constexpr int kDedupMaxEntries = 2048;  // batch-wide de-duplication runs while B * k fits this many LDS slots
+constexpr int32_t kNoDoc = 0x7fffffff;
 
 __global__ __launch_bounds__(kPlanWaves * 64) void gather_plan_kernel(const int32_t* __restrict__ doc_sel,
                                                                       const int32_t* __restrict__ doc_chunk_off,
                                                                       int32_t n_docs, int32_t B, int32_t k,
+                                                                      int32_t capacity_rows, int32_t dedup,
                                                                       int32_t* __restrict__ cu_sel,
-                                                                      int32_t* __restrict__ plan /* [B*k][3] */) {
-  extern __shared__ int32_t totals[];          // [B + 1]
+                                                                      int32_t* __restrict__ plan /* [B*k][4] */) {
+  extern __shared__ int32_t smem[];            // totals [B + 1] | sorted documents [B * k] | destination rows [B * k]
+  int32_t* totals = smem;
+  int32_t* s_doc = smem + (B + 1);
+  int32_t* s_dst = s_doc + (dedup ? B * k : 0);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   // pass 1 and 2 share this per-sample routine: sorted unique documents in lanes, chunk counts, in-sample offsets
   auto sample = [&](int b, int32_t& d_out, int32_t& n_out, int32_t& off_out) -> int32_t {
-    int32_t d = 0x7fffffff;
+    int32_t d = kNoDoc;
     if (lane < k) {
       const int32_t x = doc_sel[(int64_t)b * k + lane];
       if (x >= 0 && x < n_docs) d = x;
@@ -123,7 +153,7 @@ __global__ __launch_bounds__(kPlanWaves * 64) void gather_plan_kernel(const int3
         d = (lower == asc) ? min(d, o) : max(d, o);
       }
     const int32_t prev = __shfl_up(d, 1);
-    const bool keep = d != 0x7fffffff && (lane == 0 || prev != d);
+    const bool keep = d != kNoDoc && (lane == 0 || prev != d);
     int32_t n = keep ? doc_chunk_off[d + 1] - doc_chunk_off[d] : 0;
     int32_t incl = n;
 #pragma unroll
@@ -146,30 +176,57 @@ __global__ __launch_bounds__(kPlanWaves * 64) void gather_plan_kernel(const int3
     for (int b = 0; b < B; ++b) { run += totals[b + 1]; totals[b + 1] = run; }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i <= B; i += kPlanWaves * 64) cu_sel[i] = totals[i];
+  // rows past the output's capacity are never written by the copy kernel: the prefix sums stop there too, so a
+  // consumer of cu_sel never addresses a row that was not filled
+  for (int i = threadIdx.x; i <= B; i += kPlanWaves * 64) cu_sel[i] = min(totals[i], capacity_rows);
   for (int b = wave; b < B; b += kPlanWaves) {
     int32_t d, n, off;
     sample(b, d, n, off);
     if (lane < k) {
-      int32_t* e = plan + ((int64_t)b * k + lane) * 3;
+      int32_t* e = plan + ((int64_t)b * k + lane) * kPlanInts;
       e[0] = d >= 0 ? doc_chunk_off[d] : 0;
       e[1] = n;
       e[2] = totals[b] + off;
+      e[3] = -1;
+      if (dedup) {                               // documents dropped as duplicates inside the sample sort last
+        s_doc[b * k + lane] = d >= 0 ? d : kNoDoc;
+        s_dst[b * k + lane] = totals[b] + off;
+      }
     }
+  }
+  if (!dedup) return;                            // uniform over the workgroup
+  __syncthreads();
+  // an entry whose document an earlier sample also holds copies from that sample's rows instead of the host.
+  // s_doc rows are ascending except that in-sample duplicates were replaced by kNoDoc in place, so the search
+  // below is linear over the k slots (k <= 64).
+  for (int i = threadIdx.x; i < B * k; i += kPlanWaves * 64) {
+    const int32_t d = s_doc[i];
+    if (d == kNoDoc) continue;
+    const int b = i / k;
+    int32_t from = -1;
+    for (int b2 = 0; b2 < b && from < 0; ++b2)
+      for (int j = 0; j < k; ++j)
+        if (s_doc[b2 * k + j] == d) { from = s_dst[b2 * k + j]; break; }
+    if (from >= 0) plan[(int64_t)i * kPlanInts + 3] = from;
   }
 }
 
-// grid.x = plan entry, grid.y = row group; 128 lanes move one 2 KB row of K and of V per step.
+// grid.x = plan entry, grid.y = row group; 128 lanes move one row of K and of V per step.
+// kFromDevice = false: entries without an earlier copy, rows read from the pinned host bank;
+// kFromDevice = true: the others, rows read from the earlier copy inside the output itself.
+template <bool kFromDevice>
 __global__ __launch_bounds__(128) void gather_copy_kernel(const uint4* __restrict__ k_src, const uint4* __restrict__ v_src,
                                                           const int32_t* __restrict__ plan, int32_t row_vecs,
-                                                          int64_t capacity_rows, uint4* __restrict__ k_dst,
-                                                          uint4* __restrict__ v_dst) {
-  const int32_t* e = plan + (int64_t)blockIdx.x * 3;
-  const int32_t src0 = e[0], n = e[1], dst0 = e[2];
+                                                          int64_t capacity_rows, uint4* k_dst, uint4* v_dst) {
+  const int32_t* e = plan + (int64_t)blockIdx.x * kPlanInts;
+  const int32_t n = e[1], dst0 = e[2], from = e[3];
+  if ((from >= 0) != kFromDevice) return;
+  const int32_t src0 = kFromDevice ? from : e[0];
   for (int r = blockIdx.y; r < n; r += gridDim.y) {
     if ((int64_t)dst0 + r >= capacity_rows) return;
-    const uint4* ks = k_src + ((int64_t)src0 + r) * row_vecs;
-    const uint4* vs = v_src + ((int64_t)src0 + r) * row_vecs;
+    if (kFromDevice && (int64_t)src0 + r >= capacity_rows) return;
+    const uint4* ks = (kFromDevice ? k_dst : k_src) + ((int64_t)src0 + r) * row_vecs;
+    const uint4* vs = (kFromDevice ? v_dst : v_src) + ((int64_t)src0 + r) * row_vecs;
     uint4* kd = k_dst + ((int64_t)dst0 + r) * row_vecs;
     uint4* vd = v_dst + ((int64_t)dst0 + r) * row_vecs;
     for (int i = threadIdx.x; i < row_vecs; i += 128) { kd[i] = ks[i]; vd[i] = vs[i]; }
@@ -179,7 +236,7 @@ __global__ __launch_bounds__(128) void gather_copy_kernel(const uint4* __restric
 }  // namespace
 
 extern "C" size_t msa_gather_device_workspace_bytes(int32_t B, int32_t k) {
-  return B > 0 && k > 0 ? align_up((size_t)B * k * 3 * sizeof(int32_t), 256) : 0;
+  return B > 0 && k > 0 ? align_up((size_t)B * k * kPlanInts * sizeof(int32_t), 256) : 0;
 }
 
 extern "C" int msa_gather_kv_device(const msa_bank* bank, int32_t layer, const int32_t* doc_sel, int32_t B, int32_t k,
@@ -200,14 +257,23 @@ extern "C" int msa_gather_kv_device(const msa_bank* bank, int32_t layer, const i
   }
   hipStream_t st = as_stream(stream);
   int32_t* plan = static_cast<int32_t*>(workspace);
-  gather_plan_kernel<<<1, kPlanWaves * 64, (size_t)(B + 1) * sizeof(int32_t), st>>>(
-      doc_sel, bank->doc_chunk_off_dev, (int32_t)bank->n_docs, B, k, cu_sel, plan);
+  const int32_t dedup = B > 1 && B * k <= kDedupMaxEntries ? 1 : 0;
+  const int32_t cap32 = (int32_t)std::min<int64_t>(out_capacity_chunks, 0x7fffffff);
+  const size_t lds = (size_t)(B + 1 + (dedup ? 2 * B * k : 0)) * sizeof(int32_t);
+  gather_plan_kernel<<<1, kPlanWaves * 64, lds, st>>>(doc_sel, bank->doc_chunk_off_dev, (int32_t)bank->n_docs, B, k,
+                                                      cap32, dedup, cu_sel, plan);
   MSA_LAUNCH_CHECK();
   const int32_t row_vecs = (int32_t)((size_t)bank->Hkv * bank->D * elem_bytes(bank->dtype) / 16);
   dim3 grid((unsigned)(B * k), 8);
-  gather_copy_kernel<<<grid, 128, 0, st>>>(static_cast<const uint4*>(bank->k_host[layer]),
-                                           static_cast<const uint4*>(bank->v_host[layer]), plan, row_vecs,
-                                           out_capacity_chunks, static_cast<uint4*>(k_out), static_cast<uint4*>(v_out));
+  gather_copy_kernel<false><<<grid, 128, 0, st>>>(static_cast<const uint4*>(bank->k_host[layer]),
+                                                  static_cast<const uint4*>(bank->v_host[layer]), plan, row_vecs,
+                                                  out_capacity_chunks, static_cast<uint4*>(k_out),
+                                                  static_cast<uint4*>(v_out));
   MSA_LAUNCH_CHECK();
+  if (dedup) {
+    gather_copy_kernel<true><<<grid, 128, 0, st>>>(nullptr, nullptr, plan, row_vecs, out_capacity_chunks,
+                                                   static_cast<uint4*>(k_out), static_cast<uint4*>(v_out));
+    MSA_LAUNCH_CHECK();
+  }
   return MSA_OK;
 }

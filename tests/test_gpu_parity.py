@@ -267,7 +267,19 @@ def test_gather_kv_exact(ops, dtype):
     # a short output drops the overflowing rows instead of writing past the end
     Ks, Vs, cus = ops.gather_kv_device(bank, 1, sel_dev, 10)
     torch.cuda.synchronize()
-    assert torch.equal(Ks.cpu(), wk2[:10]) and cus.cpu().tolist() == wcu2.tolist()
+    # ... and the prefix sums stop at the capacity, so no consumer addresses a row that was never filled
+    assert torch.equal(Ks.cpu(), wk2[:10]) and cus.cpu().tolist() == [min(int(x), 10) for x in wcu2.tolist()]
+    # documents shared by several samples (fetched from the host once, copied on the device for the others;
+    # src/msa_service.py:1214): every sample still gets its own complete rows, on both gather paths
+    shared = torch.tensor([[9, 3, 200, 7], [3, 9, 7, 200], [200, 200, 3, 5], [5, 3, 9, 7], [1, 2, 3, 4]], dtype=torch.int32)
+    wk3, wv3, wcu3, _ = cf.gather_selected(kh, vh, dco, shared)
+    K3, V3, cu3 = ops.gather_kv(bank, 1, shared, "cuda", stream=side)
+    side.synchronize()
+    assert cu3.tolist() == wcu3.tolist() and torch.equal(K3.cpu(), wk3) and torch.equal(V3.cpu(), wv3)
+    Kd3, Vd3, cud3 = ops.gather_kv_device(bank, 1, shared.cuda(), shared.numel() * bank.max_doc_chunks)
+    torch.cuda.synchronize()
+    n3 = int(wcu3[-1])
+    assert cud3.cpu().tolist() == wcu3.tolist() and torch.equal(Kd3[:n3].cpu(), wk3) and torch.equal(Vd3[:n3].cpu(), wv3)
     with pytest.raises(Exception, match="outside"):
         ops.gather_kv(bank, 1, torch.tensor([[300]], dtype=torch.int32), "cuda")
     with pytest.raises(Exception, match="no host K"):

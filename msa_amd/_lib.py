@@ -27,6 +27,7 @@ SIGNATURES = {
     "msa_bank_set_layer": (C.c_int, [_vp, _i32, _vp, _vp, _vp]),
     "msa_bank_destroy": (C.c_int, [_vp]),
     "msa_route_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32, _i32, _i64, _i64, _i32]),
+    "msa_route_topk_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32, _i32, _i64, _i32]),
     "msa_chunk_scores": (C.c_int, [_vp, _i32, _vp, _vp, _i32, _i32, _i32, _i32, _f32, _vp, _vp, _sz, _vp]),
     "msa_route_topk": (C.c_int, [_vp, _i32, _vp, _vp, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _vp, _vp, _vp, _sz,
                                  _vp]),

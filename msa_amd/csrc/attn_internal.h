@@ -28,8 +28,7 @@ static inline SplitPlan plan_splits(int64_t total_q, int32_t Hkv, int32_t max_kv
 // VALU split kernel (decode): one workgroup per compute unit measured best (fewer, longer key streams); the
 // kernel itself divides each sample's own length evenly over n_split.
 static inline SplitPlan plan_splits_valu(int64_t total_q, int32_t Hkv, int32_t max_kv) {
-  static const int target = [] { const char* e = getenv("MSA_ATTN_WGS"); return e ? atoi(e) : 256; }();
-  return plan_splits_for(total_q, Hkv, max_kv, target);
+  return plan_splits_for(total_q, Hkv, max_kv, 256);
 }
 
 // flash_attn.hip: bf16 partial pass over split `blockIdx.z` of the keys; writes un-normalised

@@ -24,7 +24,7 @@ extern "C" int msa_bank_create(msa_bank** out, int32_t n_layers, int64_t C, int3
   *out = nullptr;
   MSA_REQUIRE(n_layers > 0 && n_layers <= 4096, "msa_bank_create: n_layers=%d out of range", n_layers);
   MSA_REQUIRE(C > 0 && C < (int64_t)1 << 31, "msa_bank_create: C=%lld out of range", (long long)C);
-  MSA_REQUIRE(n_docs > 0 && n_docs <= C, "msa_bank_create: n_docs=%lld out of range (C=%lld)",
+  MSA_REQUIRE(n_docs > 0 && n_docs <= C && n_docs < (int64_t)1 << 31, "msa_bank_create: n_docs=%lld out of range (C=%lld)",
               (long long)n_docs, (long long)C);
   MSA_REQUIRE(D == kHeadDim, "msa_bank_create: head dim %d unsupported (need %d)", D, kHeadDim);
   MSA_REQUIRE(Hkv > 0 && Hkv <= 64, "msa_bank_create: Hkv=%d out of range", Hkv);
@@ -58,6 +58,19 @@ extern "C" int msa_bank_create(msa_bank** out, int32_t n_layers, int64_t C, int3
   if (e == hipSuccess) e = hipMalloc((void**)&b->doc_global_id_dev, id_bytes);
   if (e == hipSuccess) e = hipMemcpy(b->doc_chunk_off_dev, doc_chunk_off_host, off_bytes, hipMemcpyHostToDevice);
   if (e == hipSuccess) e = hipMemcpy(b->doc_global_id_dev, doc_global_id_host, id_bytes, hipMemcpyHostToDevice);
+  if (e == hipSuccess) {
+    int32_t* chunk_doc = (int32_t*)malloc((size_t)C * sizeof(int32_t));
+    if (chunk_doc == nullptr) {
+      msa_bank_destroy(b);
+      msa_set_error("msa_bank_create: out of host memory");
+      return MSA_EINVAL;
+    }
+    for (int64_t d = 0; d < n_docs; ++d)
+      for (int32_t c = doc_chunk_off_host[d]; c < doc_chunk_off_host[d + 1]; ++c) chunk_doc[c] = (int32_t)d;
+    e = hipMalloc((void**)&b->chunk_doc_dev, (size_t)C * sizeof(int32_t));
+    if (e == hipSuccess) e = hipMemcpy(b->chunk_doc_dev, chunk_doc, (size_t)C * sizeof(int32_t), hipMemcpyHostToDevice);
+    free(chunk_doc);
+  }
   if (e != hipSuccess) {
     msa_bank_destroy(b);
     msa_set_error("msa_bank_create: HIP error %s", hipGetErrorString(e));
@@ -84,6 +97,7 @@ extern "C" int msa_bank_destroy(msa_bank* b) {
   if (!b) return MSA_OK;
   if (b->doc_chunk_off_dev) (void)hipFree(b->doc_chunk_off_dev);
   if (b->doc_global_id_dev) (void)hipFree(b->doc_global_id_dev);
+  if (b->chunk_doc_dev) (void)hipFree(b->chunk_doc_dev);
   free(b->doc_chunk_off_host);
   free(b->doc_global_id_host);
   free((void*)b->kr_dev);

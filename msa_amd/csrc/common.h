@@ -85,6 +85,7 @@ struct msa_bank {
   int64_t n_docs;
   int32_t device;
   int32_t* doc_chunk_off_dev;   // [n_docs+1]
+  int32_t* chunk_doc_dev;       // [C] document of every chunk (the scoring epilogue folds chunk maxima per document)
   int64_t* doc_global_id_dev;   // [n_docs]
   int32_t* doc_chunk_off_host;  // [n_docs+1]
   int64_t* doc_global_id_host;  // [n_docs]

@@ -468,8 +468,6 @@ TilePlan plan_tile(int32_t N, int32_t K) {
   t.row_blocks = (groups + t.gpw - 1) / t.gpw;
   t.n_slices = std::min(std::min(kTileMaxSlices, steps), 256 / std::max(1, t.row_blocks));
   if (t.n_slices < 2) return t;
-  static const int env_tile = [] { const char* e = getenv("MSA_LINEAR_TILE"); return e ? atoi(e) : 1; }();
-  if (env_tile == 0) return t;
   const double plain_bytes = (16.0 + 16.0) * K * 2;                             // one row group + all of x
   const double tiled_bytes = (16.0 * t.gpw + 16.0) * ((double)K / t.n_slices) * 2;
   t.use = (plain_bytes - tiled_bytes) / 34e3 > 8.0;                             // bytes / (34 GB/s) in us
@@ -515,8 +513,7 @@ extern "C" int msa_skinny_linear(const void* x, const void* w, const void* resid
 
   // Many row groups per compute unit and a K that 16 wavefronts split into 5 MFMA steps each (K = 2560): the
   // streaming kernel, one workgroup per compute unit at most, an equal number of items (32 rows) each.
-  static const int env_stream = [] { const char* e = getenv("MSA_LINEAR_STREAM"); return e ? atoi(e) : 1; }();
-  if (K == 16 * 5 * 32 && env_stream != 0) {
+  if (K == 16 * 5 * 32) {
     const int n_items = epilogue == kEpiSiluMul ? N / 16 : (N + 31) / 32;
     const int iters = (n_items + 255) / 256;
     const int grid = (n_items + iters - 1) / iters;
@@ -535,19 +532,14 @@ extern "C" int msa_skinny_linear(const void* x, const void* w, const void* resid
 
   // Wavefronts per workgroup: split K far enough that the launch has a few thousand wavefronts, and
   // prefer a count that divides the K units so every wavefront streams the same number of bytes.
-  static const int env_waves = [] { const char* e = getenv("MSA_LINEAR_WAVES"); return e ? atoi(e) : 0; }();
-  static const int env_r = [] { const char* e = getenv("MSA_LINEAR_R"); return e ? atoi(e) : 0; }();
   // Row groups per wavefront: two share one load of x (every workgroup re-reads x from L2) when N is large
   // enough to still fill the chip with workgroups.
   int R = ((int64_t)N / 32 * kMaxWaves >= 3072 || epilogue == kEpiSiluMul) ? 2 : 1;
-  if (env_r == 1 && epilogue != kEpiSiluMul) R = 1;
-  if (env_r == 2) R = 2;
   // Rows per workgroup: 16 R, or fewer when that leaves compute units without a workgroup (a compute unit moves
   // only ~34 GB/s, so 256 workgroups of 10 rows beat 160 of 16 on a 2560-row matrix); the silu epilogue needs whole
   // gate / up groups.
-  static const int env_spread = [] { const char* e = getenv("MSA_LINEAR_SPREAD"); return e ? atoi(e) : 1; }();
   int rows_per_wg = 16 * R;
-  if (env_spread != 0 && epilogue != kEpiSiluMul && (N + 16 * R - 1) / (16 * R) < 256) {
+  if (epilogue != kEpiSiluMul && (N + 16 * R - 1) / (16 * R) < 256) {
     const int spread = std::max(8, (N + 255) / 256);
     if (spread > 16 * (R - 1) && spread < 16 * R) rows_per_wg = spread;
   }
@@ -557,7 +549,6 @@ extern "C" int msa_skinny_linear(const void* x, const void* w, const void* resid
   int waves = want;
   for (int cand = want; cand >= std::max(1, want / 2); --cand)
     if (units % cand == 0) { waves = cand; break; }
-  if (env_waves > 0) waves = std::max(1, std::min(std::min(env_waves, kMaxWaves), units));
 
 #define MSA_LIN(R_, E_)                                                                              \
   (norm_w ? launch<R_, E_, true>(x, w, residual, norm_w, eps, y, M, N, K, waves, rows_per_wg, st)    \

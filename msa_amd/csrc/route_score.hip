@@ -4,11 +4,12 @@
 //             = max_t (scale / Hq) * Qs[b,t,:] . kr[c,:]        with Qs[b,t,g,:] = sum_{h in g} q'[b,t,h,:]
 // (the mean over heads is linear, so the G query heads of one KV group are summed first).  That is
 // an NT GEMM  [B*S_pad, Hkv*D] x [C, Hkv*D]^T  whose output is never written: each 32-row MFMA
-// block is reduced to a column max over its scored rows in registers and merged into
-// chunk_key[B, C] (order-preserving uint32 keys) with atomicMax.
-#include <stdlib.h>
-
+// block is reduced to a column max over its scored rows in registers.  For routing the column maxima
+// of a query are folded further, across the chunks of one document, and merged with atomicMax into
+// doc_key[B, n_docs] (order-preserving uint32 keys): the max over a document's chunks happens in the
+// scoring epilogue and no per-chunk plane exists.  msa_chunk_scores keeps the per-chunk form.
 #include <algorithm>
+#include <mutex>
 #include <type_traits>
 
 #include "common.h"
@@ -20,18 +21,39 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 // ------------------------------------------------------------------------------------------
-// Prologue: normalise (cosine mode), sum the G heads of each KV group, cast, build row masks.
+// Prologue: normalise (cosine mode), sum the G heads of each KV group, cast, build row masks, clear the key plane.
 // One workgroup of Hkv*16 lanes per (b, padded token); lane (g, j) owns 8 contiguous d of group g.
+// The workgroup of every 32nd row also writes the scored-row bitmask word of its 32 rows (a ballot, no atomics),
+// workgroup 0 the zero words that pad the mask to whole M tiles, and all workgroups together clear the
+// `clear_words` key words the scoring kernel merges into with atomicMax.
 // ------------------------------------------------------------------------------------------
 template <typename TIn, typename TOut>
 __global__ void presum_queries_kernel(const TIn* __restrict__ q, const uint8_t* __restrict__ qmask, int32_t B,
                                       int32_t S, int32_t S_pad, int32_t Hq, int32_t Hkv, int32_t normalize,
-                                      TOut* __restrict__ qs, uint32_t* __restrict__ row_bits) {
+                                      TOut* __restrict__ qs, uint32_t* __restrict__ row_bits, int32_t mask_words,
+                                      uint32_t* __restrict__ key_plane, int64_t clear_words) {
   const int row = blockIdx.x;              // b * S_pad + s
   const int b = row / S_pad, s = row % S_pad;
   const int G = Hq / Hkv;
   const int g = threadIdx.x >> 4, j = threadIdx.x & 15;
-  const bool valid = s < S && (qmask == nullptr || qmask[(int64_t)b * S + s] != 0);
+  auto scored = [&](int r) {
+    const int rb = r / S_pad, rs = r % S_pad;
+    return rs < S && (qmask == nullptr || qmask[(int64_t)rb * S + rs] != 0);
+  };
+  const bool valid = scored(row);
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words; i += (int64_t)gridDim.x * blockDim.x)
+    key_plane[i] = 0u;
+  if ((row & 31) == 0 && threadIdx.x < 64) {          // rows are padded per query to a multiple of 32
+    const int nl = min((int)blockDim.x, 32);
+    uint32_t bits = 0;
+    for (int base = 0; base < 32; base += nl) {
+      const bool v = (int)threadIdx.x < nl && scored(row + base + (int)threadIdx.x);
+      bits |= (uint32_t)__ballot(v) << base;
+    }
+    if (threadIdx.x == 0) row_bits[row >> 5] = bits;
+  }
+  if (blockIdx.x == 0)
+    for (int w = (int)(gridDim.x >> 5) + (int)threadIdx.x; w < mask_words; w += blockDim.x) row_bits[w] = 0u;
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
@@ -79,12 +101,6 @@ __global__ void presum_queries_kernel(const TIn* __restrict__ q, const uint8_t* 
     *reinterpret_cast<float4*>(o) = make_float4(acc[0], acc[1], acc[2], acc[3]);
     *reinterpret_cast<float4*>(o + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
   }
-  if (threadIdx.x == 0 && valid) atomicOr(&row_bits[row >> 5], 1u << (row & 31));
-}
-
-__global__ void fill_u32_kernel(uint32_t* __restrict__ p, int64_t n, uint32_t v) {
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) p[i] = v;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -120,16 +136,20 @@ struct Mma<float> {
 };
 
 // Workgroup tile BM x BN, WAVES_M x WAVES_N wavefronts, each owning TM x TN blocks of 32 x 32.
-// kDeep: two register sets of global loads in flight (two K tiles ahead of the one being multiplied) for the
-// HBM-bound shapes, where one tile's MFMA work is shorter than a load's latency.
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool kDeep = false>
+// kSets: register sets of global loads, i.e. K tiles in flight ahead of the one being multiplied.  One is enough when
+// a tile's MFMA work outlasts a load's latency (the MFMA-bound shapes); the HBM-bound shapes (few query rows) need
+// more bytes in flight per compute unit than one tile holds.
+// kDocMax: keys are folded over the chunks of a document (chunk_doc) and merged into out_key[B, n_docs];
+// otherwise one key per (query, chunk) is merged into out_key[B, C].
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool kDocMax>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     const T* __restrict__ qs,            // [M_rows, K]  pre-summed queries, M_rows = B * S_pad
     const T* __restrict__ kr,            // [C, K]
     const uint32_t* __restrict__ row_bits,  // [ceil(M_alloc / 32)] scored-row bitmask
-    uint32_t* __restrict__ chunk_key,    // [B, C]
+    uint32_t* __restrict__ out_key,      // [B, n_docs] or [B, C], zeroed
+    const int32_t* __restrict__ chunk_doc,  // [C] document of every chunk (kDocMax)
     int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t tiles_m, int32_t tiles_n,
-    int32_t m_group, int32_t exclusive) {
+    int32_t m_group, int32_t n_docs) {
   constexpr int kThreads = WAVES_M * WAVES_N * 64;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -161,8 +181,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
 
   // Global -> register staging through buffer loads: one resource per operand tile whose extent is
   // the valid part of the tile, so rows past M_rows / C read as zero in hardware (no branches, no
-  // clamps).  Only the vector offset takes part in the range check, so the row displacement of a
-  // thread's vectors rides there; the K-tile displacement (which stays inside the row) is scalar.
+  // clamps).  The range check is defined on the vector offset, so the row displacement of a thread's
+  // vectors rides there; the K-tile displacement (which stays inside the row, so it can never carry a
+  // load past the extent) is scalar.
   const int rows_a = min(BM, M_rows - m0), rows_b = min(BN, C - n0);
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(ga) + (int64_t)m0 * row_bytes_g, 0, (int)(rows_a * row_bytes_g), 0x00020000);
@@ -170,7 +191,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
       const_cast<char*>(gb) + (int64_t)n0 * row_bytes_g, 0, (int)(rows_b * row_bytes_g), 0x00020000);
   const int voff = (tid >> 3) * (int)row_bytes_g + (tid & 7) * 16;
   const int vec_stride = (kThreads / 8) * (int)row_bytes_g;     // rows between a thread's vectors
-  constexpr int kSets = kDeep ? 2 : 1;
+  static_assert(kSets >= 1 && kSets <= 3, "one to three K tiles in flight");
   u32x4_t ra[kSets][kVecA], rb[kSets][kVecB];
   // K_r streams through once per M tile group while the query matrix is re-read by every workgroup of an XCD: the
   // non-temporal hint on the K_r loads keeps the queries in the 4 MiB L2 (traffic past L2 9.9 -> 6.9 GB per launch
@@ -202,7 +223,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     }
   };
   typedef std::integral_constant<int, 0> Set0;
-  typedef std::integral_constant<int, kSets - 1> Set1;
+  typedef std::integral_constant<int, 1 % kSets> Set1;
+  typedef std::integral_constant<int, 2 % kSets> Set2;
 
   floatx16_t acc[TM][TN];
 #pragma unroll
@@ -234,8 +256,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   };
 
   // One K tile out of LDS buffer `buf`; kMore says a next tile exists (the steady-state loop is
-  // compiled without that condition so the wait counters around the barrier stay exact).  `set_tag` names the
-  // register set that holds tile kt+1 and takes the next global loads.
+  // compiled without that condition so the wait counters around the barrier stay exact).  Tile t travels in
+  // register set t % kSets; `set_tag` names the set that holds tile kt+1, which is stored and then refilled with
+  // tile kt+1+kSets.
   auto k_tile = [&](auto more_tag, auto set_tag, int kt) {
     constexpr bool kMore = decltype(more_tag)::value;
     const int buf = kt & 1;
@@ -250,9 +273,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
       }
       if (sub == 1 && kMore) {
         store_tile(set_tag, buf ^ 1);
-        if constexpr (kDeep) {
+        if constexpr (kSets > 1) {
           __builtin_amdgcn_sched_barrier(0);   // the refill reuses the registers the stores above read
-          load_tile(set_tag, kt + 3);
+          load_tile(set_tag, kt + 1 + kSets);
         } else if (kt + 2 < k_tiles) {
           load_tile(set_tag, kt + 2);
         }
@@ -264,8 +287,32 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     }
   };
 
-  if constexpr (kDeep) {
-    // tile t travels in register set (t & 1): iteration kt stores tile kt+1 and refills its set with tile kt+3
+  if constexpr (kSets == 3) {
+    load_tile(Set0{}, 0);
+    store_tile(Set0{}, 0);
+    load_tile(Set1{}, 1);
+    load_tile(Set2{}, 2);
+    load_tile(Set0{}, 3);
+    __syncthreads();
+    load_frags(0, 0, 0);
+    int kt = 0;
+    for (; kt + 3 < k_tiles; kt += 3) {
+      k_tile(std::true_type{}, Set1{}, kt);
+      k_tile(std::true_type{}, Set2{}, kt + 1);
+      k_tile(std::true_type{}, Set0{}, kt + 2);
+    }
+    const int left = k_tiles - kt;             // 1..3 tiles
+    if (left == 1) {
+      k_tile(std::false_type{}, Set1{}, kt);
+    } else if (left == 2) {
+      k_tile(std::true_type{}, Set1{}, kt);
+      k_tile(std::false_type{}, Set2{}, kt + 1);
+    } else {
+      k_tile(std::true_type{}, Set1{}, kt);
+      k_tile(std::true_type{}, Set2{}, kt + 1);
+      k_tile(std::false_type{}, Set0{}, kt + 2);
+    }
+  } else if constexpr (kSets == 2) {
     load_tile(Set0{}, 0);
     store_tile(Set0{}, 0);
     load_tile(Set1{}, 1);
@@ -293,18 +340,32 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     k_tile(std::false_type{}, Set0{}, k_tiles - 1);
   }
 
-  // Epilogue.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of its 32x32 block.
-  // `exclusive`: every query's rows lie inside one wavefront's tile, so each (query, chunk) key has a single
-  // writer, which stores it (0 for a query without a scored token) into a plane nobody cleared.  Otherwise
-  // several wavefronts or workgroups hold parts of a query and combine through atomicMax on a zeroed plane.
+  // Epilogue.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of its 32x32 block.  Consecutive row
+  // blocks of one query are folded into `run`; emit() then merges the query's 32 column maxima of this block
+  // into the key plane.  Several wavefronts and workgroups hold parts of a query (and of a document), so the
+  // merge is an atomicMax into a zeroed plane.  emit() is reached by whole wavefronts (q and any are uniform).
   const int n_queries = M_rows / (blocks_per_query * 32);
   auto emit = [&](int q, int n, float run, bool any) {
-    if (half != 0 || n >= C || q >= n_queries) return;
-    uint32_t* dst = &chunk_key[(int64_t)q * C + n];
-    // streamed out: a cached store keeps 103 MB of keys per launch flowing through the L2 the queries live in
-    // (fetches past L2 3.69 -> 3.36 GiB-units per launch, kernel 0.4 % faster)
-    if (exclusive) __builtin_nontemporal_store(any ? f32_to_key(run) : 0u, dst);
-    else if (any) atomicMax(dst, f32_to_key(run));
+    if (!any || q >= n_queries) return;
+    const bool ok = n < C;
+    const uint32_t key = ok ? f32_to_key(run) : 0u;
+    if constexpr (kDocMax) {
+      // Chunks of a document are adjacent columns: a segmented max-scan over the 32 lanes of each half leaves a
+      // document's maximum in the last lane of its run, which alone touches memory (about two atomics per 32
+      // chunks instead of 32 stores, and no per-chunk plane to read back).
+      const int doc = ok ? chunk_doc[n] : -1 - l32;        // lanes past the bank never join a run
+      uint32_t m = key;
+#pragma unroll
+      for (int off = 1; off < 32; off <<= 1) {
+        const uint32_t om = (uint32_t)__shfl_up((int)m, off, 32);
+        const int od = __shfl_up(doc, off, 32);
+        if (l32 >= off && od == doc) m = max(m, om);
+      }
+      const int nd = __shfl_down(doc, 1, 32);
+      if (ok && half == 0 && (l32 == 31 || nd != doc)) atomicMax(&out_key[(int64_t)q * n_docs + doc], m);
+    } else {
+      if (ok && half == 0) atomicMax(&out_key[(int64_t)q * C + n], key);
+    }
   };
 #pragma unroll
   for (int j = 0; j < TN; ++j) {
@@ -347,48 +408,59 @@ __global__ void decode_scores_kernel(const uint32_t* __restrict__ key, int64_t n
   }
 }
 
-// Optional timing of the scoring kernel alone: event pairs recorded around its launch.
+// Optional timing of the scoring kernel alone: event pairs recorded around its launch.  The lock makes the record
+// list safe against concurrent callers; while timing is off a launch only reads one atomic flag.
 struct KernelTimer {
+  std::mutex mu;
+  std::atomic<int> on{0};
   hipEvent_t* start = nullptr;
   hipEvent_t* stop = nullptr;
   int cap = 0;
   int n = 0;
 } g_timer;
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, bool kDeep = false>
-int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* chunk_key, int32_t M_rows,
-                int32_t C, int32_t K, int32_t blocks_per_query, int32_t exclusive, hipStream_t st) {
-  if (exclusive && (BM / WAVES_M) % (blocks_per_query * 32) != 0) {
-    msa_set_error("score_gemm: single-writer epilogue asked for %d-row queries on %d-row wavefront tiles",
-                  blocks_per_query * 32, BM / WAVES_M);
-    return MSA_EINVAL;
-  }
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool kDocMax>
+int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key, const int32_t* chunk_doc,
+                int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t n_docs, hipStream_t st) {
   const int tiles_m = (M_rows + BM - 1) / BM, tiles_n = (C + BN - 1) / BN;
   // M tiles are walked in groups of 8 per K_r tile: a group's query rows (4 MiB in bf16) are what an XCD's L2
   // holds.  At 8 M tiles that is all of them (groups of 1, 2, 4 lose 2-14 % there); with 16 M tiles groups of 8
-  // measured 1.4 % faster than one group, with 256 (a 64k-row prefill batch) 4 %.  MSA_SCORE_MGROUP overrides.
-  int m_group = std::min(tiles_m, 8);
-  if (const char* mg = getenv("MSA_SCORE_MGROUP")) {
-    const int v = atoi(mg);
-    if (v > 0) m_group = std::min(v, tiles_m);
-  }
+  // measured 1.4 % faster than one group, with 256 (a 64k-row prefill batch) 4 %.
+  const int m_group = std::min(tiles_m, 8);
   const int m_groups = (tiles_m + m_group - 1) / m_group;
   const int grid = 8 * ((tiles_n + 7) / 8) * m_groups * m_group;
   const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
-  auto kern = score_gemm_kernel<T, BM, BN, WAVES_M, WAVES_N, kDeep>;
+  auto kern = score_gemm_kernel<T, BM, BN, WAVES_M, WAVES_N, kSets, kDocMax>;
   static std::atomic<int> lds_limit_raised{0};
   MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(kern), (int)lds));
-  const bool timed = g_timer.n < g_timer.cap;
-  if (timed) MSA_HIP(hipEventRecord(g_timer.start[g_timer.n], st));
-  kern<<<grid, WAVES_M * WAVES_N * 64, lds, st>>>(static_cast<const T*>(qs), static_cast<const T*>(kr), row_bits,
-                                                  chunk_key, M_rows, C, K, blocks_per_query, tiles_m, tiles_n, m_group,
-                                                  exclusive);
-  MSA_LAUNCH_CHECK();
-  if (timed) {
-    MSA_HIP(hipEventRecord(g_timer.stop[g_timer.n], st));
-    ++g_timer.n;
+  int slot = -1;
+  if (g_timer.on.load(std::memory_order_acquire)) {
+    std::lock_guard<std::mutex> lock(g_timer.mu);
+    if (g_timer.n < g_timer.cap) slot = g_timer.n++;
   }
+  if (slot >= 0) MSA_HIP(hipEventRecord(g_timer.start[slot], st));
+  kern<<<grid, WAVES_M * WAVES_N * 64, lds, st>>>(static_cast<const T*>(qs), static_cast<const T*>(kr), row_bits, out_key,
+                                                  chunk_doc, M_rows, C, K, blocks_per_query, tiles_m, tiles_n, m_group,
+                                                  n_docs);
+  MSA_LAUNCH_CHECK();
+  if (slot >= 0) MSA_HIP(hipEventRecord(g_timer.stop[slot], st));
   return MSA_OK;
+}
+
+// Tile choice by query rows.  Few rows are HBM-bound: narrow M tile, more workgroups in flight and K tiles of
+// global loads ahead of the one being multiplied (Little's law: a compute unit needs about 60 KB of loads in flight
+// to draw its share of the HBM rate).  Many rows are MFMA-bound: 256 x 256 tile, 8 wavefronts, one tile ahead.
+template <bool kDocMax>
+int launch_gemm_for(int32_t dtype, const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key,
+                    const int32_t* chunk_doc, int32_t M_rows, int32_t C, int32_t K, int32_t bpq, int32_t n_docs,
+                    hipStream_t st) {
+  if (dtype != MSA_BF16)
+    return launch_gemm<float, 128, 128, 2, 2, 1, kDocMax>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
+  if (M_rows <= 64)
+    return launch_gemm<bf16_t, 64, 128, 2, 2, 2, kDocMax>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
+  if (M_rows <= 128)
+    return launch_gemm<bf16_t, 128, 384, 2, 4, 1, kDocMax>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
+  return launch_gemm<bf16_t, 256, 256, 2, 4, 1, kDocMax>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
 }
 
 }  // namespace
@@ -398,16 +470,17 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
 // ------------------------------------------------------------------------------------------
 #include "route_internal.h"
 
-RouteWorkspace route_workspace_layout(int32_t B, int32_t S, int32_t Hkv, int32_t D, int64_t C, int64_t n_docs,
-                                      int32_t topk, int32_t dtype) {
+RouteWorkspace route_workspace_layout(int32_t B, int32_t S, int32_t Hkv, int32_t D, int64_t plane_cols, int64_t n_docs,
+                                      int32_t dtype) {
   RouteWorkspace w{};
   w.S_pad = (S + 31) / 32 * 32;
   w.M_rows = B * w.S_pad;
   const int64_t m_alloc = ((int64_t)w.M_rows + 255) / 256 * 256;   // every M tile may read whole mask words
+  w.mask_words = (int32_t)(m_alloc / 32);
   size_t off = 0;
   w.off_qs = off;       off = align_up(off + (size_t)w.M_rows * Hkv * D * elem_bytes(dtype), 256);
-  w.off_row_bits = off; off = align_up(off + (size_t)(m_alloc / 32) * sizeof(uint32_t), 256);
-  w.off_chunk_key = off; off = align_up(off + (size_t)B * C * sizeof(uint32_t), 256);
+  w.off_row_bits = off; off = align_up(off + (size_t)w.mask_words * sizeof(uint32_t), 256);
+  w.off_key = off;      off = align_up(off + (size_t)B * plane_cols * sizeof(uint32_t), 256);
   w.topk_blocks = topk_blocks_for(n_docs);
   w.off_cand = off;     off = align_up(off + (size_t)B * w.topk_blocks * kTopkMax * sizeof(uint64_t), 256);
   w.bytes = off;
@@ -415,13 +488,16 @@ RouteWorkspace route_workspace_layout(int32_t B, int32_t S, int32_t Hkv, int32_t
 }
 
 extern "C" int msa_profile_enable(int32_t max_records) {
+  std::lock_guard<std::mutex> lock(g_timer.mu);
+  g_timer.on.store(0, std::memory_order_release);
   for (int i = 0; i < g_timer.cap; ++i) {
     (void)hipEventDestroy(g_timer.start[i]);
     (void)hipEventDestroy(g_timer.stop[i]);
   }
   delete[] g_timer.start;
   delete[] g_timer.stop;
-  g_timer = KernelTimer{};
+  g_timer.start = g_timer.stop = nullptr;
+  g_timer.cap = g_timer.n = 0;
   MSA_REQUIRE(max_records >= 0 && max_records <= 1 << 20, "msa_profile_enable: max_records=%d", max_records);
   if (max_records == 0) return MSA_OK;
   g_timer.start = new hipEvent_t[max_records];
@@ -431,11 +507,13 @@ extern "C" int msa_profile_enable(int32_t max_records) {
     MSA_HIP(hipEventCreate(&g_timer.stop[i]));
     g_timer.cap = i + 1;
   }
+  g_timer.on.store(1, std::memory_order_release);
   return MSA_OK;
 }
 
 extern "C" int msa_profile_collect(float* ms_host, int32_t cap, int32_t* n_out) {
   MSA_REQUIRE(ms_host && n_out, "msa_profile_collect: null pointer");
+  std::lock_guard<std::mutex> lock(g_timer.mu);
   const int n = std::min(g_timer.n, cap);
   for (int i = 0; i < n; ++i) {
     MSA_HIP(hipEventSynchronize(g_timer.stop[i]));
@@ -448,15 +526,23 @@ extern "C" int msa_profile_collect(float* ms_host, int32_t cap, int32_t* n_out) 
 
 extern "C" size_t msa_route_workspace_bytes(int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D, int64_t C,
                                             int64_t n_docs, int32_t topk) {
-  (void)Hq;
+  (void)Hq; (void)topk;
   if (B <= 0 || S <= 0 || Hkv <= 0 || D <= 0 || C <= 0 || n_docs <= 0) return 0;
-  // sized for fp32 queries so one workspace serves both dtypes
-  return route_workspace_layout(B, S, Hkv, D, C, n_docs, topk, MSA_F32).bytes;
+  // sized for fp32 queries so one workspace serves both dtypes, and for the per-chunk plane of msa_chunk_scores
+  return route_workspace_layout(B, S, Hkv, D, std::max(C, n_docs), n_docs, MSA_F32).bytes;
+}
+
+extern "C" size_t msa_route_topk_workspace_bytes(int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D,
+                                                 int64_t n_docs, int32_t topk) {
+  (void)Hq; (void)topk;
+  if (B <= 0 || S <= 0 || Hkv <= 0 || D <= 0 || n_docs <= 0) return 0;
+  return route_workspace_layout(B, S, Hkv, D, n_docs, n_docs, MSA_F32).bytes;
 }
 
 int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
-                         int32_t S, int32_t Hq, int32_t mode, float scale, void* workspace, size_t workspace_bytes,
-                         hipStream_t st, RouteWorkspace* layout_out, float* mul_out, const char* who) {
+                         int32_t S, int32_t Hq, int32_t mode, float scale, bool doc_max, void* workspace,
+                         size_t workspace_bytes, hipStream_t st, RouteWorkspace* layout_out, float* mul_out,
+                         const char* who) {
   MSA_REQUIRE(bank != nullptr, "%s: null bank", who);
   MSA_REQUIRE(layer >= 0 && layer < bank->n_layers, "%s: layer %d out of range", who, layer);
   if (bank->kr_dev[layer] == nullptr) {
@@ -473,7 +559,8 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
   MSA_REQUIRE(sc > 0.f && sc < INFINITY, "%s: scale must be positive and finite", who);
   MSA_REQUIRE((int64_t)B * ((S + 31) / 32 * 32) < (int64_t)1 << 24, "%s: too many query rows", who);
 
-  const RouteWorkspace w = route_workspace_layout(B, S, bank->Hkv, bank->D, bank->C, bank->n_docs, kTopkMax, bank->dtype);
+  const int64_t plane_cols = doc_max ? bank->n_docs : bank->C;
+  const RouteWorkspace w = route_workspace_layout(B, S, bank->Hkv, bank->D, plane_cols, bank->n_docs, bank->dtype);
   if (w.bytes > workspace_bytes) {
     msa_set_error("%s: workspace of %zu bytes, need %zu", who, workspace_bytes, w.bytes);
     return MSA_ESIZE;
@@ -481,75 +568,27 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
   char* ws = static_cast<char*>(workspace);
   void* qs = ws + w.off_qs;
   uint32_t* row_bits = reinterpret_cast<uint32_t*>(ws + w.off_row_bits);
-  uint32_t* chunk_key = reinterpret_cast<uint32_t*>(ws + w.off_chunk_key);
-  // Tile choice by query rows: small M is HBM-bound (narrow M tile, more workgroups in flight, two K tiles of
-  // global loads ahead: 3 % faster than one at 16-64 rows; at 128 rows the deeper prefetch measured slower and
-  // the wider tiles spill with it), large M is MFMA-bound (256 x 256 tile, 8 wavefronts).  MSA_SCORE_TILE
-  // overrides for tuning.
-  // wave_rows[v] = rows of one wavefront's tile in variant v (BM / WAVES_M).
-  static const int wave_rows[11] = {32, 64, 128, 64, 64, 64, 64, 32, 128, 64, 32};
-  const char* ev = getenv("MSA_SCORE_TILE");
-  const int variant = ev ? atoi(ev) : (w.M_rows <= 64 ? 10 : w.M_rows <= 128 ? 6 : 2);
-  if (bank->dtype == MSA_BF16 && (variant < 0 || variant > 10)) {
-    msa_set_error("MSA_SCORE_TILE=%d unknown", variant);
-    return MSA_EINVAL;
-  }
-  // A query whose rows fit one wavefront's tile has a single writer per chunk key: the kernel stores
-  // and the key plane needs no clearing (at the 100M-token bank the plane is 103 MB per launch).
-  // MSA_SCORE_EXCLUSIVE=0 forces the atomicMax form (for A/B measurements).
-  const char* ex_env = getenv("MSA_SCORE_EXCLUSIVE");
-  const int32_t exclusive =
-      (bank->dtype == MSA_BF16 ? wave_rows[variant] : 64) % w.S_pad == 0 && !(ex_env && atoi(ex_env) == 0) ? 1 : 0;
-
-  // row masks start at zero; so do the chunk keys when wavefronts combine through atomicMax (both live in one
-  // contiguous span of the workspace)
-  const int64_t zero_words =
-      (int64_t)(((exclusive ? w.off_chunk_key : w.off_cand) - w.off_row_bits) / sizeof(uint32_t));
-  fill_u32_kernel<<<(int)std::min<int64_t>((zero_words + 1023) / 1024, 4096), 256, 0, st>>>(row_bits, zero_words, 0u);
-  MSA_LAUNCH_CHECK();
+  uint32_t* key = reinterpret_cast<uint32_t*>(ws + w.off_key);
 
   const int normalize = mode == MSA_MODE_COSINE ? 1 : 0;
   const int pthreads = bank->Hkv * 16;
+  const int64_t clear_words = (int64_t)B * plane_cols;
   if (bank->dtype == MSA_BF16)
     presum_queries_kernel<bf16_t, bf16_t><<<w.M_rows, pthreads, 0, st>>>(
         static_cast<const bf16_t*>(q), qmask_u8, B, S, w.S_pad, Hq, bank->Hkv, normalize, static_cast<bf16_t*>(qs),
-        row_bits);
+        row_bits, w.mask_words, key, clear_words);
   else
     presum_queries_kernel<float, float><<<w.M_rows, pthreads, 0, st>>>(
         static_cast<const float*>(q), qmask_u8, B, S, w.S_pad, Hq, bank->Hkv, normalize, static_cast<float*>(qs),
-        row_bits);
+        row_bits, w.mask_words, key, clear_words);
   MSA_LAUNCH_CHECK();
 
   const int32_t K = bank->Hkv * bank->D;
   const int32_t bpq = w.S_pad / 32;
-  int rc;
-  if (bank->dtype == MSA_BF16) {
-#define MSA_GEMM(BM_, BN_, WM_, WN_)                                                                              \
-  launch_gemm<bf16_t, BM_, BN_, WM_, WN_>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C, \
-                                          K, bpq, exclusive, st)
-#define MSA_GEMM_DEEP(BM_, BN_, WM_, WN_)                                                                 \
-  launch_gemm<bf16_t, BM_, BN_, WM_, WN_, true>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows,   \
-                                                (int32_t)bank->C, K, bpq, exclusive, st)
-    switch (variant) {
-      case 0: rc = MSA_GEMM(64, 128, 2, 2); break;
-      case 1: rc = MSA_GEMM(128, 256, 2, 4); break;
-      case 2: rc = MSA_GEMM(256, 256, 2, 4); break;
-      case 3: rc = MSA_GEMM(256, 256, 4, 2); break;
-      case 4: rc = MSA_GEMM(128, 128, 2, 2); break;
-      case 5: rc = MSA_GEMM(128, 128, 2, 4); break;
-      case 6: rc = MSA_GEMM(128, 384, 2, 4); break;
-      case 7: rc = MSA_GEMM(128, 256, 4, 2); break;
-      case 8: rc = MSA_GEMM(128, 256, 1, 8); break;
-      case 9: rc = MSA_GEMM(128, 192, 2, 2); break;
-      case 10: rc = MSA_GEMM_DEEP(64, 128, 2, 2); break;
-      default: msa_set_error("MSA_SCORE_TILE=%d unknown", variant); return MSA_EINVAL;
-    }
-#undef MSA_GEMM
-#undef MSA_GEMM_DEEP
-  } else {
-    rc = launch_gemm<float, 128, 128, 2, 2>(qs, bank->kr_dev[layer], row_bits, chunk_key, w.M_rows, (int32_t)bank->C, K,
-                                            bpq, exclusive, st);
-  }
+  const int rc = doc_max ? launch_gemm_for<true>(bank->dtype, qs, bank->kr_dev[layer], row_bits, key, bank->chunk_doc_dev,
+                                                 w.M_rows, (int32_t)bank->C, K, bpq, (int32_t)bank->n_docs, st)
+                         : launch_gemm_for<false>(bank->dtype, qs, bank->kr_dev[layer], row_bits, key, nullptr, w.M_rows,
+                                                  (int32_t)bank->C, K, bpq, (int32_t)bank->n_docs, st);
   if (rc != MSA_OK) return rc;
   *layout_out = w;
   *mul_out = sc / (float)Hq;
@@ -563,11 +602,11 @@ extern "C" int msa_chunk_scores(const msa_bank* bank, int32_t layer, const void*
   RouteWorkspace w;
   float mul;
   hipStream_t st = as_stream(stream);
-  int rc = route_scores_to_keys(bank, layer, q, qmask_u8, B, S, Hq, mode, scale, workspace, workspace_bytes, st, &w,
-                                &mul, "msa_chunk_scores");
+  int rc = route_scores_to_keys(bank, layer, q, qmask_u8, B, S, Hq, mode, scale, false, workspace, workspace_bytes, st,
+                                &w, &mul, "msa_chunk_scores");
   if (rc != MSA_OK) return rc;
   const int64_t n = (int64_t)B * bank->C;
-  const uint32_t* key = reinterpret_cast<const uint32_t*>(static_cast<char*>(workspace) + w.off_chunk_key);
+  const uint32_t* key = reinterpret_cast<const uint32_t*>(static_cast<char*>(workspace) + w.off_key);
   decode_scores_kernel<<<(int)std::min<int64_t>((n + 255) / 256, 8192), 256, 0, st>>>(key, n, mul, chunk_scores);
   MSA_LAUNCH_CHECK();
   return MSA_OK;

@@ -1,4 +1,4 @@
-// Streaming document top-k: segmented max over each document's chunk keys fused with a
+// Streaming document top-k over the per-document keys the scoring kernel's epilogue leaves: a
 // wavefront-level bitonic select, an LDS merge across the workgroup's wavefronts, and a final
 // per-query merge of the per-workgroup candidate lists.
 //
@@ -45,29 +45,21 @@ __device__ __forceinline__ uint64_t wave_merge_desc(uint64_t best, uint64_t batc
   return v;
 }
 
-// Keys of one batch of 64 consecutive documents are contiguous in a query's row of the key plane.  The
-// wavefront copies that range into its own LDS window with aligned 16-byte loads (a lane reading its
-// document's keys straight from memory touches a different cache line per lane and instruction), then
-// every lane takes the maximum over its document's slice of the window.  Documents that cannot enter the
-// wavefront's top-k (composite not above the k-th best so far) are dropped by a ballot; the rest queue in
-// LDS and are sorted and merged 64 at a time, so the bitonic network runs a few times per wavefront, not
-// once per batch.
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-constexpr int kStageKeys = 2048;      // keys per LDS window, including up to 3 leading keys of alignment slack
+// The scoring kernel leaves one key per (query, document).  A wavefront walks its share of a workgroup's
+// documents 256 at a time (four coalesced loads in flight per lane).  Documents that cannot enter the wavefront's
+// top-k (composite not above the k-th best so far) are dropped by a ballot; the rest queue in LDS and are
+// sorted and merged 64 at a time, so the bitonic network runs a few times per wavefront, not once per batch.
+constexpr int kLoadsPerLane = 4;
 
-__global__ __launch_bounds__(kWaves * 64) void doc_topk_kernel(const uint32_t* __restrict__ chunk_key,
-                                                               const int32_t* __restrict__ doc_chunk_off,
-                                                               int64_t C, int32_t n_docs, int32_t topk,
-                                                               uint64_t* __restrict__ cand) {
-  __shared__ __attribute__((aligned(16))) uint32_t stage[kWaves][kStageKeys];
+__global__ __launch_bounds__(kWaves * 64) void doc_topk_kernel(const uint32_t* __restrict__ doc_key, int32_t n_docs,
+                                                               int32_t topk, uint64_t* __restrict__ cand) {
   __shared__ uint64_t pend[kWaves][128];
   __shared__ uint64_t lists[kWaves][64];
   const int b = blockIdx.y;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t* key = chunk_key + (int64_t)b * C;
+  const uint32_t* key = doc_key + (int64_t)b * n_docs;
   const int d_begin = blockIdx.x * kTopkDocsPerBlock;
   const int d_end = min(d_begin + kTopkDocsPerBlock, n_docs);
-  uint32_t* win = stage[wave];
   uint64_t* queue = pend[wave];
 
   uint64_t best = 0, thr = 0;
@@ -82,55 +74,27 @@ __global__ __launch_bounds__(kWaves * 64) void doc_topk_kernel(const uint32_t* _
     thr = shfl_u64(best, topk - 1);
   };
 
-  for (int base = d_begin + wave * 64; base < d_end; base += kWaves * 64) {   // wave-uniform trip count
-    const int d = base + lane;
-    int c0 = 0, c1 = 0;
-    if (d < d_end) { c0 = doc_chunk_off[d]; c1 = doc_chunk_off[d + 1]; }
-    const int r0 = __builtin_amdgcn_readfirstlane(c0);                                   // lane 0 is always a document
-    const int r1 = __builtin_amdgcn_readfirstlane(doc_chunk_off[min(base + 64, d_end)]);
-    uint32_t m = 0;
-    for (int w0 = r0; w0 < r1; w0 += kStageKeys - 4) {
-      const int wn = min(kStageKeys - 4, r1 - w0);
-      // window start moved down to a 16-byte boundary of the plane: `lead` keys of slack in front
-      const uint32_t* src = key + w0;
-      const int lead = (int)((reinterpret_cast<uintptr_t>(src) >> 2) & 3);
-      const u32x4_t* src4 = reinterpret_cast<const u32x4_t*>(src - lead);
-      const int n_vec = (lead + wn + 3) >> 2;                                            // <= kStageKeys / 4
-      u32x4_t x[kStageKeys / 256];
+  for (int base = d_begin + wave * 64 * kLoadsPerLane; base < d_end; base += kWaves * 64 * kLoadsPerLane) {   // wave-uniform
+    uint32_t kv[kLoadsPerLane];
 #pragma unroll
-      for (int u = 0; u < kStageKeys / 256; ++u) {
-        const int i = lane + 64 * u;
-        x[u] = i < n_vec ? __builtin_nontemporal_load(src4 + i) : u32x4_t{0, 0, 0, 0};
-      }
-#pragma unroll
-      for (int u = 0; u < kStageKeys / 256; ++u) {
-        const int i = lane + 64 * u;
-        if (i < n_vec) *reinterpret_cast<u32x4_t*>(win + 4 * i) = x[u];
-      }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-      __builtin_amdgcn_wave_barrier();
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-      const int lo = max(c0, w0) - w0 + lead, hi = min(c1, w0 + wn) - w0 + lead;         // empty when hi <= lo
-      for (int i = lo; i < hi; i += 8) {
-        uint32_t kv[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) kv[u] = win[min(i + u, hi - 1)];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) m = max(m, kv[u]);
-      }
-      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                             // reads done before the next window lands
-      __builtin_amdgcn_wave_barrier();
+    for (int u = 0; u < kLoadsPerLane; ++u) {
+      const int d = base + u * 64 + lane;
+      kv[u] = d < d_end ? __builtin_nontemporal_load(key + d) : 0u;
     }
-    const uint64_t v = d < d_end ? ((uint64_t)m << 32) | (uint64_t)(0xffffffffu - (uint32_t)d) : 0;
-    const bool in = v > thr;
-    const uint64_t mask = __ballot(in);
-    if (mask != 0) {
-      const int pos = n_pend + __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
-      if (in) queue[pos] = v;
-      n_pend += __builtin_popcountll(mask);
-      if (n_pend >= 64) {
-        n_pend -= 64;
-        flush(n_pend, 64);
+#pragma unroll
+    for (int u = 0; u < kLoadsPerLane; ++u) {
+      const int d = base + u * 64 + lane;
+      const uint64_t v = d < d_end ? ((uint64_t)kv[u] << 32) | (uint64_t)(0xffffffffu - (uint32_t)d) : 0;
+      const bool in = v > thr;
+      const uint64_t mask = __ballot(in);
+      if (mask != 0) {
+        const int pos = n_pend + __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0));
+        if (in) queue[pos] = v;
+        n_pend += __builtin_popcountll(mask);
+        if (n_pend >= 64) {
+          n_pend -= 64;
+          flush(n_pend, 64);
+        }
       }
     }
   }
@@ -195,14 +159,14 @@ extern "C" int msa_route_topk(const msa_bank* bank, int32_t layer, const void* q
   RouteWorkspace w;
   float mul;
   hipStream_t st = as_stream(stream);
-  int rc = route_scores_to_keys(bank, layer, q, qmask_u8, B, S, Hq, mode, scale, workspace, workspace_bytes, st, &w,
+  int rc = route_scores_to_keys(bank, layer, q, qmask_u8, B, S, Hq, mode, scale, true, workspace, workspace_bytes, st, &w,
                                 &mul, "msa_route_topk");
   if (rc != MSA_OK) return rc;
   char* ws = static_cast<char*>(workspace);
-  const uint32_t* key = reinterpret_cast<const uint32_t*>(ws + w.off_chunk_key);
+  const uint32_t* key = reinterpret_cast<const uint32_t*>(ws + w.off_key);
   uint64_t* cand = reinterpret_cast<uint64_t*>(ws + w.off_cand);
   dim3 grid((unsigned)w.topk_blocks, (unsigned)B);
-  doc_topk_kernel<<<grid, kWaves * 64, 0, st>>>(key, bank->doc_chunk_off_dev, bank->C, (int32_t)bank->n_docs, topk, cand);
+  doc_topk_kernel<<<grid, kWaves * 64, 0, st>>>(key, (int32_t)bank->n_docs, topk, cand);
   MSA_LAUNCH_CHECK();
   merge_topk_kernel<<<B, kMergeWaves * 64, 0, st>>>(cand, w.topk_blocks, bank->doc_global_id_dev, mul, topk, scores_out, doc_out,
                                       doc_global_out);

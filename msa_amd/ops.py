@@ -137,8 +137,12 @@ class Bank:
               "msa_bank_set_layer")
         self._keep[layer] = (kr, k_host, v_host)
 
-    def workspace(self, B: int, S: int, Hq: int, topk: int, device) -> torch.Tensor:
-        need = _lib.load().msa_route_workspace_bytes(B, S, Hq, self.Hkv, self.D, self.C, self.n_docs, topk)
+    def workspace(self, B: int, S: int, Hq: int, topk: int, device, chunk_plane: bool = False) -> torch.Tensor:
+        """Scratch for ``route_topk`` (pre-summed queries, row masks, one key per document, candidate lists);
+        with ``chunk_plane`` also room for the ``[B, C]`` key plane ``chunk_scores`` needs."""
+        lib = _lib.load()
+        need = (lib.msa_route_workspace_bytes(B, S, Hq, self.Hkv, self.D, self.C, self.n_docs, topk) if chunk_plane
+                else lib.msa_route_topk_workspace_bytes(B, S, Hq, self.Hkv, self.D, self.n_docs, topk))
         if self._ws is None or self._ws.numel() < need or self._ws.device != torch.device(device):
             self._ws = torch.empty(need, dtype=torch.uint8, device=device)
         return self._ws
@@ -173,7 +177,7 @@ def chunk_scores(bank: Bank, layer: int, q: torch.Tensor, qmask: Optional[torch.
                  scale: float = 1.0) -> torch.Tensor:
     """fp32 ``[B, C]`` chunk scores (mean over heads, max over scored tokens)."""
     B, S, Hq, qm = _route_args(bank, q, qmask, mode)
-    ws = bank.workspace(B, S, Hq, 16, q.device)
+    ws = bank.workspace(B, S, Hq, 16, q.device, chunk_plane=True)
     out = torch.empty((B, bank.C), dtype=torch.float32, device=q.device)
     check(_lib.load().msa_chunk_scores(bank.handle, layer, ptr(q), ptr(qm), B, S, Hq, MODES[mode], scale, ptr(out),
                                        ptr(ws), ws.numel(), _stream()), "msa_chunk_scores")

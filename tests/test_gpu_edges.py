@@ -363,9 +363,10 @@ def test_greedy_sample_against_argmax(ops, dtype, B, V):
 
 @pytest.mark.parametrize("B,S", [(16, 128), (4, 64), (3, 96), (2, 200), (1, 128), (5, 32), (9, 1), (20, 128)])
 def test_score_epilogue_forms_on_a_dirty_workspace(ops, B, S):
-    """Queries that fit one wavefront's tile are stored by a single writer into a key plane nobody cleared; the others
-    combine through atomicMax on a cleared plane.  Both must give the oracle's scores whatever the workspace held
-    before, and a query without a scored token must come back as -inf everywhere."""
+    """The scoring epilogue merges keys with atomicMax into a plane that the prologue kernel clears (per chunk for
+    chunk_scores, per document for route_topk) and reads row masks that the prologue writes word by word.  Both must
+    give the oracle's scores whatever the workspace held before, for queries that fit one wavefront's tile and for
+    queries that span several, and a query without a scored token must come back as -inf everywhere."""
     say(f"epilogue forms B={B} S={S}")
     bank, kr, dco, _ = _bank(ops, [3, 1, 7, 2, 9, 4, 1, 1, 12] * 41, 8, torch.bfloat16, 900 + B)
     q = _randn((B, S, 32, 128), 901 + S, torch.bfloat16)
@@ -373,7 +374,7 @@ def test_score_epilogue_forms_on_a_dirty_workspace(ops, B, S):
     mask[0, S // 2 + 1:] = False
     if B > 1:
         mask[B - 1] = False
-    bank.workspace(B, S, 32, 16, "cuda").fill_(0xFF)
+    bank.workspace(B, S, 32, 16, "cuda", chunk_plane=True).fill_(0xFF)
     got = ops.chunk_scores(bank, 0, q.cuda(), mask.cuda()).cpu()
     want = cf.chunk_scores(q, mask, kr, "cosine")
     live = mask.any(dim=1)

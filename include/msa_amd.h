@@ -113,6 +113,19 @@ int msa_route_topk(const msa_bank* bank, int32_t layer, const void* q, const uin
                    float* scores_out, int32_t* doc_out, int64_t* doc_global_out, void* workspace,
                    size_t workspace_bytes, void* stream);
 
+/* msa_route_topk for callers that cannot allocate or carry a workspace: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same arguments and results as
+ * msa_route_topk (bit for bit: it runs the same kernels), but the scratch is a device array built into the library,
+ * MSA_ROUTE_STATIC_SCRATCH_BYTES per device for the life of the process, and the call allocates nothing.  Sizes
+ * whose scratch need (msa_route_topk_workspace_bytes) exceeds that are refused with MSA_ESIZE; 16 queries of 128
+ * tokens over 87,000 documents need about 10 MiB.  The array's device address is looked up on the first call on
+ * each device (make that call outside graph capture).  All calls on one device share the array: calls that overlap
+ * in time on one device (different streams or threads) race and must be serialised by the caller. */
+#define MSA_ROUTE_STATIC_SCRATCH_BYTES (16 << 20)
+int msa_route_topk_static(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8,
+                          int32_t B, int32_t S, int32_t Hq, int32_t mode, float scale, int32_t topk,
+                          float* scores_out, int32_t* doc_out, int64_t* doc_global_out, void* stream);
+
 /* Measurement hook (no counterpart in the reference): while enabled, every launch of the scoring
  * kernel inside msa_chunk_scores / msa_route_topk is bracketed by a HIP event pair on its own
  * stream, up to max_records launches (0 disables and frees the events).  msa_profile_collect waits

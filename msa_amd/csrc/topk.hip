@@ -4,6 +4,8 @@
 //
 // Candidates are 64-bit composites (score key << 32 | ~doc) so one unsigned compare orders by
 // score descending, then document index ascending; 0 is the empty slot.
+#include <mutex>
+
 #include "route_internal.h"
 
 namespace {
@@ -172,4 +174,59 @@ extern "C" int msa_route_topk(const msa_bank* bank, int32_t layer, const void* q
                                       doc_global_out);
   MSA_LAUNCH_CHECK();
   return MSA_OK;
+}
+
+// ------------------------------------------------------------------------------------------
+// msa_route_topk without a workspace argument and without any allocation: the scratch (pre-summed queries, row
+// masks, one key per (query, document), candidate lists) lives in a device array of this code object.  Every
+// device the library runs on holds its own copy of the array at its own address, looked up once per device.
+// ------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[MSA_ROUTE_STATIC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Address of the current device's copy of `scratch` (the array's name is only a host-side handle).
+int scratch_of_current_device(void** out) {
+  int dev = -1;
+  MSA_HIP(hipGetDevice(&dev));
+  MSA_REQUIRE(dev >= 0 && dev < kMaxDevices, "msa_route_topk_static: device %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    MSA_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    MSA_REQUIRE(p != nullptr && ((uintptr_t)p & 255) == 0, "msa_route_topk_static: bad scratch address");
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return MSA_OK;
+}
+
+}  // namespace
+
+extern "C" int msa_route_topk_static(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8,
+                                     int32_t B, int32_t S, int32_t Hq, int32_t mode, float scale, int32_t topk,
+                                     float* scores_out, int32_t* doc_out, int64_t* doc_global_out, void* stream) {
+  MSA_REQUIRE(bank != nullptr, "msa_route_topk_static: null bank");
+  MSA_REQUIRE(B > 0 && S > 0 && Hq > 0, "msa_route_topk_static: B=%d S=%d Hq=%d", B, S, Hq);
+  const size_t need = route_workspace_layout(B, S, bank->Hkv, bank->D, bank->n_docs, bank->n_docs, bank->dtype).bytes;
+  if (need > (size_t)MSA_ROUTE_STATIC_SCRATCH_BYTES) {
+    msa_set_error("msa_route_topk_static: B=%d x S=%d queries over %lld documents need %zu bytes of scratch, the "
+                  "built-in buffer holds %d; use msa_route_topk with a workspace", B, S, (long long)bank->n_docs,
+                  need, MSA_ROUTE_STATIC_SCRATCH_BYTES);
+    return MSA_ESIZE;
+  }
+  int dev = -1;
+  MSA_HIP(hipGetDevice(&dev));
+  MSA_REQUIRE(dev == bank->device, "msa_route_topk_static: bank lives on device %d, current device is %d", bank->device, dev);
+  void* ws = nullptr;
+  const int rc = scratch_of_current_device(&ws);
+  if (rc != MSA_OK) return rc;
+  // every byte of the scratch a call reads is written by that call's own kernels first (the prologue writes the
+  // queries and all mask words and clears the key plane; the select kernel writes every candidate list)
+  return msa_route_topk(bank, layer, q, qmask_u8, B, S, Hq, mode, scale, topk, scores_out, doc_out, doc_global_out, ws,
+                        MSA_ROUTE_STATIC_SCRATCH_BYTES, stream);
 }

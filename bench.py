@@ -510,8 +510,8 @@ def main():
 
     if extras is not None and not args.no_e2e:
         # configs[4] end to end (the "sparse decode tok/s" half of the metric); ~25 GB next to the 100M bank's 60 GB
-        from msa_amd import e2e_decode
-        r = e2e_decode.main(["--steps", "256"], quiet=True)
+        import bench_e2e
+        r = bench_e2e.main(["--steps", "256"], quiet=True)
         extras["e2e_sparse_decode"] = {"workload": r["config"]["workload"] + ", 10M-token bank, B=16, 4K context, greedy",
                                        "tokens_per_s": r["value"], "ms_per_decode_step": r["ms_per_decode_step"],
                                        "prefill_s": r["prefill_s"], "decode_steps": r["config"]["decode_steps"],

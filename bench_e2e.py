@@ -2,7 +2,7 @@
 36 layers, routing on the upper 18, a synthetic pooled memory bank, top-16 documents, a 4K-token
 local context per query, batch 16, greedy decoding.
 
-    python -m msa_amd.e2e_decode [--bank-tokens 10000000] [--batch 16] [--context 4096] [--steps 256]
+    python bench_e2e.py [--bank-tokens 10000000] [--batch 16] [--context 4096] [--steps 256]
 
 Prints one JSON line with prefill time and decode tokens/s.  The bank is synthetic at the pooled
 level (N(0,1) rows, K_r L2-normalised): encoding 10M tokens through a 4B-parameter model is not part
@@ -18,10 +18,14 @@ import time
 import numpy as np
 import torch
 
-from .config import GenerateConfig, MemoryConfig, ModelConfig, MSAConfig
-from .model import MSAForCausalLM, encode_block
-from .msa_service import MSAService
-from .prefill import Document, num_chunks, prepare_block_inputs
+import os
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+from msa_amd.config import GenerateConfig, MemoryConfig, ModelConfig, MSAConfig
+from msa_amd.model import MSAForCausalLM, encode_block
+from msa_amd.msa_service import MSAService
+from msa_amd.prefill import Document, num_chunks, prepare_block_inputs
 
 
 def build_service(cfg: MSAConfig, bank_tokens: int, seed: int = 0) -> MSAService:
@@ -94,7 +98,7 @@ def main(argv=None, quiet: bool = False):
                     help="also decode N steps eagerly and require identical tokens from the graph replays")
     args = ap.parse_args(argv)
     if not torch.cuda.is_available():
-        sys.exit("e2e_decode: no GPU visible; the HIP path has no CPU fallback")
+        sys.exit("bench_e2e: no GPU visible; the HIP path has no CPU fallback")
     dev = torch.device("cuda:0")
     cfg = MSAConfig(num_hidden_layers=args.layers)
     if args.layers != 36:
@@ -135,7 +139,7 @@ def main(argv=None, quiet: bool = False):
         if not verified:
             diff = ref != toks[:, :args.verify_graph]
             first = int(diff.any(dim=0).nonzero()[0])
-            sys.exit(f"e2e_decode: graph replays and eager decoding produced different tokens: first at step {first}, "
+            sys.exit(f"bench_e2e: graph replays and eager decoding produced different tokens: first at step {first}, "
                      f"{int(diff.any(dim=1).sum())} of {B} samples differ")
     last_router = svc.router_layer_ids[-1]
     kv = cache.cache_kwargs[last_router]["kv_lengths"].cpu().tolist()

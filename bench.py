@@ -29,10 +29,38 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 HQ, HKV, D, P, TOPK = 32, 8, 128, 64, 16
-# Bytes past L2 per launch of the scoring kernel at the default workload, from rocprofv3 --pmc FETCH_SIZE and
-# WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a plain 1 GiB device copy
-# (FETCH_SIZE x2.0, WRITE_SIZE x1.0); see profiles/score_gemm_c4_100M_bank.txt.
-SCORE_TRAFFIC_DEFAULT_WORKLOAD = (2.0 * 3_374_335 + 1.0 * 156_209) * 1024
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def measured_traffic(kernel: str, workload: str):
+    """Bytes past L2 per launch of `kernel` at `workload`, from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+    summaries under profiles/: a line `TRAFFIC kernel=<k> workload=<w> fetch_kib=<n> write_kib=<n> fetch_scale=<f>
+    write_scale=<f>` (KiB per dispatch and the factors a plain device copy of known size gives for the same
+    counters).  None when no summary covers the workload."""
+    try:
+        names = sorted(os.listdir(PROFILES))
+    except OSError:
+        return None
+    for name in names:
+        if not name.endswith((".txt", ".md")):
+            continue
+        for line in open(os.path.join(PROFILES, name), errors="replace"):
+            if not line.startswith("TRAFFIC "):
+                continue
+            kv = dict(f.split("=", 1) for f in line.split()[1:] if "=" in f)
+            if kv.get("kernel") == kernel and kv.get("workload") == workload:
+                return (float(kv["fetch_scale"]) * float(kv["fetch_kib"]) + float(kv["write_scale"]) * float(kv["write_kib"])) * 1024
+    return None
+
+
+def cpu_model() -> str:
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def log(msg):
@@ -294,6 +322,9 @@ def main():
                          "memcpy: ids to the host, one hipMemcpyAsync per document run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
+    ap.add_argument("--sweep-only", action="store_true",
+                    help="run the bandwidth-regime sweep (one query per scan) and stop; with --layers 1 this is the "
+                         "short run the rocprofv3 summaries of that regime come from")
     ap.add_argument("--no-extras", action="store_true", help="skip the pooling and decode-attention side measurements")
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end sparse decode run among the extras")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -453,35 +484,10 @@ def main():
         gbs = bytes_layer / (kern_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
-    if (args.tokens, B, S) == (100_000_000, 16, 128):
-        roof["traffic"] = SCORE_TRAFFIC_DEFAULT_WORKLOAD
+    roof["traffic"] = measured_traffic("score_gemm_kernel", f"tokens={args.tokens},B={B},S={S}")
     roof.update({"kernel": "score_gemm_kernel", "kernel_ms": round(kern_ms, 4), "launches_timed": n_rec.value,
                  "flops_per_launch": flops, "algorithmic_bytes_per_launch": bytes_layer,
                  "hbm_gbs_at_this_batch": round(bytes_layer / (kern_ms * 1e-3) / 1e9, 1)})
-
-    # ---- bandwidth-bound regime: one query (and fewer tokens) per scan of layer 0
-    sweep = []
-    if not args.no_sweep:
-        for b1, s1 in ((1, 1), (1, 16), (1, 64), (1, 128), (2, 128), (4, 128)):
-            q1 = qs[0][:b1, :s1].contiguous()
-            sc = torch.empty((b1, TOPK), dtype=torch.float32, device=dev)
-            dc = torch.empty((b1, TOPK), dtype=torch.int32, device=dev)
-            reps = 5
-            for r in range(reps + 1):
-                if r == 1:
-                    torch.cuda.synchronize()
-                    _lib.check(lib.msa_profile_enable(reps), "msa_profile_enable")
-                _lib.check(lib.msa_route_topk(bank.handle, 0, q1.data_ptr(), None, b1, s1, HQ, _lib.MODE_COSINE, 1.0,
-                                              TOPK, sc.data_ptr(), dc.data_ptr(), None, ws.data_ptr(), ws.numel(),
-                                              main_stream.cuda_stream), "msa_route_topk")
-            torch.cuda.synchronize()
-            buf = (C.c_float * reps)()
-            _lib.check(lib.msa_profile_collect(buf, reps, C.byref(n_rec)), "msa_profile_collect")
-            ms1 = float(np.mean(list(buf)[: n_rec.value]))
-            by = C_total * HKV * D * 2 + b1 * s1 * HKV * D * 2
-            sweep.append({"B": b1, "S": s1, "kernel_ms": round(ms1, 4), "GB/s": round(by / ms1 / 1e6, 1),
-                          "frac_hbm": round(by / ms1 / 1e6 / HBM_PEAK_GBS, 4)})
-        _lib.check(lib.msa_profile_enable(0), "msa_profile_enable")
 
     if args.calibrate_copy:
         src = torch.empty(1 << 29, dtype=torch.bfloat16, device=dev).fill_(1.0)     # 1 GiB
@@ -490,6 +496,39 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    # ---- bandwidth-bound regime: one query (and fewer tokens) per scan of layer 0.  `call_ms` is the whole
+    # msa_route_topk call (prologue, scan with the per-document max in its epilogue, top-k select and merge) timed
+    # with events on its stream over back-to-back calls; `frac_hbm` is the algorithmic bytes over that time.
+    sweep = []
+    if not args.no_sweep:
+        for b1, s1 in ((1, 1), (1, 16), (1, 64), (1, 128), (2, 128), (4, 128)):
+            q1 = qs[0][:b1, :s1].contiguous()
+            sc = torch.empty((b1, TOPK), dtype=torch.float32, device=dev)
+            dc = torch.empty((b1, TOPK), dtype=torch.int32, device=dev)
+            reps = 10
+
+            def call():
+                _lib.check(lib.msa_route_topk(bank.handle, 0, q1.data_ptr(), None, b1, s1, HQ, _lib.MODE_COSINE, 1.0,
+                                              TOPK, sc.data_ptr(), dc.data_ptr(), None, ws.data_ptr(), ws.numel(),
+                                              main_stream.cuda_stream), "msa_route_topk")
+            call_ms = time_cuda(call, reps)
+            torch.cuda.synchronize()
+            _lib.check(lib.msa_profile_enable(reps), "msa_profile_enable")
+            for _ in range(reps):
+                call()
+            torch.cuda.synchronize()
+            buf = (C.c_float * reps)()
+            _lib.check(lib.msa_profile_collect(buf, reps, C.byref(n_rec)), "msa_profile_collect")
+            ms1 = float(np.mean(list(buf)[: n_rec.value]))
+            by = C_total * HKV * D * 2 + b1 * s1 * HQ * D * 2 + C_total * 4 + b1 * TOPK * 16
+            sweep.append({"B": b1, "S": s1, "call_ms": round(call_ms, 4), "GB/s": round(by / call_ms / 1e6, 1),
+                          "frac_hbm": round(by / call_ms / 1e6 / HBM_PEAK_GBS, 4), "scan_kernel_ms": round(ms1, 4),
+                          "scan_kernel_frac_hbm": round(by / ms1 / 1e6 / HBM_PEAK_GBS, 4)})
+        _lib.check(lib.msa_profile_enable(0), "msa_profile_enable")
+    if args.sweep_only:
+        print(json.dumps({"hbm_regime_sweep": sweep}), flush=True)
+        return
 
     extras = None
     if not args.no_extras:
@@ -506,7 +545,7 @@ def main():
                          f"first {Cs} of {C_total} chunks of layer 0 for the same {B}x{S} queries; "
                          f"{', '.join(f'{k} {v:.2f} s' for k, v in times.items())}; best extrapolated linearly "
                          f"x{C_total / Cs:.1f} chunks x{L} layers",
-               "host_cpus": os.cpu_count()}
+               "host_cpus": os.cpu_count(), "cpu_model": cpu_model()}
 
     if extras is not None and not args.no_e2e:
         # configs[4] end to end (the "sparse decode tok/s" half of the metric); ~25 GB next to the 100M bank's 60 GB

@@ -141,7 +141,12 @@ struct Mma<float> {
 // more bytes in flight per compute unit than one tile holds.
 // kDocMax: keys are folded over the chunks of a document (chunk_doc) and merged into out_key[B, n_docs];
 // otherwise one key per (query, chunk) is merged into out_key[B, C].
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool kDocMax>
+// kStream: one workgroup per compute-unit slot walks N tiles blockIdx.x, blockIdx.x + gridDim.x, ... (one M tile
+// only) with the load / store / multiply pipeline running across tile boundaries: the first K tiles of the next N
+// tile are already in flight while the last ones of the current tile are multiplied and its epilogue runs, so the
+// HBM stream never drains between tiles.  That is what the HBM-bound shapes need; the MFMA-bound ones keep one
+// workgroup per tile, which leaves compute units free for kernels of other streams.
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool kDocMax, bool kStream>
 __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     const T* __restrict__ qs,            // [M_rows, K]  pre-summed queries, M_rows = B * S_pad
     const T* __restrict__ kr,            // [C, K]
@@ -162,12 +167,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so each XCD gets one
   // contiguous range of K_r tiles.  Inside it the M tiles are walked in groups of m_group: a group's
   // query rows stay in that XCD's L2 while its K_r tiles stream past once per group.
-  const int n_per_xcd = (tiles_n + 7) / 8;
-  const int within = blockIdx.x / 8;
-  const int per_group = n_per_xcd * m_group;
-  const int rem = within % per_group;
-  const int tile_n = (blockIdx.x % 8) * n_per_xcd + rem / m_group;
-  const int tile_m = (within / per_group) * m_group + rem % m_group;
+  int tile_n, tile_m;
+  if constexpr (kStream) {
+    tile_n = blockIdx.x;
+    tile_m = 0;
+  } else {
+    const int n_per_xcd = (tiles_n + 7) / 8;
+    const int within = blockIdx.x / 8;
+    const int per_group = n_per_xcd * m_group;
+    const int rem = within % per_group;
+    tile_n = (blockIdx.x % 8) * n_per_xcd + rem / m_group;
+    tile_m = (within / per_group) * m_group + rem % m_group;
+  }
   if (tile_n >= tiles_n || tile_m >= tiles_m) return;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
@@ -184,14 +195,18 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   // clamps).  The range check is defined on the vector offset, so the row displacement of a thread's
   // vectors rides there; the K-tile displacement (which stays inside the row, so it can never carry a
   // load past the extent) is scalar.
-  const int rows_a = min(BM, M_rows - m0), rows_b = min(BN, C - n0);
+  const int rows_a = min(BM, M_rows - m0);
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(ga) + (int64_t)m0 * row_bytes_g, 0, (int)(rows_a * row_bytes_g), 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
-      const_cast<char*>(gb) + (int64_t)n0 * row_bytes_g, 0, (int)(rows_b * row_bytes_g), 0x00020000);
+  auto bank_rsrc = [&](int first_row) {       // the N tile starting at chunk `first_row` (empty past the bank)
+    const int rows = max(0, min(BN, C - first_row));
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(gb) + (int64_t)min(first_row, C) * row_bytes_g, 0,
+                                             (int)(rows * row_bytes_g), 0x00020000);
+  };
+  __amdgpu_buffer_rsrc_t rsrc_b = bank_rsrc(n0);
   const int voff = (tid >> 3) * (int)row_bytes_g + (tid & 7) * 16;
   const int vec_stride = (kThreads / 8) * (int)row_bytes_g;     // rows between a thread's vectors
-  static_assert(kSets >= 1 && kSets <= 3, "one to three K tiles in flight");
+  static_assert(kSets == 1 || kSets == 2, "one or two K tiles in flight");
   u32x4_t ra[kSets][kVecA], rb[kSets][kVecB];
   // K_r streams through once per M tile group while the query matrix is re-read by every workgroup of an XCD: the
   // non-temporal hint on the K_r loads keeps the queries in the 4 MiB L2 (traffic past L2 9.9 -> 6.9 GB per launch
@@ -209,6 +224,17 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     for (int i = 0; i < kVecB; ++i)
       rb[set][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo + i * vec_stride, kt * kRowBytes, kStreamHint);
   };
+  // kStream: the loads walk the workgroup's whole sequence of (N tile, K tile) steps; past its last tile they
+  // fetch nothing.
+  int ld_n0 = n0, ld_kt = 0;
+  auto load_next = [&](auto set_tag) {
+    load_tile(set_tag, ld_n0 < C ? ld_kt : k_tiles);
+    if (++ld_kt == k_tiles) {
+      ld_kt = 0;
+      ld_n0 = (int)min((int64_t)ld_n0 + (int64_t)gridDim.x * BN, (int64_t)C);
+      rsrc_b = bank_rsrc(ld_n0);
+    }
+  };
   auto store_tile = [&](auto set_tag, int buf) {
     constexpr int set = decltype(set_tag)::value;
 #pragma unroll
@@ -224,7 +250,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   };
   typedef std::integral_constant<int, 0> Set0;
   typedef std::integral_constant<int, 1 % kSets> Set1;
-  typedef std::integral_constant<int, 2 % kSets> Set2;
 
   floatx16_t acc[TM][TN];
 #pragma unroll
@@ -255,13 +280,13 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     for (int j = 0; j < TN; ++j) fb[slot][j] = Mma<T>::load(pb + j * 32 * kRowStride, sub, half);
   };
 
-  // One K tile out of LDS buffer `buf`; kMore says a next tile exists (the steady-state loop is
+  // One K tile out of LDS buffer `step & 1`; kMore says a next step exists (the steady-state loop is
   // compiled without that condition so the wait counters around the barrier stay exact).  Tile t travels in
-  // register set t % kSets; `set_tag` names the set that holds tile kt+1, which is stored and then refilled with
-  // tile kt+1+kSets.
-  auto k_tile = [&](auto more_tag, auto set_tag, int kt) {
+  // register set t % kSets; `set_tag` names the set that holds the next step's tile, which is stored and then
+  // refilled with the tile kSets steps further on.
+  auto k_tile = [&](auto more_tag, auto set_tag, int step) {
     constexpr bool kMore = decltype(more_tag)::value;
-    const int buf = kt & 1;
+    const int buf = step & 1;
 #pragma unroll
     for (int sub = 0; sub < kSub; ++sub) {
       if (sub + 1 < kSub) {
@@ -273,11 +298,14 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
       }
       if (sub == 1 && kMore) {
         store_tile(set_tag, buf ^ 1);
-        if constexpr (kSets > 1) {
+        if constexpr (kStream) {
           __builtin_amdgcn_sched_barrier(0);   // the refill reuses the registers the stores above read
-          load_tile(set_tag, kt + 1 + kSets);
-        } else if (kt + 2 < k_tiles) {
-          load_tile(set_tag, kt + 2);
+          load_next(set_tag);
+        } else if constexpr (kSets > 1) {
+          __builtin_amdgcn_sched_barrier(0);
+          load_tile(set_tag, step + 1 + kSets);
+        } else if (step + 2 < k_tiles) {
+          load_tile(set_tag, step + 2);
         }
       }
 #pragma unroll
@@ -287,63 +315,11 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     }
   };
 
-  if constexpr (kSets == 3) {
-    load_tile(Set0{}, 0);
-    store_tile(Set0{}, 0);
-    load_tile(Set1{}, 1);
-    load_tile(Set2{}, 2);
-    load_tile(Set0{}, 3);
-    __syncthreads();
-    load_frags(0, 0, 0);
-    int kt = 0;
-    for (; kt + 3 < k_tiles; kt += 3) {
-      k_tile(std::true_type{}, Set1{}, kt);
-      k_tile(std::true_type{}, Set2{}, kt + 1);
-      k_tile(std::true_type{}, Set0{}, kt + 2);
-    }
-    const int left = k_tiles - kt;             // 1..3 tiles
-    if (left == 1) {
-      k_tile(std::false_type{}, Set1{}, kt);
-    } else if (left == 2) {
-      k_tile(std::true_type{}, Set1{}, kt);
-      k_tile(std::false_type{}, Set2{}, kt + 1);
-    } else {
-      k_tile(std::true_type{}, Set1{}, kt);
-      k_tile(std::true_type{}, Set2{}, kt + 1);
-      k_tile(std::false_type{}, Set0{}, kt + 2);
-    }
-  } else if constexpr (kSets == 2) {
-    load_tile(Set0{}, 0);
-    store_tile(Set0{}, 0);
-    load_tile(Set1{}, 1);
-    load_tile(Set0{}, 2);
-    __syncthreads();
-    load_frags(0, 0, 0);
-    int kt = 0;
-    for (; kt + 2 < k_tiles; kt += 2) {
-      k_tile(std::true_type{}, Set1{}, kt);
-      k_tile(std::true_type{}, Set0{}, kt + 1);
-    }
-    if (kt + 1 < k_tiles) {
-      k_tile(std::true_type{}, Set1{}, kt);
-      k_tile(std::false_type{}, Set0{}, kt + 1);
-    } else {
-      k_tile(std::false_type{}, Set1{}, kt);
-    }
-  } else {
-    load_tile(Set0{}, 0);
-    store_tile(Set0{}, 0);
-    if (k_tiles > 1) load_tile(Set0{}, 1);
-    __syncthreads();
-    load_frags(0, 0, 0);
-    for (int kt = 0; kt + 1 < k_tiles; ++kt) k_tile(std::true_type{}, Set0{}, kt);
-    k_tile(std::false_type{}, Set0{}, k_tiles - 1);
-  }
-
-  // Epilogue.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of its 32x32 block.  Consecutive row
-  // blocks of one query are folded into `run`; emit() then merges the query's 32 column maxima of this block
-  // into the key plane.  Several wavefronts and workgroups hold parts of a query (and of a document), so the
-  // merge is an atomicMax into a zeroed plane.  emit() is reached by whole wavefronts (q and any are uniform).
+  // Epilogue of the N tile starting at chunk `tile_n0`.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of
+  // its 32x32 block.  Consecutive row blocks of one query are folded into `run`; emit() then merges the query's 32
+  // column maxima of this block into the key plane.  Several wavefronts and workgroups hold parts of a query (and
+  // of a document), so the merge is an atomicMax into a zeroed plane.  emit() is reached by whole wavefronts (q
+  // and any are uniform).
   const int n_queries = M_rows / (blocks_per_query * 32);
   auto emit = [&](int q, int n, float run, bool any) {
     if (!any || q >= n_queries) return;
@@ -367,34 +343,100 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
       if (ok && half == 0) atomicMax(&out_key[(int64_t)q * C + n], key);
     }
   };
+  auto epilogue = [&](int tile_n0) {
 #pragma unroll
-  for (int j = 0; j < TN; ++j) {
-    const int n = n0 + wn * WN + j * 32 + l32;
-    float run = -INFINITY;
-    bool any = false;
-    int run_q = -1;
+    for (int j = 0; j < TN; ++j) {
+      const int n = tile_n0 + wn * WN + j * 32 + l32;
+      float run = -INFINITY;
+      bool any = false;
+      int run_q = -1;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int blk = (m0 + wm * WM + i * 32) >> 5;      // global 32-row block index
-      const int qid = blk / blocks_per_query;
-      const uint32_t bits = row_bits[blk];               // 0 for blocks past M_rows (buffer is padded)
-      if (qid != run_q) {
-        if (run_q >= 0) emit(run_q, n, run, any);
-        run = -INFINITY; any = false; run_q = qid;
-      }
-      if (bits != 0) {
-        float mx = -INFINITY;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int r = 8 * (e >> 2) + 4 * half + (e & 3);
-          if (bits & (1u << r)) mx = fmaxf(mx, acc[i][j][e]);
+      for (int i = 0; i < TM; ++i) {
+        const int blk = (m0 + wm * WM + i * 32) >> 5;      // global 32-row block index
+        const int qid = blk / blocks_per_query;
+        const uint32_t bits = row_bits[blk];               // 0 for blocks past M_rows (buffer is padded)
+        if (qid != run_q) {
+          if (run_q >= 0) emit(run_q, n, run, any);
+          run = -INFINITY; any = false; run_q = qid;
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        run = fmaxf(run, mx);
-        any = true;
+        if (bits != 0) {
+          float mx = -INFINITY;
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int r = 8 * (e >> 2) + 4 * half + (e & 3);
+            if (bits & (1u << r)) mx = fmaxf(mx, acc[i][j][e]);
+          }
+          mx = fmaxf(mx, __shfl_xor(mx, 32));
+          run = fmaxf(run, mx);
+          any = true;
+        }
+      }
+      emit(run_q, n, run, any);
+    }
+  };
+
+  if constexpr (kStream) {
+    // The workgroup's tiles form one sequence of steps (K tiles are even in number, so set tags and LDS buffers
+    // alternate the same way in every tile); an epilogue sits where a tile's last step ends, with the next tile's
+    // first operand fragments already in registers and its loads in flight.
+    const int my_tiles = (tiles_n - tile_n + (int)gridDim.x - 1) / (int)gridDim.x;
+    const int steps = my_tiles * k_tiles;
+    load_next(Set0{});
+    store_tile(Set0{}, 0);
+    load_next(Set1{});
+    if constexpr (kSets == 2) load_next(Set0{});
+    __syncthreads();
+    load_frags(0, 0, 0);
+    int done_n0 = n0, in_tile = 0;
+    for (int step = 0; step + 2 < steps; step += 2) {
+      k_tile(std::true_type{}, Set1{}, step);
+      k_tile(std::true_type{}, Set0{}, step + 1);
+      in_tile += 2;
+      if (in_tile == k_tiles) {
+        epilogue(done_n0);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        in_tile = 0;
+        done_n0 += (int)gridDim.x * BN;
       }
     }
-    emit(run_q, n, run, any);
+    k_tile(std::true_type{}, Set1{}, steps - 2);
+    k_tile(std::false_type{}, Set0{}, steps - 1);
+    epilogue(done_n0);
+  } else {
+    if constexpr (kSets == 2) {
+      // tile t travels in register set (t & 1): iteration kt stores tile kt+1 and refills its set with tile kt+3
+      load_tile(Set0{}, 0);
+      store_tile(Set0{}, 0);
+      load_tile(Set1{}, 1);
+      load_tile(Set0{}, 2);
+      __syncthreads();
+      load_frags(0, 0, 0);
+      int kt = 0;
+      for (; kt + 2 < k_tiles; kt += 2) {
+        k_tile(std::true_type{}, Set1{}, kt);
+        k_tile(std::true_type{}, Set0{}, kt + 1);
+      }
+      if (kt + 1 < k_tiles) {
+        k_tile(std::true_type{}, Set1{}, kt);
+        k_tile(std::false_type{}, Set0{}, kt + 1);
+      } else {
+        k_tile(std::false_type{}, Set1{}, kt);
+      }
+    } else {
+      load_tile(Set0{}, 0);
+      store_tile(Set0{}, 0);
+      if (k_tiles > 1) load_tile(Set0{}, 1);
+      __syncthreads();
+      load_frags(0, 0, 0);
+      for (int kt = 0; kt + 1 < k_tiles; ++kt) k_tile(std::true_type{}, Set0{}, kt);
+      k_tile(std::false_type{}, Set0{}, k_tiles - 1);
+    }
+    epilogue(n0);
   }
 }
 
@@ -419,18 +461,40 @@ struct KernelTimer {
   int n = 0;
 } g_timer;
 
-template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool kDocMax>
+constexpr size_t kLdsPerCu = 160 * 1024;
+
+// Compute units of the current device (asked once; the library drives one device per process).
+int compute_units() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    return cus;
+  }();
+  return n;
+}
+
+template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool kDocMax, bool kStream>
 int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key, const int32_t* chunk_doc,
                 int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t n_docs, hipStream_t st) {
-  const int tiles_m = (M_rows + BM - 1) / BM, tiles_n = (C + BN - 1) / BN;
+  const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
+  const int tiles_m = (M_rows + BM - 1) / BM;
+  const int tiles_n = (C + BN - 1) / BN;
   // M tiles are walked in groups of 8 per K_r tile: a group's query rows (4 MiB in bf16) are what an XCD's L2
   // holds.  At 8 M tiles that is all of them (groups of 1, 2, 4 lose 2-14 % there); with 16 M tiles groups of 8
   // measured 1.4 % faster than one group, with 256 (a 64k-row prefill batch) 4 %.
   const int m_group = std::min(tiles_m, 8);
   const int m_groups = (tiles_m + m_group - 1) / m_group;
-  const int grid = 8 * ((tiles_n + 7) / 8) * m_groups * m_group;
-  const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
-  auto kern = score_gemm_kernel<T, BM, BN, WAVES_M, WAVES_N, kSets, kDocMax>;
+  int grid = 8 * ((tiles_n + 7) / 8) * m_groups * m_group;
+  if (kStream) {      // one workgroup per slot the compute units offer (LDS decides how many fit), each walking several tiles
+    if (tiles_m != 1) {
+      msa_set_error("score_gemm: the streaming form takes one M tile, got %d", tiles_m);
+      return MSA_EINVAL;
+    }
+    grid = std::min(tiles_n, compute_units() * std::max<int>(1, (int)(kLdsPerCu / lds)));
+  }
+  auto kern = score_gemm_kernel<T, BM, BN, WAVES_M, WAVES_N, kSets, kDocMax, kStream>;
   static std::atomic<int> lds_limit_raised{0};
   MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(kern), (int)lds));
   int slot = -1;
@@ -447,20 +511,22 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
   return MSA_OK;
 }
 
-// Tile choice by query rows.  Few rows are HBM-bound: narrow M tile, more workgroups in flight and K tiles of
-// global loads ahead of the one being multiplied (Little's law: a compute unit needs about 60 KB of loads in flight
-// to draw its share of the HBM rate).  Many rows are MFMA-bound: 256 x 256 tile, 8 wavefronts, one tile ahead.
+// Tile choice by query rows.  Up to 64 rows: narrow M tile, two workgroups per compute unit, two K tiles of global
+// loads ahead (3 % faster than one).  Up to 128 rows: the widest N tile that fits LDS, so the query tile a workgroup
+// re-reads from L2 per K_r tile is the smallest share of its intake (128 x 384 beats 128 x 256 by 3 % and 128 x 128
+// by 8 %; a second or third register set of loads in flight, or 16 wavefronts instead of 8, measured 0-6 % slower
+// here: the bytes in flight are not what limits this shape).  More rows are MFMA-bound: 256 x 256 tile.
 template <bool kDocMax>
 int launch_gemm_for(int32_t dtype, const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key,
                     const int32_t* chunk_doc, int32_t M_rows, int32_t C, int32_t K, int32_t bpq, int32_t n_docs,
                     hipStream_t st) {
   if (dtype != MSA_BF16)
-    return launch_gemm<float, 128, 128, 2, 2, 1, kDocMax>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
+    return launch_gemm<float, 128, 128, 2, 2, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
   if (M_rows <= 64)
-    return launch_gemm<bf16_t, 64, 128, 2, 2, 2, kDocMax>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
+    return launch_gemm<bf16_t, 64, 128, 2, 2, 2, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
   if (M_rows <= 128)
-    return launch_gemm<bf16_t, 128, 384, 2, 4, 1, kDocMax>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
-  return launch_gemm<bf16_t, 256, 256, 2, 4, 1, kDocMax>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
+    return launch_gemm<bf16_t, 128, 384, 2, 4, 1, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
+  return launch_gemm<bf16_t, 256, 256, 2, 4, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
 }
 
 }  // namespace

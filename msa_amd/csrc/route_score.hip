@@ -198,12 +198,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   const int rows_a = min(BM, M_rows - m0);
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(ga) + (int64_t)m0 * row_bytes_g, 0, (int)(rows_a * row_bytes_g), 0x00020000);
-  auto bank_rsrc = [&](int first_row) {       // the N tile starting at chunk `first_row` (empty past the bank)
-    const int rows = max(0, min(BN, C - first_row));
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(gb) + (int64_t)min(first_row, C) * row_bytes_g, 0,
-                                             (int)(rows * row_bytes_g), 0x00020000);
-  };
-  __amdgpu_buffer_rsrc_t rsrc_b = bank_rsrc(n0);
+  const int rows_b = min(BN, C - n0);
+  const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<char*>(gb) + (int64_t)n0 * row_bytes_g, 0, (int)(rows_b * row_bytes_g), 0x00020000);
+  __amdgpu_buffer_rsrc_t rsrc_ld = rsrc_b;      // kStream: the N tile the loads have reached
   const int voff = (tid >> 3) * (int)row_bytes_g + (tid & 7) * 16;
   const int vec_stride = (kThreads / 8) * (int)row_bytes_g;     // rows between a thread's vectors
   static_assert(kSets == 1 || kSets == 2, "one or two K tiles in flight");
@@ -221,8 +219,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     for (int i = 0; i < kVecA; ++i)
       ra[set][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, vo + i * vec_stride, kt * kRowBytes, 0);
 #pragma unroll
-    for (int i = 0; i < kVecB; ++i)
-      rb[set][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo + i * vec_stride, kt * kRowBytes, kStreamHint);
+    for (int i = 0; i < kVecB; ++i) {
+      if constexpr (kStream)
+        rb[set][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_ld, vo + i * vec_stride, kt * kRowBytes, kStreamHint);
+      else
+        rb[set][i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, vo + i * vec_stride, kt * kRowBytes, kStreamHint);
+    }
   };
   // kStream: the loads walk the workgroup's whole sequence of (N tile, K tile) steps; past its last tile they
   // fetch nothing.
@@ -232,7 +234,8 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     if (++ld_kt == k_tiles) {
       ld_kt = 0;
       ld_n0 = (int)min((int64_t)ld_n0 + (int64_t)gridDim.x * BN, (int64_t)C);
-      rsrc_b = bank_rsrc(ld_n0);
+      rsrc_ld = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(gb) + (int64_t)ld_n0 * row_bytes_g, 0,
+                                                  (int)(min(BN, C - ld_n0) * row_bytes_g), 0x00020000);
     }
   };
   auto store_tile = [&](auto set_tag, int buf) {

@@ -312,12 +312,19 @@ class MemorySparseAttention(nn.Module):
             raise ValueError("compact KV cache not found: did prefill stage 2 run?")
         kc, vc, kv_len = ck["compacked_key_cache"], ck["compacked_value_cache"], ck["kv_lengths"]
         Hq, Hkv, D = self.config.num_attention_heads, self.num_kv_heads, self.head_dim
-        if S != 1:
+        # qa_mode (:375-380): the step's attention mask decides which samples gain a key, so a sample that is
+        # masked at this step (finished, or padding of an injected block) appends nothing.  The per-sample lengths
+        # play the part of the reference's growing [B, L] mask; a masked sample's output row is zero here (the
+        # reference computes a value nobody reads).
+        masked_step = S == 1 and attention_mask is not None and bool(cache.meta.get("qa_mode", False))
+        if S != 1 or masked_step:
             valid = attention_mask == 1 if attention_mask is not None else torch.ones((B, S), dtype=torch.bool, device=q.device)
             n_new = valid.sum(dim=1)
-            n_host = cache.meta.get("q_lens_host")
+            n_host = None if masked_step else cache.meta.get("q_lens_host")
             if n_host is None or len(n_host) != B:
                 n_host = n_new.tolist()
+            if max(n_host) == 0:
+                return self.o_proj(torch.zeros((B, S, Hq * D), device=q.device, dtype=q.dtype)), None
             cu_new = F.pad(n_new.cumsum(0), (1, 0)).to(torch.int32)
             self._claim_rows(ck, max(n_host))
             ops.cache_append_rows(k[valid], v[valid], cu_new, max(n_host), kc, vc, kv_len)

@@ -14,7 +14,7 @@ from . import ops
 from .cache import CustomDynamicCache, create_cache
 from .config import MSAConfig
 from .memory_sparse_attention import MemorySparseAttention, RMSNorm, rotary_embedding
-from .prefill import query_position_ids
+from .prefill import query_position_ids, source_block_position_ids
 
 
 class MLP(nn.Module):
@@ -78,6 +78,8 @@ class MSADecoderLayer(nn.Module):
             return False
         B, S, H = hidden_states.shape
         if S != 1 or B > ops.SKINNY_MAX_ROWS or cache is None or not hidden_states.is_contiguous():
+            return False
+        if cache.meta.get("qa_mode", False):       # the step's attention mask decides who appends: generic path
             return False
         a = self.self_attn
         if cache.cache_kwargs[a.layer_idx].get("stage") != "generate" or a.q_proj.bias is not None:
@@ -235,19 +237,21 @@ class MSAForCausalLM(nn.Module):
 
 @torch.no_grad()
 def generate_interleaved(model: "MSAForCausalLM", input_ids, attention_mask, doc_ids, max_new_tokens: int, inject,
-                         top_k_docs: Optional[int] = None):
+                         top_k_docs: Optional[int] = None, require_recall_topk: bool = False):
     """Greedy decoding with Memory-Interleave rounds (the control flow of src/msa/generate.py:190-259 without the
-    tokenizer: text handling stays with the caller).  After every new token ``inject(step, tokens [B, step])`` may
-    return a list of ``B`` token-id lists; a non-empty list replaces the sample's just-generated token as the next
-    model input (the reference feeds the retrieved documents' text instead of the round-end marker), an empty one
-    lets the sample continue with its own token.  The lists are fed as one left-padded block whose positions
-    continue each sample's own, appended to the compact caches by the ragged path of the decode stage, and the
-    next token is read at the block's last position.  Returns ``(tokens [B, max_new_tokens], cache)``."""
+    tokenizer: text handling stays with the caller).  Stage 2 routes on the tokens whose ``doc_ids`` are 0.  After
+    every new token ``inject(step, tokens [B, step])`` may return a list of ``B`` token-id lists; a non-empty list
+    replaces the sample's just-generated token as the next model input (the reference feeds the retrieved
+    documents' text instead of the round-end marker), an empty one lets the sample continue with its own token.
+    The lists are fed as one left-padded block with the reference's positions (``source_block_position_ids``),
+    appended to the compact caches by the ragged path of the decode stage, and the next token is read at the
+    block's last position.  Returns ``(tokens [B, max_new_tokens], cache)``."""
     cfg = model.config
     B, S = input_ids.shape
     dev = input_ids.device
     k = cfg.msa_config.top_k_docs if top_k_docs is None else top_k_docs
     cache = create_cache()
+    cache.meta["require_recall_topk"] = require_recall_topk
     for i in range(cfg.num_hidden_layers):
         cache.record_kwargs(i, {"stage": "prefill_stage2"})
     n_valid = attention_mask.sum(dim=1).tolist()
@@ -256,8 +260,7 @@ def generate_interleaved(model: "MSAForCausalLM", input_ids, attention_mask, doc
     tok = model.lm_head(h[:, -1:]).argmax(-1)                 # [B, 1]
     for i in range(cfg.num_hidden_layers):
         cache.cache_kwargs[i]["stage"] = "generate"
-    last_pos = pos[:, -1].clone()                             # position of the last token each sample has fed
-    last_pos_bound = 3 + k + max(n_valid) - 1                 # host-side bound of the same
+    last_pos = [3 + k + n - 1 for n in n_valid]               # position of the last token each sample has fed
     attn0 = model.model.layers[0].self_attn
     rows_free = min(layer.self_attn.decode_reserve for layer in model.model.layers)
     out = [tok]
@@ -271,29 +274,48 @@ def generate_interleaved(model: "MSAForCausalLM", input_ids, attention_mask, doc
             raise RuntimeError(f"step {step} appends {widest} rows per sample but only {rows_free} of the "
                                f"decode_reserve rows are left; raise decode_reserve on the layers before stage 2")
         rows_free -= widest
-        last_pos_bound += widest
-        attn0.check_positions(last_pos_bound)
-        if blocks is None or all(len(b) == 1 for b in blocks):
+        lens = [1] * B if blocks is None else [len(b) for b in blocks]
+        attn0.check_positions(max(p + n for p, n in zip(last_pos, lens)))
+        if widest == 1:
             ids = tok if blocks is None else torch.tensor(blocks, dtype=torch.long, device=dev)
-            p = (last_pos + 1).unsqueeze(1)
+            p = torch.tensor([[x + 1] for x in last_pos], dtype=torch.long, device=dev)
             h = model.model(ids, torch.ones_like(ids), p, cache, torch.full_like(ids, -1))
-            last_pos += 1
         else:
-            width = max(len(b) for b in blocks)
-            ids = torch.zeros((B, width), dtype=torch.long)
-            mask = torch.zeros((B, width), dtype=torch.long)
-            p = torch.zeros((B, width), dtype=torch.long)
+            ids = torch.zeros((B, widest), dtype=torch.long)
+            mask = torch.zeros((B, widest), dtype=torch.long)
             for b, blk in enumerate(blocks):
-                n = len(blk)
-                ids[b, width - n:] = torch.tensor(blk)
-                mask[b, width - n:] = 1
-                first = int(last_pos[b]) + 1
-                p[b] = torch.tensor([first] * (width - n) + list(range(first, first + n)))   # padding repeats the first position
-            h = model.model(ids.to(dev), mask.to(dev), p.to(dev), cache, torch.zeros((B, width), dtype=torch.long, device=dev))
-            last_pos += torch.tensor([len(b) for b in blocks], device=dev)
+                ids[b, widest - len(blk):] = torch.tensor(blk)
+                mask[b, widest - len(blk):] = 1
+            p = torch.tensor(source_block_position_ids(last_pos, lens, widest), dtype=torch.long)
+            h = model.model(ids.to(dev), mask.to(dev), p.to(dev), cache, torch.zeros((B, widest), dtype=torch.long, device=dev))
+        last_pos = [x + n for x, n in zip(last_pos, lens)]
         tok = model.lm_head(h[:, -1:]).argmax(-1)
         out.append(tok)
     return torch.cat(out, dim=1), cache
+
+
+@torch.no_grad()
+def generate_with_hops(model: "MSAForCausalLM", input_ids, attention_mask, doc_ids, max_new_tokens: int, regenerate,
+                       inject=None, max_hops: int = 4, top_k_docs: Optional[int] = None):
+    """The multi-hop loop around generation (src/app/benchmark.py:202-212 with ``should_regenerate`` and
+    src/msa_service.py:1734-1770 ``_apply_template_regenerate``): after a generation pass,
+    ``regenerate(hop, tokens [B, T])`` may return a new batch ``(input_ids, attention_mask, doc_ids)`` — the
+    regenerated prompt, in which ``doc_ids`` marks with 0 the regions that query the memory and with -1 the rest —
+    or ``None`` to stop.  Every hop is a fresh stage-2 pass: the router scores the new prompt's marked tokens against
+    the bank, the selected documents' K / V are fetched again and a new compact cache is built.  Returns the list of
+    ``(tokens, cache)`` of all passes; the recalled documents of each pass are in its cache's ``recall_topk``."""
+    passes = []
+    batch = (input_ids, attention_mask, doc_ids)
+    for hop in range(max_hops + 1):
+        toks, cache = generate_interleaved(model, batch[0], batch[1], batch[2], max_new_tokens, inject,
+                                           top_k_docs=top_k_docs, require_recall_topk=True)
+        passes.append((toks, cache))
+        if hop == max_hops or regenerate is None:
+            break
+        batch = regenerate(hop, toks)
+        if batch is None:
+            break
+    return passes
 
 
 def encode_block(model: MSAForCausalLM, block_input, device) -> CustomDynamicCache:

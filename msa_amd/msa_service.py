@@ -124,6 +124,39 @@ class Memory:
         return self.msa_model_config.num_hidden_layers
 
     # ---------------------------------------------------------------- bank fill (:497-582)
+    def set_prefill_worker(self, worker) -> None:
+        """The stage-1 worker :meth:`generate_blocks` drives (the reference starts one per GPU as a child process,
+        :500-513; here it lives in this process and is handed in)."""
+        self._prefill_worker = worker
+
+    def generate_blocks(self, docs: List[Document], worker=None) -> None:
+        """Builds the bank from documents exactly as the reference does (:497-582): an existing dump under
+        ``$MEMORY_DATA_PATH/gpu<world>/<gpu_id>`` is loaded instead; otherwise the documents are split into blocks
+        of at most ``memory_config.block_size`` chunks, every block is encoded by the worker's ``inference`` and its
+        pooled K / V / K_r are copied into the bank at the running chunk offset, the pooled document ids are merged,
+        and the bank is dumped when the variable is set."""
+        path = os.environ.get("MEMORY_DATA_PATH", "")
+        if path:
+            path = os.path.join(path, f"gpu{self.generate_config.world}", str(self.gpu_id))
+            if os.path.exists(path):
+                self.deserialize(path, docs)
+                assert len(docs) == self.block_desc.nr_docs
+                return
+        worker = worker or getattr(self, "_prefill_worker", None)
+        if worker is None:
+            raise ValueError("generate_blocks needs a stage-1 worker (set_prefill_worker or the worker argument)")
+        self.begin(docs)
+        recv = 0
+        for block in worker.split_docs(docs, self.memory_config.block_size):
+            meta = worker.inference(block)
+            recv += meta["nr_docs"]
+            self.add_block(meta["past_key_values"])
+            meta["past_key_values"].clear_kvcache()
+        assert recv == len(docs), f"encoded {recv} of {len(docs)} documents"
+        self.finish()
+        if path:
+            self.serialize(path)
+
     def begin(self, docs: List[Document]) -> None:
         self.block_desc.init_docs(docs, self.device)
         self._kv_offset = 0

@@ -4,7 +4,7 @@ position ids restarting at 0 for every document, ceil(len / P) chunks per docume
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import List, Sequence
+from typing import Dict, List, Sequence
 
 import torch
 
@@ -79,3 +79,57 @@ def query_position_ids(n_tokens: int, top_k: int, template_len: int = 3, left_pa
     (src/msa_service.py:1823-1864)."""
     first = template_len + top_k
     return [first] * left_pad + [first + i for i in range(n_tokens)]
+
+
+def source_block_position_ids(last_positions: Sequence[int], n_tokens: Sequence[int], width: int) -> List[List[int]]:
+    """Positions of a left-padded block of source tokens injected between generation rounds
+    (src/msa/generate.py:235-236): column ``j`` of sample ``b`` gets
+    ``j + last_positions[b] + n_tokens[b] - width + 1``, so the sample's first real token (column
+    ``width - n_tokens[b]``) continues at ``last_positions[b] + 1`` and the rest count up from there.  The same
+    expression runs below that for the padding columns in front; those tokens are masked out everywhere, and their
+    positions are floored at 0 here because the rotary tables start there."""
+    out = []
+    for last, n in zip(last_positions, n_tokens):
+        out.append([max(0, j + int(last) + int(n) - width + 1) for j in range(width)])
+    return out
+
+
+class PrefillStage1Worker:
+    """The encode worker with the reference's call surface (src/prefill.py:94-305), in process: no queues, no
+    tokenizer (documents arrive tokenised), the model handed in instead of loaded from a path.
+
+    ``inference(block)`` returns what the reference's worker sends back (:300-303, :142-157):
+    ``{"chunk_sizes", "past_key_values", "nr_docs", "doc_ids", "nr_chunks"}`` with the pooled K / V / K_r of every
+    router layer in ``past_key_values`` (getters ``get_kvcache`` / ``get_router_kcache``,
+    ``cache_kwargs[layer]["pooled_doc_ids" | "template_prefix_kcache" | "template_prefix_vcache"]``)."""
+
+    def __init__(self, gpu_id: int, model, template_head_ids: Sequence[int], pooling_kernel_size: int,
+                 template_id: int = -2):
+        self.gpu_id = gpu_id
+        self.device = torch.device(f"cuda:{gpu_id}")
+        self.model = model
+        self.template_head_ids = list(template_head_ids)
+        self.pooling_kernel_size = pooling_kernel_size
+        self.template_id = template_id
+
+    def num_model_layers(self) -> int:
+        return self.model.config.num_hidden_layers
+
+    @staticmethod
+    def split_docs(docs: List[Document], block_size: int) -> List[List[Document]]:
+        return split_docs(docs, block_size)
+
+    def _prepare_block_inputs(self, block: List[Document]) -> BlockModelInput:
+        return prepare_block_inputs(block, self.template_head_ids, self.pooling_kernel_size, self.template_id)
+
+    def _inference(self, model_input: BlockModelInput) -> Dict:
+        from .model import encode_block            # the model module imports this one
+        cache = encode_block(self.model, model_input, self.device)
+        return {"chunk_sizes": model_input.chunk_sizes, "past_key_values": cache}
+
+    def inference(self, block: List[Document]) -> Dict:
+        meta = self._inference(self._prepare_block_inputs(block))
+        meta["nr_docs"] = len(block)
+        meta["doc_ids"] = [item.doc_id for item in block]
+        meta["nr_chunks"] = [item.num_chunks for item in block]
+        return meta

@@ -411,3 +411,233 @@ def test_decoder_layer_glue_matches_plain_torch(env, dtype):
             act = torch.nn.functional.silu(normed @ w["mlp.gate_proj.weight"].T) * (normed @ w["mlp.up_proj.weight"].T)
             want = hd + act @ w["mlp.down_proj.weight"].T
         assert cf.rel_err(got.cpu(), want) < 2e-2
+
+
+def _layer_bank(env, layer, layer64, lens, g):
+    """Stage 1 of a single router layer over `lens` documents, fed to a service block by block; returns the service
+    and the fp64 oracle's pooled bank, template prefix and document table."""
+    pf, svc_mod = env["prefill"], env["svc"]
+    docs = _docs(env, lens)
+    service = svc_mod.MSAService(0, env["config"].GenerateConfig(devices=[0]),
+                                 env["config"].ModelConfig(doc_top_k=TOPK, pooling_kernel_size=P, router_layer_idx="1"),
+                                 env["config"].MemoryConfig(pooling_kernel_size=P), env["cfg"])
+    service.begin(docs)
+    bank_k, bank_v, bank_rk, prefix = [], [], [], None
+    for blk in pf.split_docs(docs, 8):
+        inp = pf.prepare_block_inputs(blk, HEAD_IDS, P)
+        T = inp.doc_ids.shape[1]
+        hs = torch.randn((1, T, HID), generator=g)
+        cos, sin = _tables(env, inp.position_ids)
+        cache = env["model"].create_cache()
+        cache.record_kwargs(1, {"stage": "prefill_stage1"})
+        with torch.no_grad():
+            layer(hs.cuda(), inp.doc_ids.cuda(), inp.doc_attention_mask.cuda(), (cos.cuda(), sin.cuda()), cache)
+            _, k64, v64 = layer64._project(hs.double(), (cos.double(), sin.double()))
+            rk64 = layer64.router_k_proj(hs.double()).view(T, HKV, D)
+        _, _, cs, cl, _ = cf.chunk_table(inp.doc_lens, P, 3)
+        bank_k.append(cf.pool_chunks(k64[0], cs, cl))
+        bank_v.append(cf.pool_chunks(v64[0], cs, cl))
+        bank_rk.append(cf.l2_normalize(cf.pool_chunks(rk64, cs, cl)))
+        if prefix is None:
+            prefix = (k64[0, :3], v64[0, :3])
+        service.add_block(cache)
+    service.finish()
+    _, dco, _, _, _ = cf.chunk_table(lens, P)
+    return service, torch.cat(bank_k), torch.cat(bank_v), torch.cat(bank_rk), prefix, dco
+
+
+def _stage2_with_oracle(env, layer, layer64, bank, hs2, mask, doc_ids, n_q):
+    """Stage 2 of the layer on a left-padded batch; returns the cache and, per sample, the oracle's context rows
+    ``(K, V)`` = [prefix | selected chunks | the sample's own tokens] built from the documents the layer recalled
+    (which are checked against the oracle's scores of the tokens marked 0 in ``doc_ids``)."""
+    pf = env["prefill"]
+    bank_k, bank_v, bank_rk, prefix, dco = bank
+    B, S = mask.shape
+    pos = torch.tensor([pf.query_position_ids(n, TOPK, 3, S - n) for n in n_q])
+    cos, sin = _tables(env, pos)
+    cache = env["model"].create_cache()
+    cache.meta["require_recall_topk"] = True
+    cache.record_kwargs(1, {"stage": "prefill_stage2"})
+    with torch.no_grad():
+        out, _ = layer(hs2.cuda(), doc_ids.cuda(), mask.cuda(), (cos.cuda(), sin.cuda()), cache)
+        q64, k64, v64 = layer64._project(hs2.double(), (cos.double(), sin.double()))
+        rq64 = layer64.router_q_proj(hs2.double()).view(B, S, HQ, D)
+    scored = (doc_ids == 0) & mask.bool()                       # only the marked tokens query the memory
+    ds = cf.doc_scores(cf.chunk_scores(rq64, scored, bank_rk, "cosine"), dco)
+    got_i = torch.tensor([[d - 100 for d in r["topk_doc_ids"]] for r in cache.cache_kwargs[1]["recall_topk"]])
+    assert not cf.topk_acceptable(ds, got_i, TOPK, gap=1e-4)
+    mk, mv, cu_sel, _ = cf.gather_selected(bank_k, bank_v, dco, got_i)
+    ctx = []
+    for b in range(B):
+        lo = S - n_q[b]
+        kk = torch.cat([prefix[0], mk[cu_sel[b]:cu_sel[b + 1]], k64[b, lo:]])
+        vv = torch.cat([prefix[1], mv[cu_sel[b]:cu_sel[b + 1]], v64[b, lo:]])
+        want = cf.attention(q64[b, lo:], kk, vv, causal=True)
+        with torch.no_grad():
+            assert cf.rel_err(out[b:b + 1, lo:].cpu(), layer64.o_proj(want.reshape(1, n_q[b], HQ * D))) < TOL
+        ctx.append((kk, vv))
+    return cache, ctx, pos, ds, got_i
+
+
+def test_injected_block_rerouted_hop_and_masked_step_against_oracle(env):
+    """The Memory-Interleave pieces against the fp64 oracle on one router layer (fp32): a ragged left-padded block of
+    source tokens injected in the decode stage at the reference's positions (src/msa/generate.py:235-236) attends
+    over the explicit [stage-2 context | block so far] keys and lands in the compact cache; the decode step after it
+    sees all of it; a step whose attention mask is 0 for a sample (qa_mode, src/msa/memory_sparse_attention.py:
+    375-380) gives that sample no new key; and a second hop routes again with only the tokens its regenerated prompt
+    marks with 0 (src/msa_service.py:1734-1770)."""
+    say("layer: injected block, masked step and re-routed hop against the oracle")
+    pf = env["prefill"]
+    layer = _layer(env, seed=2)
+    layer64 = copy.deepcopy(layer).double()
+    layer = layer.cuda()
+    g = torch.Generator().manual_seed(13)
+    lens = [5, 8, 17, 1, 30, 9, 16, 23, 12, 7, 40]
+    service, bank_k, bank_v, bank_rk, prefix, dco = _layer_bank(env, layer, layer64, lens, g)
+    bank = (bank_k, bank_v, bank_rk, prefix, dco)
+    layer.set_memory_client(service)
+    n_q = [7, 4]
+    B, S = 2, 7
+    mask = torch.tensor([[1] * 7, [0] * 3 + [1] * 4])
+    hs2 = torch.randn((B, S, HID), generator=g)
+    cache, ctx, pos, ds1, sel1 = _stage2_with_oracle(env, layer, layer64, bank, hs2, mask, torch.zeros((B, S), dtype=torch.long), n_q)
+    cache.cache_kwargs[1]["stage"] = "generate"
+    len0 = cache.cache_kwargs[1]["kv_lengths"].cpu().tolist()
+
+    # ---- the injected block: 5 and 2 source tokens, left-padded to 5 columns
+    n_new, W = [5, 2], 5
+    last_pos = pos[:, -1].tolist()
+    p_blk = torch.tensor(pf.source_block_position_ids(last_pos, n_new, W))
+    m_blk = torch.tensor([[1] * 5, [0, 0, 0, 1, 1]])
+    # the reference's arithmetic, on the columns that hold tokens
+    ref_pos = torch.arange(W).unsqueeze(0).expand(B, -1) + pos[:, -1:] + m_blk.sum(dim=1, keepdim=True) - W + 1
+    assert torch.equal(p_blk[m_blk.bool()], ref_pos[m_blk.bool()])
+    assert p_blk[0].tolist() == [last_pos[0] + 1 + i for i in range(5)] and p_blk[1, 3:].tolist() == [last_pos[1] + 1, last_pos[1] + 2]
+    hs_blk = torch.randn((B, W, HID), generator=g)
+    cos, sin = _tables(env, p_blk)
+    with torch.no_grad():
+        out_blk, _ = layer(hs_blk.cuda(), torch.zeros((B, W), dtype=torch.long).cuda(), m_blk.cuda(),
+                           (cos.cuda(), sin.cuda()), cache)
+        q64, k64, v64 = layer64._project(hs_blk.double(), (cos.double(), sin.double()))
+    kw = cache.cache_kwargs[1]
+    assert kw["kv_lengths"].cpu().tolist() == [len0[b] + n_new[b] for b in range(B)]
+    for b in range(B):
+        lo = W - n_new[b]
+        ctx[b] = (torch.cat([ctx[b][0], k64[b, lo:]]), torch.cat([ctx[b][1], v64[b, lo:]]))
+        want = cf.attention(q64[b, lo:], ctx[b][0], ctx[b][1], causal=True)        # row i sees the block up to i
+        with torch.no_grad():
+            assert cf.rel_err(out_blk[b:b + 1, lo:].cpu(), layer64.o_proj(want.reshape(1, n_new[b], HQ * D))) < TOL
+        assert float(out_blk[b, :lo].abs().max()) == 0.0 if lo else True
+        L = len0[b] + n_new[b]
+        assert cf.rel_err(kw["compacked_key_cache"][b, :L].cpu(), ctx[b][0]) < TOL       # the whole context, row for row
+        assert cf.rel_err(kw["compacked_value_cache"][b, :L].cpu(), ctx[b][1]) < TOL
+
+    # ---- the decode step behind the block sees [context | block | itself]
+    last_pos = [last_pos[b] + n_new[b] for b in range(B)]
+    hs3 = torch.randn((B, 1, HID), generator=g)
+    pos3 = torch.tensor([[x + 1] for x in last_pos])
+    cos, sin = _tables(env, pos3)
+    with torch.no_grad():
+        out3, _ = layer(hs3.cuda(), torch.full((B, 1), -1).cuda(), torch.ones(B, 1, dtype=torch.long).cuda(),
+                        (cos.cuda(), sin.cuda()), cache)
+        q64, k64, v64 = layer64._project(hs3.double(), (cos.double(), sin.double()))
+        for b in range(B):
+            ctx[b] = (torch.cat([ctx[b][0], k64[b]]), torch.cat([ctx[b][1], v64[b]]))
+            want = layer64.o_proj(cf.attention(q64[b], ctx[b][0], ctx[b][1]).reshape(1, 1, HQ * D))
+            assert cf.rel_err(out3[b:b + 1].cpu(), want) < TOL
+
+    # ---- qa_mode: a step whose mask is 0 for sample 1 appends nothing for it
+    cache.meta["qa_mode"] = True
+    before = kw["kv_lengths"].cpu().tolist()
+    hs4 = torch.randn((B, 1, HID), generator=g)
+    pos4 = pos3 + 1
+    cos, sin = _tables(env, pos4)
+    with torch.no_grad():
+        out4, _ = layer(hs4.cuda(), torch.full((B, 1), -1).cuda(), torch.tensor([[1], [0]]).cuda(),
+                        (cos.cuda(), sin.cuda()), cache)
+        q64, k64, v64 = layer64._project(hs4.double(), (cos.double(), sin.double()))
+        want = layer64.o_proj(cf.attention(q64[0], torch.cat([ctx[0][0], k64[0]]), torch.cat([ctx[0][1], v64[0]])).reshape(1, 1, HQ * D))
+    assert kw["kv_lengths"].cpu().tolist() == [before[0] + 1, before[1]]
+    assert cf.rel_err(out4[0:1].cpu(), want) < TOL and float(out4[1].abs().max()) == 0.0
+
+    # ---- second hop: a regenerated prompt routes again, with the tokens it marks 0 only
+    n_q2 = [6, 9]
+    S2 = 9
+    mask2 = torch.tensor([[0] * 3 + [1] * 6, [1] * 9])
+    doc2 = torch.tensor([[-1, -1, -1, 0, 0, -1, -1, 0, -1], [0, 0, 0, -1, -1, -1, -1, -1, 0]])
+    hs5 = torch.randn((B, S2, HID), generator=g)
+    cache2, _, _, ds2, sel2 = _stage2_with_oracle(env, layer, layer64, bank, hs5, mask2, doc2, n_q2)
+    # had every token been scored the documents' scores would differ: the mask reached the router
+    with torch.no_grad():
+        rq_all = layer64.router_q_proj(hs5.double()).view(B, S2, HQ, D)
+    ds_all = cf.doc_scores(cf.chunk_scores(rq_all, mask2.bool(), bank_rk, "cosine"), dco)
+    assert float((ds_all - ds2).abs().max()) > 1e-3
+    assert cache2 is not cache and "compacked_key_cache" in cache2.cache_kwargs[1]    # a new, independent compact cache
+
+
+def test_generate_blocks_worker_surface_and_hop_loop(env, tmp_path, monkeypatch):
+    """``Memory.generate_blocks(docs)`` with a stage-1 worker (src/msa_service.py:497-582, src/prefill.py:142-157,
+    300-303) builds the same bank, bit for bit, as feeding the blocks by hand; with MEMORY_DATA_PATH it dumps the
+    bank and a second service loads the dump instead of encoding.  Then the hop loop: every hop is a fresh stage-2
+    pass over the regenerated prompt."""
+    say("model: generate_blocks through the worker, stored bank, hop loop")
+    pf, svc_mod, M = env["prefill"], env["svc"], env["model"]
+    model = M.MSAForCausalLM(env["cfg"]).init_random(0.05, seed=7).to(torch.bfloat16).cuda().eval()
+    docs = _docs(env, [20, 33, 9, 41, 16, 27, 11], first_id=0)
+
+    def new_service():
+        return svc_mod.MSAService(0, env["config"].GenerateConfig(devices=[0]),
+                                  env["config"].ModelConfig(doc_top_k=TOPK, pooling_kernel_size=P, router_layer_idx="1"),
+                                  env["config"].MemoryConfig(block_size=12, pooling_kernel_size=P), env["cfg"])
+    by_hand = new_service()
+    by_hand.begin(docs)
+    for blk in pf.split_docs(docs, 12):
+        by_hand.add_block(M.encode_block(model, pf.prepare_block_inputs(blk, HEAD_IDS, P), "cuda"))
+    by_hand.finish()
+
+    worker = pf.PrefillStage1Worker(0, model, HEAD_IDS, P)
+    meta = worker.inference(pf.split_docs(docs, 12)[0])
+    assert set(meta) == {"chunk_sizes", "past_key_values", "nr_docs", "doc_ids", "nr_chunks"}
+    first = pf.split_docs(docs, 12)[0]
+    assert meta["nr_docs"] == len(first) and meta["doc_ids"] == [d.doc_id for d in first]
+    assert meta["nr_chunks"] == [d.num_chunks for d in first] == meta["chunk_sizes"]
+    pkv = meta["past_key_values"]
+    assert pkv.get_kvcache(1)[0].shape == (1, HKV, sum(meta["chunk_sizes"]), D) and pkv.get_router_kcache(1) is not None
+    assert {"pooled_doc_ids", "template_prefix_kcache", "template_prefix_vcache"} <= set(pkv.cache_kwargs[1])
+
+    monkeypatch.setenv("MEMORY_DATA_PATH", str(tmp_path))
+    built = new_service()
+    built.generate_blocks(docs, worker)
+    for a, b in ((by_hand._rk[1], built._rk[1]), (by_hand._k[1], built._k[1]), (by_hand._v[1], built._v[1])):
+        assert torch.equal(a.cpu(), b.cpu())
+    assert torch.equal(by_hand.block_desc.pool_ids_cpu, built.block_desc.pool_ids_cpu)
+    assert torch.equal(by_hand.block_desc.doc_offsets_cpu, built.block_desc.doc_offsets_cpu)
+    assert (tmp_path / "gpu1" / "0").exists()
+    loaded = new_service()
+    loaded.generate_blocks(docs)                               # no worker: the dump is there
+    assert torch.equal(loaded._rk[1].cpu(), built._rk[1].cpu()) and torch.equal(loaded._k[1], built._k[1])
+    monkeypatch.delenv("MEMORY_DATA_PATH")
+    with pytest.raises(ValueError, match="stage-1 worker"):
+        new_service().generate_blocks(docs)
+
+    # ---- hop loop on the loaded bank
+    loaded.setup_memory_client(model)
+    ids = torch.tensor([[5, 6, 7, 8, 9, 10], [0, 0, 11, 12, 13, 14]]).cuda()
+    mask = torch.tensor([[1] * 6, [0, 0, 1, 1, 1, 1]]).cuda()
+    ids2 = torch.tensor([[41, 42, 43, 44, 45, 46, 47, 48], [0, 0, 0, 51, 52, 53, 54, 55]]).cuda()
+    mask2 = torch.tensor([[1] * 8, [0, 0, 0, 1, 1, 1, 1, 1]]).cuda()
+    doc2 = torch.tensor([[0, 0, -1, -1, -1, 0, -1, -1], [0, 0, 0, -1, 0, 0, -1, -1]]).cuda()
+    seen = []
+
+    def regenerate(hop, toks):
+        seen.append((hop, tuple(toks.shape)))
+        return (ids2, mask2, doc2) if hop == 0 else None
+
+    passes = M.generate_with_hops(model, ids, mask, torch.zeros_like(ids), 4, regenerate)
+    assert len(passes) == 2 and seen == [(0, (2, 4)), (1, (2, 4))]
+    (t1, c1), (t2, c2) = passes
+    direct, cd = M.generate_interleaved(model, ids2, mask2, doc2, 4, None, require_recall_topk=True)
+    assert torch.equal(t2, direct)                             # hop 2 is a complete pass of its own over the new prompt
+    r2, rd = c2.cache_kwargs[1]["recall_topk"], cd.cache_kwargs[1]["recall_topk"]
+    assert [r["topk_doc_ids"] for r in r2] == [r["topk_doc_ids"] for r in rd]
+    assert c2 is not c1 and t1.shape == t2.shape == (2, 4)

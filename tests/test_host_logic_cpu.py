@@ -126,3 +126,32 @@ def test_bank_files_round_trip(tmp_path):
     os.remove(f"{path}/bank.json")
     with pytest.raises(FileNotFoundError):
         bank_io.BankFiles(path)
+
+
+def test_source_block_positions_follow_the_reference_formula():
+    """src/msa/generate.py:235-236: arange(W) + position_ids + sum(attention_mask) - W + 1 on the columns that hold
+    tokens; the padding columns in front are floored at 0."""
+    import torch
+    from msa_amd import prefill as pf
+    last = [25, 40, 3]
+    n = [5, 2, 1]
+    W = 5
+    got = torch.tensor(pf.source_block_position_ids(last, n, W))
+    mask = torch.tensor([[1] * 5, [0, 0, 0, 1, 1], [0, 0, 0, 0, 1]])
+    ref = torch.arange(W).unsqueeze(0).expand(3, -1) + torch.tensor(last).unsqueeze(1) + mask.sum(dim=1, keepdim=True) - W + 1
+    assert torch.equal(got[mask.bool()], ref[mask.bool()])
+    assert got[0].tolist() == [26, 27, 28, 29, 30] and got[1].tolist()[3:] == [41, 42] and got[2, 4] == 4
+    assert (got >= 0).all() and got[2].tolist() == [0, 1, 2, 3, 4]
+    assert torch.equal(got[1, :3], ref[1, :3])                     # in front of real tokens the same expression runs on
+
+
+def test_prefill_worker_block_inputs_and_split():
+    from msa_amd import prefill as pf
+    docs = [pf.Document(doc_id=10 + i, num_chunks=pf.num_chunks(n, 8), input_ids=list(range(1, n + 1))) for i, n in enumerate([9, 16, 3, 30])]
+    w = pf.PrefillStage1Worker(0, None, [7, 8, 9], 8)
+    blocks = w.split_docs(docs, 5)
+    assert [[d.doc_id for d in b] for b in blocks] == [[10, 11, 12], [13]]      # 2 + 2 + 1 chunks fill a block of 5
+    inp = w._prepare_block_inputs(blocks[0])
+    assert inp.doc_ids[0, :3].tolist() == [-2, -2, -2] and inp.doc_ids[0, 3:12].tolist() == [1] * 9
+    assert inp.position_ids[0, 3:12].tolist() == list(range(9)) and inp.position_ids[0, 12] == 0
+    assert inp.chunk_sizes == [2, 2, 1]

@@ -225,6 +225,19 @@ int msa_qk_norm_rope(const void* q, const void* k, const void* v, int64_t q_row_
                      const void* q_norm_w, const void* k_norm_w, float eps, const float* rope_cos,
                      const float* rope_sin, int32_t rope_rows, int32_t dtype, int64_t N, int32_t Hq,
                      int32_t Hkv, int32_t D, void* q_out, void* k_out, void* v_out, void* stream);
+/* Fused projection of a block of tokens (the encode path of stage 1 and the query prefill of stage 2): one bf16 GEMM
+ * x[T, K] . w[N, K]^T over the concatenated weights of q_proj / k_proj / v_proj and, on router layers, router_k_proj
+ * or router_q_proj (src/msa/memory_sparse_attention.py:125-127, 178, 263), with q_norm / k_norm and
+ * apply_rotary_pos_emb (:129-133) applied to the q and k heads in the GEMM's epilogue, exactly as msa_qk_norm_rope
+ * would to the bf16 projection output.  Rows of w, 128 per head: Hr_front router heads | Hq q heads | Hkv k heads |
+ * Hkv v heads | Hr_back router heads (so one [rk | q | k | v | rq] matrix serves stage 1 with Hr_front = Hkv, stage 2
+ * with a pointer 1024 rows in and Hr_back = Hq, and the decode step's q | k | v slice).  K a multiple of 64.
+ * Outputs are dense: q_out [T, Hq, 128], k_out / v_out [T, Hkv, 128], r_out [T, Hr_front + Hr_back, 128]
+ * (router heads are stored as projected: no norm, no rotary). */
+int msa_qkv_proj(const void* x, int64_t T, int32_t K, const void* w, int32_t Hq, int32_t Hkv, int32_t Hr_front,
+                 int32_t Hr_back, const int64_t* positions, const void* q_norm_w, const void* k_norm_w, float eps,
+                 const float* rope_cos, const float* rope_sin, int32_t rope_rows, void* q_out, void* k_out,
+                 void* v_out, void* r_out, void* stream);
 /* msa_qk_norm_rope for a decode step (one new token per sample, N = B) fused with msa_cache_append: the
  * normalised, rotated k row and the v row of sample b are written to kcache / vcache [b][kv_len[b]] and
  * kv_len[b] is incremented (src/msa/memory_sparse_attention.py:129-133 followed by the cache update at

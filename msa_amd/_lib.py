@@ -46,6 +46,8 @@ SIGNATURES = {
     "msa_flash_attn": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _vp]),
     "msa_qk_norm_rope": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _f32, _vp, _vp, _i32, _i32, _i64, _i32,
                                    _i32, _i32, _vp, _vp, _vp, _vp]),
+    "msa_qkv_proj": (C.c_int, [_vp, _i64, _i32, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _f32, _vp, _vp, _i32, _vp, _vp, _vp,
+                               _vp, _vp]),
     "msa_qk_norm_rope_append": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _f32, _vp, _vp, _i32, _i32, _i32,
                                           _i32, _i32, _i32, _vp, _vp, _vp, _i32, _vp, _vp]),
     "msa_rmsnorm": (C.c_int, [_vp, _vp, _vp, _i32, _i64, _i32, _f32, _vp, _vp]),

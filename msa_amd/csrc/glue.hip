@@ -7,17 +7,6 @@
 
 namespace {
 
-__device__ __forceinline__ float row16_sum(float v) {   // all-reduce over the 16 lanes of a DPP row
-  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x124, 0xf, 0xf, false));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x122, 0xf, 0xf, false));
-  v += __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x121, 0xf, 0xf, false));
-  return v;
-}
-__device__ __forceinline__ float row16_ror8(float v) {  // value of the lane 8 places away in the row
-  return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
-}
-
 template <typename T>
 __device__ __forceinline__ void load8g(const T* p, float (&x)[8]) {
   if constexpr (sizeof(T) == 2) {

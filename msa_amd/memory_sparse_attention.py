@@ -114,21 +114,57 @@ class MemorySparseAttention(nn.Module):
         cos, sin = position_embeddings
         return apply_rotary_bshd(q, cos, sin).contiguous(), apply_rotary_bshd(k, cos, sin).contiguous(), v.contiguous()
 
-    def _project_fused(self, hidden_states, position_ids):
-        """Same result as :meth:`_project` from integer positions: one GEMM over the concatenated q / k / v
-        weights, then per-head RMSNorm + rotary (+ the dense copy of V) in one HIP kernel."""
+    def _project_fused(self, hidden_states, position_ids, router: Optional[str] = None):
+        """Same result as :meth:`_project` from integer positions, plus the router projection the stage needs
+        (``router`` = "k": router_k_proj, "q": router_q_proj): ``(q, k, v, r)`` with ``r`` ``None`` when not asked for.
+        bf16: one native GEMM over the concatenated weights with the per-head RMSNorm + rotary in its epilogue
+        (``ops.qkv_proj``); fp32: one GEMM over q / k / v, the norm + rotary kernel, and the router module."""
         B, S, _ = hidden_states.shape
         Hq, Hkv, D = self.config.num_attention_heads, self.num_kv_heads, self.head_dim
-        w_qkv, tables = self._fused_weight(hidden_states.device), self._rope_tables(hidden_states.device)
-        qkv = F.linear(hidden_states.reshape(B * S, -1), w_qkv)
-        q, k, v = ops.qk_norm_rope(qkv, Hq, Hkv, D, position_ids.reshape(-1).contiguous(), self.q_norm.weight,
-                                   self.k_norm.weight, self.q_norm.variance_epsilon, tables)
-        return q.view(B, S, Hq, D), k.view(B, S, Hkv, D), v.view(B, S, Hkv, D)
+        tables = self._rope_tables(hidden_states.device)
+        x = hidden_states.reshape(B * S, -1)
+        pos = position_ids.reshape(-1).contiguous()
+        has_router = self.is_router_layer and self.decouple_router
+        if hidden_states.dtype == torch.bfloat16 and D == 128 and x.shape[1] % 64 == 0:
+            w_all = self._all_weight(hidden_states.device)
+            lo = Hkv * D if has_router else 0                   # rows of router_k_proj in front of q | k | v
+            if has_router and router == "k":
+                q, k, v, r = ops.qkv_proj(x.contiguous(), w_all[:lo + (Hq + 2 * Hkv) * D], Hq, Hkv, pos, self.q_norm.weight,
+                                          self.k_norm.weight, self.q_norm.variance_epsilon, tables, router_front=Hkv)
+            elif has_router and router == "q":
+                q, k, v, r = ops.qkv_proj(x.contiguous(), w_all[lo:], Hq, Hkv, pos, self.q_norm.weight, self.k_norm.weight,
+                                          self.q_norm.variance_epsilon, tables, router_back=Hq)
+            else:
+                q, k, v, r = ops.qkv_proj(x.contiguous(), w_all[lo:lo + (Hq + 2 * Hkv) * D], Hq, Hkv, pos, self.q_norm.weight,
+                                          self.k_norm.weight, self.q_norm.variance_epsilon, tables)
+            r = None if r is None else r.view(B, S, -1, D)
+            return q.view(B, S, Hq, D), k.view(B, S, Hkv, D), v.view(B, S, Hkv, D), r
+        qkv = F.linear(x, self._fused_weight(hidden_states.device))
+        q, k, v = ops.qk_norm_rope(qkv, Hq, Hkv, D, pos, self.q_norm.weight, self.k_norm.weight,
+                                   self.q_norm.variance_epsilon, tables)
+        r = None
+        if has_router and router == "k":
+            r = self.router_k_proj(hidden_states).view(B, S, Hkv, D)
+        elif has_router and router == "q":
+            r = self.router_q_proj(hidden_states).view(B, S, Hq, D)
+        return q.view(B, S, Hq, D), k.view(B, S, Hkv, D), v.view(B, S, Hkv, D), r
+
+    def _all_weight(self, device):
+        """[router_k_proj | q_proj | k_proj | v_proj | router_q_proj] rows in one matrix (q | k | v alone on layers
+        without a decoupled router): stage 1 multiplies by the first four, stage 2 by the last four, a decode step by
+        the middle three, all as contiguous row ranges of this one copy."""
+        if self._qkv_weight is None or self._qkv_weight.device != device:
+            parts = [self.q_proj.weight, self.k_proj.weight, self.v_proj.weight]
+            if self.is_router_layer and self.decouple_router:
+                parts = [self.router_k_proj[0].weight] + parts + [self.router_q_proj[0].weight]
+            self._qkv_weight = torch.cat(parts, dim=0).contiguous()
+        return self._qkv_weight
 
     def _fused_weight(self, device):
-        if self._qkv_weight is None or self._qkv_weight.device != device:
-            self._qkv_weight = torch.cat([self.q_proj.weight, self.k_proj.weight, self.v_proj.weight], dim=0).contiguous()
-        return self._qkv_weight
+        w = self._all_weight(device)
+        Hq, Hkv, D = self.config.num_attention_heads, self.num_kv_heads, self.head_dim
+        lo = Hkv * D if (self.is_router_layer and self.decouple_router) else 0
+        return w[lo:lo + (Hq + 2 * Hkv) * D]
 
     def _rope_tables(self, device):
         # one row per position the configuration allows; positions beyond it are refused where they are made
@@ -186,18 +222,20 @@ class MemorySparseAttention(nn.Module):
                                                  position_embeddings=None, past_key_value=None, position_ids=None,
                                                  **kwargs):
         stage = past_key_value.cache_kwargs[self.layer_idx]["stage"]
+        r = None
         if position_ids is not None and hidden_states.is_cuda and self.q_proj.bias is None:
-            q, k, v = self._project_fused(hidden_states, position_ids)       # [B, S, H, D] token-major
+            router = {"prefill_stage1": "k", "prefill_stage2": "q"}.get(stage)
+            q, k, v, r = self._project_fused(hidden_states, position_ids, router)   # [B, S, H, D] token-major
         else:
             q, k, v = self._project(hidden_states, position_embeddings)
         if stage == "prefill_stage1":
-            return self._stage1(hidden_states, doc_ids, attention_mask, q, k, v, past_key_value)
+            return self._stage1(hidden_states, doc_ids, attention_mask, q, k, v, past_key_value, r)
         if stage == "prefill_stage2":
-            return self._stage2(hidden_states, doc_ids, attention_mask, q, k, v, past_key_value)
+            return self._stage2(hidden_states, doc_ids, attention_mask, q, k, v, past_key_value, r)
         return self._generate(hidden_states, q, k, v, past_key_value, attention_mask)
 
     # ------------------------------------------------------------------------------------------ stage 1
-    def _stage1(self, hidden_states, doc_ids, attention_mask, q, k, v, cache):
+    def _stage1(self, hidden_states, doc_ids, attention_mask, q, k, v, cache, router_k=None):
         """Encodes one packed block ``[template | doc 1 | doc 2 | ...]``: document-wise causal
         attention, and on router layers chunk-mean pooling of K (rotated), V and K_r
         (src/msa/memory_sparse_attention.py:137-243)."""
@@ -215,7 +253,12 @@ class MemorySparseAttention(nn.Module):
                   "template_prefix_vcache": v[:, :n_template].transpose(1, 2)}
         if self.is_router_layer:
             table = ops.chunk_table(doc_lens, P, first_token=n_template, device=hidden_states.device)
-            rk = self.router_k_proj(hidden_states).view(T, Hkv, D).contiguous() if self.decouple_router else None
+            if not self.decouple_router:
+                rk = None
+            elif router_k is not None:                       # came out of the fused projection
+                rk = router_k.reshape(T, Hkv, D)
+            else:
+                rk = self.router_k_proj(hidden_states).view(T, Hkv, D).contiguous()
             normalize = self.aux_loss_method == "INFONCE"
             pk, pv, prk = ops.pool_chunks(k[0], v[0], rk if rk is not None else k[0], table, normalize_kr=normalize)
             cache.update(pk.transpose(0, 1).unsqueeze(0), pv.transpose(0, 1).unsqueeze(0), self.layer_idx)
@@ -234,7 +277,7 @@ class MemorySparseAttention(nn.Module):
         return self.o_proj(out.view(1, T, Hq * D)), None
 
     # ------------------------------------------------------------------------------------------ stage 2
-    def _stage2(self, hidden_states, doc_ids, attention_mask, q, k, v, cache):
+    def _stage2(self, hidden_states, doc_ids, attention_mask, q, k, v, cache, router_q=None):
         """Routes the query batch, pulls the winners' pooled K / V, lays out
         ``[template prefix | selected chunks | query tokens]`` per sample and attends causally
         (src/msa/memory_sparse_attention.py:245-359)."""
@@ -261,7 +304,12 @@ class MemorySparseAttention(nn.Module):
         mem_k = mem_v = cu_sel = None
         max_sel = 0
         if self.is_router_layer:
-            rq = self.router_q_proj(hidden_states).view(B, S, Hq, D) if self.decouple_router else q
+            if not self.decouple_router:
+                rq = q
+            elif router_q is not None:                       # came out of the fused projection
+                rq = router_q
+            else:
+                rq = self.router_q_proj(hidden_states).view(B, S, Hq, D)
             query_mask = (doc_ids == 0) & valid
             fused = self.aux_loss_method == "INFONCE"
             if hasattr(self.memory_client, "doc_query_device"):

@@ -341,6 +341,31 @@ def qk_norm_rope(qkv: torch.Tensor, Hq: int, Hkv: int, D: int, positions: torch.
     return q, k, v
 
 
+def qkv_proj(x: torch.Tensor, w: torch.Tensor, Hq: int, Hkv: int, positions: torch.Tensor, q_norm_w, k_norm_w, eps: float,
+             rope: Tuple[torch.Tensor, torch.Tensor], router_front: int = 0, router_back: int = 0):
+    """Fused projection of ``x [T, K]`` (bf16) through ``w [(router_front + Hq + 2 Hkv + router_back) * 128, K]``:
+    returns ``q [T, Hq, 128]`` and ``k [T, Hkv, 128]`` (per-head RMSNorm + rotary at ``positions [T]`` done in the
+    GEMM's epilogue), ``v [T, Hkv, 128]`` and the router heads ``r [T, router_front + router_back, 128]`` (``None``
+    without router heads), all dense."""
+    _need_cuda(x, w, positions, q_norm_w, k_norm_w, rope[0], rope[1])
+    T, K = x.shape
+    D = 128
+    heads = router_front + Hq + 2 * Hkv + router_back
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or tuple(w.shape) != (heads * D, K):
+        raise ValueError(f"qkv_proj: x [T, K] and w [{heads * D}, K] in bf16")
+    if positions.dtype != torch.int64 or positions.numel() != T:
+        raise ValueError("qkv_proj: positions int64 [T]")
+    dev = x.device
+    q = torch.empty((T, Hq, D), dtype=x.dtype, device=dev)
+    k = torch.empty((T, Hkv, D), dtype=x.dtype, device=dev)
+    v = torch.empty((T, Hkv, D), dtype=x.dtype, device=dev)
+    r = torch.empty((T, router_front + router_back, D), dtype=x.dtype, device=dev) if router_front + router_back else None
+    check(_lib.load().msa_qkv_proj(ptr(x), T, K, ptr(w), Hq, Hkv, router_front, router_back, ptr(positions), ptr(q_norm_w),
+                                   ptr(k_norm_w), eps, ptr(rope[0]), ptr(rope[1]), rope[0].shape[0], ptr(q), ptr(k), ptr(v),
+                                   ptr(r), _stream()), "msa_qkv_proj")
+    return q, k, v, r
+
+
 def qk_norm_rope_append(qkv: torch.Tensor, Hq: int, Hkv: int, D: int, positions: torch.Tensor, q_norm_w, k_norm_w,
                         eps: float, rope: Tuple[torch.Tensor, torch.Tensor], kcache: torch.Tensor, vcache: torch.Tensor,
                         kv_len: torch.Tensor) -> torch.Tensor:

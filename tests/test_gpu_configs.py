@@ -186,7 +186,11 @@ def test_config4_end_to_end_qwen3_4b_shape(ops):
     layer_idx = svc.router_layer_ids[0]                     # 18: the first routed layer
     attn = model.model.layers[layer_idx].self_attn
     grabbed = {}
-    hook = attn.router_q_proj.register_forward_hook(lambda m, a, out: grabbed.setdefault("rq", out.detach().clone()))
+    # the layer's input at stage 2 (its router projection runs inside the fused projection kernel; the oracle side
+    # projects the same hidden states with the router weights below)
+    def grab(module, args):                                  # a pre-hook that returns something replaces the inputs
+        grabbed.setdefault("h", args[0].detach().clone())
+    hook = attn.register_forward_pre_hook(grab)
     tok_eager, cache = model.generate_greedy(ids, mask, doc_ids, steps, require_recall_topk=True, use_graph=False)
     hook.remove()
     tok_graph, cache_g = model.generate_greedy(ids, mask, doc_ids, steps, use_graph=True)
@@ -198,7 +202,8 @@ def test_config4_end_to_end_qwen3_4b_shape(ops):
     assert kv_len == cache_g.cache_kwargs[layer_idx]["kv_lengths"].cpu().tolist()
 
     # ---- routing of the first routed layer against the oracle on sampled documents
-    rq = grabbed["rq"].view(B, S, HQ, D)
+    assert grabbed["h"].shape == (B, S, cfg.hidden_size)
+    rq = torch.nn.functional.linear(grabbed["h"], attn.router_q_proj[0].weight).view(B, S, HQ, D)
     rec = ck["recall_topk"]
     rng = np.random.default_rng(9)
     slot = svc._layer_slot[layer_idx]

@@ -418,6 +418,55 @@ def test_config1_routing_layer_fp32(ops):
     assert cf.rel_err(out.cpu(), want) < 1e-5
 
 
+# ------------------------------------------------------------------ fused projection GEMM
+@pytest.mark.parametrize("T,K,Hq,Hkv,front,back", [(300, 320, 4, 2, 2, 0), (70, 64, 8, 1, 0, 8), (513, 2560, 32, 8, 8, 0),
+                                                    (1000, 2560, 32, 8, 0, 32), (257, 192, 3, 1, 0, 0)])
+def test_qkv_proj_gemm_with_norm_rope_epilogue(ops, T, K, Hq, Hkv, front, back):
+    """x . [router | q | k | v | router]^T with the q / k RMSNorm + rotary in the GEMM's epilogue against fp64
+    F.linear + Qwen3RMSNorm + the rotary by the table entries the kernel reads (and the fp64 rotary at small
+    positions); v and the router heads are the plain projection.  Ragged token counts (partial M tiles), head
+    counts that leave half an N tile empty, router heads in front (stage 1) or behind (stage 2)."""
+    say(f"qkv_proj T={T} K={K} Hq={Hq} Hkv={Hkv} router front={front} back={back}")
+    D, eps, theta = 128, 1e-6, 1e6
+    heads = front + Hq + 2 * Hkv + back
+    x = _randn((T, K), 300 + T, torch.bfloat16)
+    w = (_randn((heads * D, K), 301 + K, torch.float32) * K ** -0.5).to(torch.bfloat16)
+    qw = (1 + 0.1 * _randn((D,), 302, torch.float32)).to(torch.bfloat16)
+    kw = (1 + 0.1 * _randn((D,), 303, torch.float32)).to(torch.bfloat16)
+    g = torch.Generator().manual_seed(304)
+    pos = torch.randint(0, 4000, (T,), generator=g, dtype=torch.int64)
+    pos[: min(T, 40)] = torch.arange(min(T, 40))
+    rope = ops.rope_tables(4096, D, theta)
+    q, k, v, r = ops.qkv_proj(x.cuda(), w.cuda(), Hq, Hkv, pos.cuda(), qw.cuda(), kw.cuda(), eps, rope,
+                              router_front=front, router_back=back)
+    torch.cuda.synchronize()
+    y = (x.double() @ w.double().T).view(T, heads, D)
+
+    def norm(t, wt):
+        return t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps) * wt.double()
+    c, s_ = rope[0].cpu().double()[pos][:, None, :], rope[1].cpu().double()[pos][:, None, :]
+
+    def rot(t):
+        a, b = t[..., :64], t[..., 64:]
+        return torch.cat([a * c - b * s_, b * c + a * s_], dim=-1)
+    nq, nk = norm(y[:, front:front + Hq], qw), norm(y[:, front + Hq:front + Hq + Hkv], kw)
+    tol = 1e-2
+    assert q.shape == (T, Hq, D) and k.shape == (T, Hkv, D) and v.shape == (T, Hkv, D)
+    assert cf.rel_err(q.cpu(), rot(nq)) < tol and cf.rel_err(k.cpu(), rot(nk)) < tol
+    small = pos < 64
+    assert cf.rel_err(q.cpu()[small], cf.apply_rope(nq[small], pos[small], theta)) < tol
+    assert cf.rel_err(v.cpu(), y[:, front + Hq + Hkv:front + Hq + 2 * Hkv]) < tol
+    if front + back:
+        want_r = torch.cat([y[:, :front], y[:, front + Hq + 2 * Hkv:]], dim=1)
+        assert r.shape == (T, front + back, D) and cf.rel_err(r.cpu(), want_r) < tol
+    else:
+        assert r is None
+    # the two-step path (vendor GEMM, then the norm + rotary kernel) lands on the same values up to bf16 rounding
+    qkv = torch.nn.functional.linear(x.cuda(), w.cuda()[front * D:(front + Hq + 2 * Hkv) * D])
+    q2, k2, v2 = ops.qk_norm_rope(qkv, Hq, Hkv, D, pos.cuda(), qw.cuda(), kw.cuda(), eps, rope)
+    assert cf.rel_err(q.cpu(), q2.double().cpu()) < 2e-2 and cf.rel_err(k.cpu(), k2.double().cpu()) < 2e-2
+
+
 # ------------------------------------------------------------------ fused layer helpers
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_qk_norm_rope_rmsnorm_silu(ops, dtype):

@@ -524,7 +524,8 @@ def main():
             by = C_total * HKV * D * 2 + b1 * s1 * HQ * D * 2 + C_total * 4 + b1 * TOPK * 16
             sweep.append({"B": b1, "S": s1, "call_ms": round(call_ms, 4), "GB/s": round(by / call_ms / 1e6, 1),
                           "frac_hbm": round(by / call_ms / 1e6 / HBM_PEAK_GBS, 4), "scan_kernel_ms": round(ms1, 4),
-                          "scan_kernel_frac_hbm": round(by / ms1 / 1e6 / HBM_PEAK_GBS, 4)})
+                          "scan_kernel_frac_hbm": round(by / ms1 / 1e6 / HBM_PEAK_GBS, 4), "algorithmic_bytes": by,
+                          "traffic": measured_traffic("score_gemm_kernel", f"tokens={args.tokens},B={b1},S={s1}")})
         _lib.check(lib.msa_profile_enable(0), "msa_profile_enable")
     if args.sweep_only:
         print(json.dumps({"hbm_regime_sweep": sweep}), flush=True)

@@ -362,6 +362,8 @@ def main():
                 e = min(C_total, s + step)
                 h[s:e].copy_(torch.randn((e - s, HKV, D), generator=g, device=dev).to(torch.bfloat16))
             dst.append(h)
+        if n_host > 2:
+            log(f"host K/V: layer buffer {i + 1} of {n_host} filled")
     log(f"host K/V: {n_host} layer buffer(s), {2 * n_host * C_total * HKV * D * 2 / 1e9:.1f} GB pinned")
 
     qs, wants, krs = [], [], []

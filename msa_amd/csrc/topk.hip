@@ -12,8 +12,25 @@ namespace {
 
 constexpr int kWaves = 4;
 
+// Lane i receives the value of lane i ^ m.  Masks up to 8 stay inside a row of 16 lanes and are data-parallel
+// moves (a few cycles); 16 and 32 cross rows and go through the LDS crossbar.  The sort networks below are chains of
+// dependent exchanges, so this latency is what the top-k kernels spend their time on.
+__device__ __forceinline__ uint32_t xor_lanes_u32(uint32_t v, int m) {
+  const int x = (int)v;
+  switch (m) {
+    case 1: return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0xB1, 0xF, 0xF, false);    // quad_perm [1,0,3,2]
+    case 2: return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0x4E, 0xF, 0xF, false);    // quad_perm [2,3,0,1]
+    case 4: {
+      // lanes 0-3 and 8-11 of a row read four lanes up (row_shl:4), the others four lanes down (row_shr:4)
+      const int t = __builtin_amdgcn_update_dpp(x, x, 0x104, 0xF, 0x5, false);
+      return (uint32_t)__builtin_amdgcn_update_dpp(t, x, 0x114, 0xF, 0xA, false);
+    }
+    case 8: return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0x128, 0xF, 0xF, false);   // row_ror:8
+    default: return (uint32_t)__shfl_xor(x, m);
+  }
+}
 __device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int m) {
-  return (uint64_t)__shfl_xor((unsigned long long)v, m);
+  return ((uint64_t)xor_lanes_u32((uint32_t)(v >> 32), m) << 32) | xor_lanes_u32((uint32_t)v, m);
 }
 __device__ __forceinline__ uint64_t shfl_u64(uint64_t v, int src) {
   return (uint64_t)__shfl((unsigned long long)v, src);

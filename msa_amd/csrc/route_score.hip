@@ -319,29 +319,60 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   };
 
   // Epilogue of the N tile starting at chunk `tile_n0`.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of
-  // its 32x32 block.  Consecutive row blocks of one query are folded into `run`; emit() then merges the query's 32
-  // column maxima of this block into the key plane.  Several wavefronts and workgroups hold parts of a query (and
-  // of a document), so the merge is an atomicMax into a zeroed plane.  emit() is reached by whole wavefronts (q
-  // and any are uniform).
+  // its 32x32 block.  Consecutive row blocks of one query are folded into `run` (each half of the wavefront over its
+  // own rows); emit() joins the halves and merges the query's 32 column maxima of this block into the key plane.
+  // Several wavefronts and workgroups hold parts of a query (and of a document), so the merge is an atomicMax into
+  // a zeroed plane.  emit() is reached by whole wavefronts (q and any are uniform).
+  //
+  // With one workgroup per compute unit nothing else runs while an epilogue waits, so it must not wait on memory:
+  // the scored-row words of the wavefront's row blocks and the documents of its columns are requested ahead (before
+  // the K loop / a tile ahead) and only consumed here, and the lane exchanges of the document fold are row moves.
   const int n_queries = M_rows / (blocks_per_query * 32);
-  auto emit = [&](int q, int n, float run, bool any) {
+  uint32_t rbits[TM];                                   // scored-row word of each row block (same in every lane)
+#pragma unroll
+  for (int i = 0; i < TM; ++i) rbits[i] = row_bits[(m0 + wm * WM + i * 32) >> 5];   // 0 past M_rows (buffer is padded)
+  int cdoc[TN];                                         // document of each column; lanes past the bank never join a run
+  auto fetch_docs = [&](int tile_n0) {
+    if constexpr (kDocMax) {
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int n = tile_n0 + wn * WN + j * 32 + l32;
+        cdoc[j] = n < C ? chunk_doc[n] : -1 - l32;
+      }
+    }
+  };
+  auto emit = [&](int q, int n, int doc, float run_half, bool any) {
     if (!any || q >= n_queries) return;
+    const float run = fmaxf(run_half, __shfl_xor(run_half, 32));
     const bool ok = n < C;
     const uint32_t key = ok ? f32_to_key(run) : 0u;
     if constexpr (kDocMax) {
       // Chunks of a document are adjacent columns: a segmented max-scan over the 32 lanes of each half leaves a
       // document's maximum in the last lane of its run, which alone touches memory (about two atomics per 32
-      // chunks instead of 32 stores, and no per-chunk plane to read back).
-      const int doc = ok ? chunk_doc[n] : -1 - l32;        // lanes past the bank never join a run
-      uint32_t m = key;
-#pragma unroll
-      for (int off = 1; off < 32; off <<= 1) {
-        const uint32_t om = (uint32_t)__shfl_up((int)m, off, 32);
-        const int od = __shfl_up(doc, off, 32);
-        if (l32 >= off && od == doc) m = max(m, om);
+      // chunks instead of 32 stores, and no per-chunk plane to read back).  `dist` is a lane's distance from the
+      // first lane of its run, from a ballot of the run heads; the scan itself moves keys only: four shifts inside
+      // the rows of 16 lanes, then lane 15 of the lower row joins the runs that cross into the upper one.  Lanes a
+      // shift cannot reach read 0, the identity of max over keys.
+      const int prev = __builtin_amdgcn_update_dpp(doc, doc, 0x138, 0xF, 0xF, false);      // wave_shr:1
+      const uint64_t heads64 = __ballot(l32 == 0 || prev != doc);
+      const uint32_t heads = half ? (uint32_t)(heads64 >> 32) : (uint32_t)heads64;
+      const uint32_t upto = heads & ((2u << l32) - 1u);                  // heads at or below this lane (never empty)
+      const int dist = l32 - (31 - __builtin_clz(upto));
+      const bool last = l32 == 31 || ((heads >> (l32 + 1)) & 1u);
+      int m = (int)key;
+#define MSA_SCAN_STEP(OFF, CTRL)                                                          \
+      {                                                                                   \
+        const int o = __builtin_amdgcn_update_dpp(0, m, CTRL, 0xF, 0xF, true);            \
+        if (dist >= OFF) m = (int)max((uint32_t)m, (uint32_t)o);                          \
       }
-      const int nd = __shfl_down(doc, 1, 32);
-      if (ok && half == 0 && (l32 == 31 || nd != doc)) atomicMax(&out_key[(int64_t)q * n_docs + doc], m);
+      MSA_SCAN_STEP(1, 0x111)   // row_shr:1
+      MSA_SCAN_STEP(2, 0x112)
+      MSA_SCAN_STEP(4, 0x114)
+      MSA_SCAN_STEP(8, 0x118)
+#undef MSA_SCAN_STEP
+      const int low = __builtin_amdgcn_update_dpp(0, m, 0x142, 0xA, 0xF, false);          // row_bcast:15 into rows 1, 3
+      if (dist > (l32 & 15)) m = (int)max((uint32_t)m, (uint32_t)low);
+      if (ok && half == 0 && last) atomicMax(&out_key[(int64_t)q * n_docs + doc], (uint32_t)m);
     } else {
       if (ok && half == 0) atomicMax(&out_key[(int64_t)q * C + n], key);
     }
@@ -350,6 +381,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n = tile_n0 + wn * WN + j * 32 + l32;
+      const int doc = kDocMax ? cdoc[j] : 0;
       float run = -INFINITY;
       bool any = false;
       int run_q = -1;
@@ -357,24 +389,28 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
       for (int i = 0; i < TM; ++i) {
         const int blk = (m0 + wm * WM + i * 32) >> 5;      // global 32-row block index
         const int qid = blk / blocks_per_query;
-        const uint32_t bits = row_bits[blk];               // 0 for blocks past M_rows (buffer is padded)
+        const uint32_t bits = __builtin_amdgcn_readfirstlane(rbits[i]);
         if (qid != run_q) {
-          if (run_q >= 0) emit(run_q, n, run, any);
+          if (run_q >= 0) emit(run_q, n, doc, run, any);
           run = -INFINITY; any = false; run_q = qid;
         }
-        if (bits != 0) {
+        if (bits == 0xffffffffu) {                          // every row scored: no per-row tests
+          float mx = acc[i][j][0];
+#pragma unroll
+          for (int e = 1; e < 16; ++e) mx = fmaxf(mx, acc[i][j][e]);
+          run = fmaxf(run, mx);
+          any = true;
+        } else if (bits != 0) {
+          const uint32_t mine = bits >> (4 * half);         // this half's rows: bit 8*(e/4) + e%4
           float mx = -INFINITY;
 #pragma unroll
-          for (int e = 0; e < 16; ++e) {
-            const int r = 8 * (e >> 2) + 4 * half + (e & 3);
-            if (bits & (1u << r)) mx = fmaxf(mx, acc[i][j][e]);
-          }
-          mx = fmaxf(mx, __shfl_xor(mx, 32));
+          for (int e = 0; e < 16; ++e)
+            if (mine & (1u << (8 * (e >> 2) + (e & 3)))) mx = fmaxf(mx, acc[i][j][e]);
           run = fmaxf(run, mx);
           any = true;
         }
       }
-      emit(run_q, n, run, any);
+      emit(run_q, n, doc, run, any);
     }
   };
 
@@ -390,6 +426,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     if constexpr (kSets == 2) load_next(Set0{});
     __syncthreads();
     load_frags(0, 0, 0);
+    fetch_docs(n0);
     int done_n0 = n0, in_tile = 0;
     for (int step = 0; step + 2 < steps; step += 2) {
       k_tile(std::true_type{}, Set1{}, step);
@@ -405,6 +442,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
             for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
         in_tile = 0;
         done_n0 += (int)gridDim.x * BN;
+        fetch_docs(done_n0);
       }
     }
     k_tile(std::true_type{}, Set1{}, steps - 2);
@@ -419,6 +457,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
       load_tile(Set0{}, 2);
       __syncthreads();
       load_frags(0, 0, 0);
+      fetch_docs(n0);
       int kt = 0;
       for (; kt + 2 < k_tiles; kt += 2) {
         k_tile(std::true_type{}, Set1{}, kt);
@@ -436,6 +475,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
       if (k_tiles > 1) load_tile(Set0{}, 1);
       __syncthreads();
       load_frags(0, 0, 0);
+      fetch_docs(n0);
       for (int kt = 0; kt + 1 < k_tiles; ++kt) k_tile(std::true_type{}, Set0{}, kt);
       k_tile(std::false_type{}, Set0{}, k_tiles - 1);
     }

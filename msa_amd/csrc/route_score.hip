@@ -331,6 +331,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   uint32_t rbits[TM];                                   // scored-row word of each row block (same in every lane)
 #pragma unroll
   for (int i = 0; i < TM; ++i) rbits[i] = row_bits[(m0 + wm * WM + i * 32) >> 5];   // 0 past M_rows (buffer is padded)
+  // query of the wavefront's first row block and that block's place in the query: later blocks follow by counting
+  // (one division per wavefront, ahead of the K loop, instead of one per block in the epilogue)
+  const int blk0 = (m0 + wm * WM) >> 5;
+  const int q_first = blk0 / blocks_per_query, r_first = blk0 - q_first * blocks_per_query;
   int cdoc[TN];                                         // document of each column; lanes past the bank never join a run
   auto fetch_docs = [&](int tile_n0) {
     if constexpr (kDocMax) {
@@ -384,16 +388,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
       const int doc = kDocMax ? cdoc[j] : 0;
       float run = -INFINITY;
       bool any = false;
-      int run_q = -1;
+      int run_q = q_first, r = r_first;                    // query of row block i, its block index inside the query
 #pragma unroll
       for (int i = 0; i < TM; ++i) {
-        const int blk = (m0 + wm * WM + i * 32) >> 5;      // global 32-row block index
-        const int qid = blk / blocks_per_query;
         const uint32_t bits = __builtin_amdgcn_readfirstlane(rbits[i]);
-        if (qid != run_q) {
-          if (run_q >= 0) emit(run_q, n, doc, run, any);
-          run = -INFINITY; any = false; run_q = qid;
+        if (r == blocks_per_query) {                       // row block i opens the next query
+          emit(run_q, n, doc, run, any);
+          run = -INFINITY; any = false; ++run_q; r = 0;
         }
+        ++r;
         if (bits == 0xffffffffu) {                          // every row scored: no per-row tests
           float mx = acc[i][j][0];
 #pragma unroll

@@ -329,12 +329,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   // the K loop / a tile ahead) and only consumed here, and the lane exchanges of the document fold are row moves.
   const int n_queries = M_rows / (blocks_per_query * 32);
   uint32_t rbits[TM];                                   // scored-row word of each row block (same in every lane)
-#pragma unroll
-  for (int i = 0; i < TM; ++i) rbits[i] = row_bits[(m0 + wm * WM + i * 32) >> 5];   // 0 past M_rows (buffer is padded)
   // query of the wavefront's first row block and that block's place in the query: later blocks follow by counting
-  // (one division per wavefront, ahead of the K loop, instead of one per block in the epilogue)
-  const int blk0 = (m0 + wm * WM) >> 5;
-  const int q_first = blk0 / blocks_per_query, r_first = blk0 - q_first * blocks_per_query;
+  // (one division per wavefront, under the first tile's load latency, instead of one per block in the epilogue)
+  int q_first = 0, r_first = 0;
+  auto fetch_rows = [&]() {
+#pragma unroll
+    for (int i = 0; i < TM; ++i) rbits[i] = row_bits[(m0 + wm * WM + i * 32) >> 5];   // 0 past M_rows (buffer is padded)
+    const int blk0 = (m0 + wm * WM) >> 5;
+    q_first = blk0 / blocks_per_query;
+    r_first = blk0 - q_first * blocks_per_query;
+  };
   int cdoc[TN];                                         // document of each column; lanes past the bank never join a run
   auto fetch_docs = [&](int tile_n0) {
     if constexpr (kDocMax) {
@@ -429,6 +433,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     if constexpr (kSets == 2) load_next(Set0{});
     __syncthreads();
     load_frags(0, 0, 0);
+    fetch_rows();
     fetch_docs(n0);
     int done_n0 = n0, in_tile = 0;
     for (int step = 0; step + 2 < steps; step += 2) {
@@ -460,6 +465,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
       load_tile(Set0{}, 2);
       __syncthreads();
       load_frags(0, 0, 0);
+      fetch_rows();
       fetch_docs(n0);
       int kt = 0;
       for (; kt + 2 < k_tiles; kt += 2) {
@@ -478,6 +484,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
       if (k_tiles > 1) load_tile(Set0{}, 1);
       __syncthreads();
       load_frags(0, 0, 0);
+      fetch_rows();
       fetch_docs(n0);
       for (int kt = 0; kt + 1 < k_tiles; ++kt) k_tile(std::true_type{}, Set0{}, kt);
       k_tile(std::false_type{}, Set0{}, k_tiles - 1);

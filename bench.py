@@ -317,7 +317,7 @@ def main():
     ap.add_argument("--seq", type=int, default=128)
     ap.add_argument("--host-kv-layers", type=int, default=2,
                     help="distinct pinned host K/V layer buffers (routed layers share them round-robin)")
-    ap.add_argument("--gather", choices=["device", "memcpy"], default="memcpy",
+    ap.add_argument("--gather", choices=["device", "memcpy"], default="device",
                     help="device: plan + copy kernels read the pinned bank directly, no ids on the host; "
                          "memcpy: ids to the host, one hipMemcpyAsync per document run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -384,6 +384,8 @@ def main():
     gids = [torch.empty((B, TOPK), dtype=torch.int64, device=dev) for _ in range(L)]
     docs_host = [torch.empty((B, TOPK), dtype=torch.int32, pin_memory=True) for _ in range(L)]
     ready = [torch.cuda.Event() for _ in range(L)]
+    scored = [torch.cuda.Event() for _ in range(L)]
+    ids_stream = torch.cuda.Stream()
     cap_chunks = B * TOPK * 32
     gk = [torch.empty((cap_chunks, HKV, D), dtype=torch.bfloat16, device=dev) for _ in range(2)]
     gv = [torch.empty((cap_chunks, HKV, D), dtype=torch.bfloat16, device=dev) for _ in range(2)]
@@ -391,26 +393,40 @@ def main():
     main_stream = torch.cuda.current_stream()
     sel_chunks = [0] * L
 
+    host_s = {"wait": 0.0, "copy_calls": 0.0, "route_calls": 0.0}   # host time: waiting for a layer's ids, issuing its copies, its kernels
+
     def route(li):
+        t_r = time.perf_counter()
         _lib.check(lib.msa_route_topk(bank.handle, li, qs[li].data_ptr(), None, B, S, HQ, _lib.MODE_COSINE, 1.0, TOPK,
                                       scores[li].data_ptr(), docs[li].data_ptr(), gids[li].data_ptr(), ws.data_ptr(),
                                       ws.numel(), main_stream.cuda_stream), "msa_route_topk")
-        docs_host[li].copy_(docs[li], non_blocking=True)
-        ready[li].record(main_stream)
+        # The ids leave on a stream of their own: a copy queued on the scan's stream would hold the next layer's
+        # kernels back whenever the copy engine is still busy with the previous layer's K / V.
+        scored[li].record(main_stream)
+        ids_stream.wait_event(scored[li])
+        with torch.cuda.stream(ids_stream):
+            docs_host[li].copy_(docs[li], non_blocking=True)
+        ready[li].record(ids_stream)
+        host_s["route_calls"] += time.perf_counter() - t_r
+
 
     def gather(li):
+        t_a = time.perf_counter()
         ready[li].synchronize()
+        t_b = time.perf_counter()
         cu = torch.empty(B + 1, dtype=torch.int64)
         _lib.check(lib.msa_gather_plan(bank.handle, docs_host[li].data_ptr(), B, TOPK, cu.data_ptr()), "msa_gather_plan")
         sel_chunks[li] = int(cu[-1])
         _lib.check(lib.msa_gather_kv(bank.handle, li, docs_host[li].data_ptr(), B, TOPK, gk[li & 1].data_ptr(),
                                      gv[li & 1].data_ptr(), cap_chunks, side.cuda_stream), "msa_gather_kv")
+        host_s["wait"] += t_b - t_a
+        host_s["copy_calls"] += time.perf_counter() - t_b
 
     cu_dev = [torch.empty(B + 1, dtype=torch.int32, device=dev) for _ in range(L)]
     gws = torch.empty(lib.msa_gather_device_workspace_bytes(B, TOPK), dtype=torch.uint8, device=dev)
 
     def gather_device(li):
-        side.wait_event(ready[li])         # no host wait: the side stream picks the ids up on the device
+        side.wait_event(scored[li])        # no host wait: the side stream picks the ids up on the device
         _lib.check(lib.msa_gather_kv_device(bank.handle, li, docs[li].data_ptr(), B, TOPK, gk[li & 1].data_ptr(),
                                             gv[li & 1].data_ptr(), cap_chunks, cu_dev[li].data_ptr(), gws.data_ptr(),
                                             gws.numel(), side.cuda_stream), "msa_gather_kv_device")
@@ -440,6 +456,7 @@ def main():
     torch.cuda.synchronize()
     _lib.check(lib.msa_profile_enable(args.steps * L), "msa_profile_enable")
     torch.cuda.synchronize()
+    host_s["wait"] = host_s["copy_calls"] = host_s["route_calls"] = 0.0
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
@@ -567,7 +584,8 @@ def main():
         "config": {"workload": "configs[3]: 100M-token bank, K_r HBM-resident, K/V pinned host, B=16 x S=128, top-16",
                    "bank_tokens": args.tokens, "chunks": C_total, "docs": n_docs, "routed_layers": L, "batch": B,
                    "query_tokens": S, "top_k": TOPK, "kr_hbm_gb": round(C_total * HKV * D * 2 * L / 1e9, 1),
-                   "host_kv_layer_buffers": n_host, "gather": args.gather, "selected_chunks_per_layer": int(np.mean(sel_chunks)),
+                   "host_kv_layer_buffers": n_host, "gather": args.gather,
+                   "gather_host_ms_per_layer": {k: round(v / (args.steps * L) * 1e3, 3) for k, v in host_s.items()}, "selected_chunks_per_layer": int(np.mean(sel_chunks)),
                    "mode": "cosine/mean-heads/max-tokens/max-chunks"},
         "roofline": roof, "cpu_baseline": cpu, "hbm_regime_sweep": sweep, "other_kernels": extras, "parity": "needles exact on all layers",
     }

@@ -9,6 +9,8 @@
 
 #include "common.h"
 
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
 namespace {
 
 // Sorted unique valid documents of sample b; returns false on an out-of-range index.
@@ -214,22 +216,44 @@ __global__ __launch_bounds__(kPlanWaves * 64) void gather_plan_kernel(const int3
 // grid.x = plan entry, grid.y = row group; 128 lanes move one row of K and of V per step.
 // kFromDevice = false: entries without an earlier copy, rows read from the pinned host bank;
 // kFromDevice = true: the others, rows read from the earlier copy inside the output itself.
+// The kernel stays within 16 vector registers (rows travel through buffer resources, i.e. scalar addresses and one
+// vector offset): a scoring workgroup of the routing scan takes 496 of a SIMD's 512, and only a wavefront that fits
+// beside it runs under the scan instead of taking a compute unit's turn between two of its workgroups (the copy is
+// PCIe-bound: it needs residency, not registers).
+// Few workgroups: PCIe reads are slow to return and a compute unit's memory pipeline serves its wavefronts in order, so
+// every compute unit that hosts a copy wavefront slows the scoring workgroup beside it.  32 workgroups keep 128 KB in
+// flight, enough for the link, and leave the other compute units alone (scan under the copy 5.81 ms against 6.15 ms
+// with 2048 workgroups, 5.75 ms without a copy).
+constexpr int kCopyGridX = 16, kCopyGridY = 2;
 template <bool kFromDevice>
 __global__ __launch_bounds__(128) void gather_copy_kernel(const uint4* __restrict__ k_src, const uint4* __restrict__ v_src,
-                                                          const int32_t* __restrict__ plan, int32_t row_vecs,
-                                                          int64_t capacity_rows, uint4* k_dst, uint4* v_dst) {
-  const int32_t* e = plan + (int64_t)blockIdx.x * kPlanInts;
+                                                          const int32_t* __restrict__ plan, int32_t n_entries,
+                                                          int32_t row_vecs, int64_t capacity_rows, uint4* k_dst,
+                                                          uint4* v_dst) {
+  const int row_bytes = row_vecs * 16;
+  for (int ent = blockIdx.x; ent < n_entries; ent += gridDim.x) {
+  const int32_t* e = plan + (int64_t)ent * kPlanInts;
   const int32_t n = e[1], dst0 = e[2], from = e[3];
-  if ((from >= 0) != kFromDevice) return;
+  if ((from >= 0) != kFromDevice) continue;
   const int32_t src0 = kFromDevice ? from : e[0];
   for (int r = blockIdx.y; r < n; r += gridDim.y) {
-    if ((int64_t)dst0 + r >= capacity_rows) return;
-    if (kFromDevice && (int64_t)src0 + r >= capacity_rows) return;
+    if ((int64_t)dst0 + r >= capacity_rows) break;
+    if (kFromDevice && (int64_t)src0 + r >= capacity_rows) break;
     const uint4* ks = (kFromDevice ? k_dst : k_src) + ((int64_t)src0 + r) * row_vecs;
     const uint4* vs = (kFromDevice ? v_dst : v_src) + ((int64_t)src0 + r) * row_vecs;
     uint4* kd = k_dst + ((int64_t)dst0 + r) * row_vecs;
     uint4* vd = v_dst + ((int64_t)dst0 + r) * row_vecs;
-    for (int i = threadIdx.x; i < row_vecs; i += 128) { kd[i] = ks[i]; vd[i] = vs[i]; }
+    const __amdgpu_buffer_rsrc_t rks = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(ks), 0, row_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rvs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(vs), 0, row_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rkd = __builtin_amdgcn_make_buffer_rsrc(kd, 0, row_bytes, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rvd = __builtin_amdgcn_make_buffer_rsrc(vd, 0, row_bytes, 0x00020000);
+    for (int off = threadIdx.x * 16; off < row_bytes; off += 128 * 16) {
+      const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(rks, off, 0, 0);
+      const u32x4_t b = __builtin_amdgcn_raw_buffer_load_b128(rvs, off, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(a, rkd, off, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(b, rvd, off, 0, 0);
+    }
+  }
   }
 }
 
@@ -264,14 +288,14 @@ extern "C" int msa_gather_kv_device(const msa_bank* bank, int32_t layer, const i
                                                       cap32, dedup, cu_sel, plan);
   MSA_LAUNCH_CHECK();
   const int32_t row_vecs = (int32_t)((size_t)bank->Hkv * bank->D * elem_bytes(bank->dtype) / 16);
-  dim3 grid((unsigned)(B * k), 8);
+  dim3 grid((unsigned)std::min(B * k, kCopyGridX), kCopyGridY);
   gather_copy_kernel<false><<<grid, 128, 0, st>>>(static_cast<const uint4*>(bank->k_host[layer]),
-                                                  static_cast<const uint4*>(bank->v_host[layer]), plan, row_vecs,
+                                                  static_cast<const uint4*>(bank->v_host[layer]), plan, B * k, row_vecs,
                                                   out_capacity_chunks, static_cast<uint4*>(k_out),
                                                   static_cast<uint4*>(v_out));
   MSA_LAUNCH_CHECK();
   if (dedup) {
-    gather_copy_kernel<true><<<grid, 128, 0, st>>>(nullptr, nullptr, plan, row_vecs, out_capacity_chunks,
+    gather_copy_kernel<true><<<grid, 128, 0, st>>>(nullptr, nullptr, plan, B * k, row_vecs, out_capacity_chunks,
                                                    static_cast<uint4*>(k_out), static_cast<uint4*>(v_out));
     MSA_LAUNCH_CHECK();
   }

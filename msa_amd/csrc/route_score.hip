@@ -19,6 +19,15 @@ namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+// 16 bytes per lane from a buffer resource straight into LDS (lane l lands at byte 16 * l behind `lds_dst`, which must be
+// the same in every lane).  The compiler's host pass has no such instruction and only needs the kernel's signature.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define MSA_LOAD_TO_LDS(rsrc, lds_dst, voffset, soffset, aux) \
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(lds_dst), 16, voffset, soffset, 0, aux)
+#else
+#define MSA_LOAD_TO_LDS(rsrc, lds_dst, voffset, soffset, aux) ((void)(rsrc), (void)(lds_dst), (void)(voffset), (void)(soffset))
+#endif
 
 // ------------------------------------------------------------------------------------------
 // Prologue: normalise (cosine mode), sum the G heads of each KV group, cast, build row masks, clear the key plane.
@@ -135,6 +144,21 @@ struct Mma<float> {
   }
 };
 
+// The MFMA-bound form (bf16, 256 x 256, one workgroup per tile) stages its operand tiles with buffer loads that write
+// LDS directly: no staging registers, no ds_write, and room for a third stage of the operand that comes from HBM.
+// LDS then holds two stages of the query tile (2 x 32 KB) and three of the K_r tile (3 x 32 KB), 160 KB in all, in
+// un-padded 128-byte rows whose 16-byte units are XOR-swizzled by (row >> 1) & 7 (conflict-free operand reads; a
+// direct load cannot pad, its 64 lanes fill 1 KB of LDS in lane order, so the swizzle is applied to the global
+// address each lane fetches).  K_r tile kt + 2 and query tile kt + 1 are requested at the start of step kt; the wait in
+// front of the step's barrier leaves the newest K_r tile in flight.  7.5 % faster than the register-staged form in a
+// stand-alone copy of the loop (1312-1320 against 1218-1229 TFLOP/s).
+constexpr int kDtlStageBytes = 256 * 128;
+constexpr int kDtlLdsBytes = 5 * kDtlStageBytes;
+template <typename T, int BM, int BN, int kSets, bool kStream>
+constexpr bool score_tile_is_direct() {
+  return sizeof(T) == 2 && BM == 256 && BN == 256 && kSets == 1 && !kStream;
+}
+
 // Workgroup tile BM x BN, WAVES_M x WAVES_N wavefronts, each owning TM x TN blocks of 32 x 32.
 // kSets: register sets of global loads, i.e. K tiles in flight ahead of the one being multiplied.  One is enough when
 // a tile's MFMA work outlasts a load's latency (the MFMA-bound shapes); the HBM-bound shapes (few query rows) need
@@ -163,6 +187,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
 
   extern __shared__ __align__(16) char lds[];
   constexpr int kBufBytes = (BM + BN) * kRowStride;   // [A tile | B tile] per buffer, two buffers
+  constexpr bool kDtl = score_tile_is_direct<T, BM, BN, kSets, kStream>();
 
   // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so each XCD gets one
   // contiguous range of K_r tiles.  Inside it the M tiles are walked in groups of m_group: a group's
@@ -318,6 +343,39 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     }
   };
 
+  // ---- direct-to-LDS form (see score_tile_is_direct) ----
+  // A wavefront's load instruction i covers rows (wave * 4 + i) * 8 .. + 8 of the operand tile: lane l lands in LDS at
+  // byte 16 * l of that 1 KB block, i.e. row l / 8, unit slot l % 8, and fetches the unit that belongs there.
+  const int dtl_row = (lane >> 3), dtl_slot = lane & 7;
+  auto dtl_voff = [&](int i) {
+    const int row = (wave * 4 + i) * 8 + dtl_row;
+    return row * (int)row_bytes_g + ((dtl_slot ^ ((row >> 1) & 7)) * 16);
+  };
+  auto dtl_load_a = [&](int stage, int kt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      MSA_LOAD_TO_LDS(rsrc_a, lds + stage * kDtlStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes, 0);
+  };
+  auto dtl_load_b = [&](int stage, int kt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      MSA_LOAD_TO_LDS(rsrc_b, lds + (2 + stage) * kDtlStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes,
+                      kStreamHint);
+  };
+  auto dtl_frags = [&](int sa, int sb, int sub, int slot) {
+    const int unit = sub * 2 + half;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = wm * WM + i * 32 + l32;
+      fa[slot][i] = *reinterpret_cast<const Frag*>(lds + sa * kDtlStageBytes + row * 128 + ((unit ^ ((row >> 1) & 7)) * 16));
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int row = wn * WN + j * 32 + l32;
+      fb[slot][j] = *reinterpret_cast<const Frag*>(lds + (2 + sb) * kDtlStageBytes + row * 128 + ((unit ^ ((row >> 1) & 7)) * 16));
+    }
+  };
+
   // Epilogue of the N tile starting at chunk `tile_n0`.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of
   // its 32x32 block.  Consecutive row blocks of one query are folded into `run` (each half of the wavefront over its
   // own rows); emit() joins the halves and merges the query's 32 column maxima of this block into the key plane.
@@ -421,7 +479,66 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     }
   };
 
-  if constexpr (kStream) {
+  if constexpr (kDtl) {
+    static_assert(kThreads == 512 && kSub == 4, "the direct-to-LDS form is laid out for 8 wavefronts of bf16");
+    // vmcnt(4) / vmcnt(0) with the other counters left alone: the four newest loads are the K_r tile two steps ahead
+    constexpr int kWaitAllButNewestB = 0x0F74, kWaitAll = 0x0F70;
+    // The workgroup barrier of this form is written out: __syncthreads() carries a release fence, for which the
+    // compiler drains every outstanding load that writes LDS (vmcnt(0)), the K_r tile two steps ahead included, which
+    // is exactly the wait the third stage exists to avoid.  The explicit vmcnt wait in front of it covers the tiles
+    // the next step reads; the LDS reads of this step are drained by lgkmcnt(0).
+    auto dtl_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    dtl_load_a(0, 0);
+    dtl_load_b(0, 0);
+    if (k_tiles > 1) {
+      dtl_load_b(1, 1);
+      __builtin_amdgcn_s_waitcnt(kWaitAllButNewestB);
+    } else {
+      __builtin_amdgcn_s_waitcnt(kWaitAll);
+    }
+    dtl_barrier();
+    dtl_frags(0, 0, 0, 0);
+    fetch_rows();
+    fetch_docs(n0);
+    // the prefetches above are four more loads in flight behind tile 0: they are older than every later tile load,
+    // so the waits below, which count from the newest, cover them
+    int sb = 0;
+    for (int kt = 0; kt < k_tiles; ++kt) {
+      const int sa = kt & 1;
+      const bool more = kt + 1 < k_tiles, more2 = kt + 2 < k_tiles;
+      const int sb1 = sb == 2 ? 0 : sb + 1, sb2 = sb1 == 2 ? 0 : sb1 + 1;
+      if (more) dtl_load_a(sa ^ 1, kt + 1);      // stage of tile kt - 1: its last reads were behind the previous barrier
+      if (more2) dtl_load_b(sb2, kt + 2);
+#pragma unroll
+      for (int sub = 0; sub < kSub; ++sub) {
+        if (sub + 1 < kSub) {
+          dtl_frags(sa, sb, sub + 1, (sub + 1) & 1);
+        } else if (more) {
+          if (more2) __builtin_amdgcn_s_waitcnt(kWaitAllButNewestB);
+          else __builtin_amdgcn_s_waitcnt(kWaitAll);
+          dtl_barrier();
+          dtl_frags(sa ^ 1, sb1, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::mma(fa[sub & 1][i], fb[sub & 1][j], acc[i][j]);
+        if (sub + 1 < kSub) {
+          // issue order of the sub-step: each of the six operand reads of the next sub-step behind one MFMA of this
+          // one, the last two MFMAs behind them (2.5 % faster than the order the scheduler picks by itself)
+#pragma unroll
+          for (int g = 0; g < 6; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+          }
+          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        }
+      }
+      sb = sb1;
+    }
+    epilogue(n0);
+  } else if constexpr (kStream) {
     // The workgroup's tiles form one sequence of steps (K tiles are even in number, so set tags and LDS buffers
     // alternate the same way in every tile); an epilogue sits where a tile's last step ends, with the next tile's
     // first operand fragments already in registers and its loads in flight.
@@ -531,7 +648,8 @@ int compute_units() {
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool kDocMax, bool kStream>
 int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key, const int32_t* chunk_doc,
                 int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t n_docs, hipStream_t st) {
-  const size_t lds = (size_t)2 * (BM + BN) * kRowStride;
+  const size_t lds = score_tile_is_direct<T, BM, BN, kSets, kStream>() ? (size_t)kDtlLdsBytes
+                                                                        : (size_t)2 * (BM + BN) * kRowStride;
   const int tiles_m = (M_rows + BM - 1) / BM;
   const int tiles_n = (C + BN - 1) / BN;
   // M tiles are walked in groups of 8 per K_r tile: a group's query rows (4 MiB in bf16) are what an XCD's L2

@@ -224,9 +224,10 @@ __global__ __launch_bounds__(kPlanWaves * 64) void gather_plan_kernel(const int3
 // every compute unit that hosts a copy wavefront slows the scoring workgroup beside it.  32 workgroups keep 128 KB in
 // flight, enough for the link, and leave the other compute units alone (scan under the copy 5.81 ms against 6.15 ms
 // with 2048 workgroups, 5.75 ms without a copy).
-constexpr int kCopyGridX = 16, kCopyGridY = 2;
+constexpr int kCopyGridX = 16, kCopyGridY = 2, kCopyThreads = 128;
+constexpr int kCopyRowLanes = 128;      // lanes that share a row (a 2 KB bf16 row is 128 lanes x 16 bytes)
 template <bool kFromDevice>
-__global__ __launch_bounds__(128) void gather_copy_kernel(const uint4* __restrict__ k_src, const uint4* __restrict__ v_src,
+__global__ __launch_bounds__(1024) void gather_copy_kernel(const uint4* __restrict__ k_src, const uint4* __restrict__ v_src,
                                                           const int32_t* __restrict__ plan, int32_t n_entries,
                                                           int32_t row_vecs, int64_t capacity_rows, uint4* k_dst,
                                                           uint4* v_dst) {
@@ -236,7 +237,8 @@ __global__ __launch_bounds__(128) void gather_copy_kernel(const uint4* __restric
   const int32_t n = e[1], dst0 = e[2], from = e[3];
   if ((from >= 0) != kFromDevice) continue;
   const int32_t src0 = kFromDevice ? from : e[0];
-  for (int r = blockIdx.y; r < n; r += gridDim.y) {
+  for (int r = blockIdx.y * (blockDim.x / kCopyRowLanes) + threadIdx.x / kCopyRowLanes; r < n;
+       r += gridDim.y * (blockDim.x / kCopyRowLanes)) {
     if ((int64_t)dst0 + r >= capacity_rows) break;
     if (kFromDevice && (int64_t)src0 + r >= capacity_rows) break;
     const uint4* ks = (kFromDevice ? k_dst : k_src) + ((int64_t)src0 + r) * row_vecs;
@@ -247,7 +249,7 @@ __global__ __launch_bounds__(128) void gather_copy_kernel(const uint4* __restric
     const __amdgpu_buffer_rsrc_t rvs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(vs), 0, row_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t rkd = __builtin_amdgcn_make_buffer_rsrc(kd, 0, row_bytes, 0x00020000);
     const __amdgpu_buffer_rsrc_t rvd = __builtin_amdgcn_make_buffer_rsrc(vd, 0, row_bytes, 0x00020000);
-    for (int off = threadIdx.x * 16; off < row_bytes; off += 128 * 16) {
+    for (int off = (threadIdx.x % kCopyRowLanes) * 16; off < row_bytes; off += kCopyRowLanes * 16) {
       const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(rks, off, 0, 0);
       const u32x4_t b = __builtin_amdgcn_raw_buffer_load_b128(rvs, off, 0, 0);
       __builtin_amdgcn_raw_buffer_store_b128(a, rkd, off, 0, 0);
@@ -289,13 +291,13 @@ extern "C" int msa_gather_kv_device(const msa_bank* bank, int32_t layer, const i
   MSA_LAUNCH_CHECK();
   const int32_t row_vecs = (int32_t)((size_t)bank->Hkv * bank->D * elem_bytes(bank->dtype) / 16);
   dim3 grid((unsigned)std::min(B * k, kCopyGridX), kCopyGridY);
-  gather_copy_kernel<false><<<grid, 128, 0, st>>>(static_cast<const uint4*>(bank->k_host[layer]),
+  gather_copy_kernel<false><<<grid, kCopyThreads, 0, st>>>(static_cast<const uint4*>(bank->k_host[layer]),
                                                   static_cast<const uint4*>(bank->v_host[layer]), plan, B * k, row_vecs,
                                                   out_capacity_chunks, static_cast<uint4*>(k_out),
                                                   static_cast<uint4*>(v_out));
   MSA_LAUNCH_CHECK();
   if (dedup) {
-    gather_copy_kernel<true><<<grid, 128, 0, st>>>(nullptr, nullptr, plan, B * k, row_vecs, out_capacity_chunks,
+    gather_copy_kernel<true><<<grid, kCopyThreads, 0, st>>>(nullptr, nullptr, plan, B * k, row_vecs, out_capacity_chunks,
                                                    static_cast<uint4*>(k_out), static_cast<uint4*>(v_out));
     MSA_LAUNCH_CHECK();
   }

@@ -196,34 +196,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   if constexpr (kStream) {
     tile_n = blockIdx.x;
     tile_m = 0;
-  }
-  // Position `vb` of the XCD-aware tile order -> (M tile, N tile); false for the padding positions of the order.
-  const int n_per_xcd = (tiles_n + 7) / 8, per_group = n_per_xcd * m_group;
-  const int total_vb = 8 * per_group * ((tiles_m + m_group - 1) / m_group);
-  auto decode_tile = [&](int vb, int& tm, int& tn) -> bool {
-    const int within = vb / 8;
+  } else {
+    const int n_per_xcd = (tiles_n + 7) / 8;
+    const int within = blockIdx.x / 8;
+    const int per_group = n_per_xcd * m_group;
     const int rem = within % per_group;
-    tn = (vb % 8) * n_per_xcd + rem / m_group;
-    tm = (within / per_group) * m_group + rem % m_group;
-    return tn < tiles_n && tm < tiles_m;
-  };
-  // The direct-to-LDS form is persistent: a workgroup takes positions blockIdx.x, + gridDim.x, ... (gridDim.x is a
-  // multiple of 8, so it stays on its XCD's range); next_tile() steps to the next real tile, or past the end.
-  auto next_tile = [&](int vb, int& tm, int& tn) -> int {
-    do vb += (int)gridDim.x;
-    while (vb < total_vb && !decode_tile(vb, tm, tn));
-    return vb;
-  };
-  int cur_vb = blockIdx.x;
-  if constexpr (!kStream) {
-    if (!decode_tile(cur_vb, tile_m, tile_n)) {
-      if (!score_tile_is_direct<T, BM, BN, kSets, kStream>()) return;
-      cur_vb = next_tile(cur_vb, tile_m, tile_n);
-      if (cur_vb >= total_vb) return;
-    }
+    tile_n = (blockIdx.x % 8) * n_per_xcd + rem / m_group;
+    tile_m = (within / per_group) * m_group + rem % m_group;
   }
   if (tile_n >= tiles_n || tile_m >= tiles_m) return;
-  int m0 = tile_m * BM, n0 = tile_n * BN;
+  const int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -369,16 +351,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     const int row = (wave * 4 + i) * 8 + dtl_row;
     return row * (int)row_bytes_g + ((dtl_slot ^ ((row >> 1) & 7)) * 16);
   };
-  __amdgpu_buffer_rsrc_t rsrc_la = rsrc_a;      // direct-to-LDS form: the query tile the loads have reached (K_r: rsrc_ld)
   auto dtl_load_a = [&](int stage, int kt) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      MSA_LOAD_TO_LDS(rsrc_la, lds + stage * kDtlStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes, 0);
+      MSA_LOAD_TO_LDS(rsrc_a, lds + stage * kDtlStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes, 0);
   };
   auto dtl_load_b = [&](int stage, int kt) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      MSA_LOAD_TO_LDS(rsrc_ld, lds + (2 + stage) * kDtlStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes,
+      MSA_LOAD_TO_LDS(rsrc_b, lds + (2 + stage) * kDtlStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes,
                       kStreamHint);
   };
   auto dtl_frags = [&](int sa, int sb, int sub, int slot) {
@@ -507,45 +488,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     // is exactly the wait the third stage exists to avoid.  The explicit vmcnt wait in front of it covers the tiles
     // the next step reads; the LDS reads of this step are drained by lgkmcnt(0).
     auto dtl_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
-    // Persistent: the workgroup's tiles form one sequence of K steps.  The query loads run one step ahead of the MFMAs
-    // and the K_r loads two, across tile boundaries, so a tile's first operands are in LDS before the previous tile's
-    // epilogue starts and the compute unit does not idle while a tile ramps up.  Each of the three positions (K_r
-    // loads, query loads, MFMAs) steps through the same tile list; a position that reaches a tile end takes over the
-    // tile of the position ahead of it (the K_r loads decode the list).
-    int tm_b = tile_m, tn_b = tile_n, vb_b = cur_vb, kt_b = 0;     // K_r loads
-    int tm_a = tile_m, tn_a = tile_n, kt_a = 0;                    // query loads
-    bool valid_a = true, valid_b = true;
-    auto set_rsrc_b = [&]() {
-      rsrc_ld = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(gb) + (int64_t)tn_b * BN * row_bytes_g, 0,
-                                                  (int)(min(BN, C - tn_b * BN) * row_bytes_g), 0x00020000);
-    };
-    auto set_rsrc_a = [&]() {
-      rsrc_la = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(ga) + (int64_t)tm_a * BM * row_bytes_g, 0,
-                                                  (int)(min(BM, M_rows - tm_a * BM) * row_bytes_g), 0x00020000);
-    };
-    auto advance_b = [&]() {
-      if (++kt_b == k_tiles) {
-        kt_b = 0;
-        vb_b = next_tile(vb_b, tm_b, tn_b);
-        valid_b = vb_b < total_vb;
-        if (valid_b) set_rsrc_b();
-      }
-    };
-    auto advance_a = [&]() {      // the K_r position is ahead by one step, so at a tile end it already names the next tile
-      if (++kt_a == k_tiles) {
-        kt_a = 0;
-        tm_a = tm_b; tn_a = tn_b;
-        valid_a = valid_b;                   // (at least two K tiles per tile: the K_r position is still in that tile)
-        if (valid_a) set_rsrc_a();
-      }
-    };
     dtl_load_a(0, 0);
-    advance_a();
     dtl_load_b(0, 0);
-    advance_b();
-    if (valid_b) {
-      dtl_load_b(1, kt_b);
-      advance_b();
+    if (k_tiles > 1) {
+      dtl_load_b(1, 1);
       __builtin_amdgcn_s_waitcnt(kWaitAllButNewestB);
     } else {
       __builtin_amdgcn_s_waitcnt(kWaitAll);
@@ -554,20 +500,15 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     dtl_frags(0, 0, 0, 0);
     fetch_rows();
     fetch_docs(n0);
-    // (the prefetches of a tile are issued before the tile loads of its first step: the waits, which count from the
-    // newest load, cover them)
-    int sa = 0, sb = 0, kt = 0;
-    for (;;) {
+    // the prefetches above are four more loads in flight behind tile 0: they are older than every later tile load,
+    // so the waits below, which count from the newest, cover them
+    int sb = 0;
+    for (int kt = 0; kt < k_tiles; ++kt) {
+      const int sa = kt & 1;
+      const bool more = kt + 1 < k_tiles, more2 = kt + 2 < k_tiles;
       const int sb1 = sb == 2 ? 0 : sb + 1, sb2 = sb1 == 2 ? 0 : sb1 + 1;
-      const bool more = valid_a, more2 = valid_b;    // a next step exists / its successor exists
-      if (more) {
-        dtl_load_a(sa ^ 1, kt_a);      // stage of the step before this one: its last reads were behind the previous barrier
-        advance_a();
-      }
-      if (more2) {
-        dtl_load_b(sb2, kt_b);
-        advance_b();
-      }
+      if (more) dtl_load_a(sa ^ 1, kt + 1);      // stage of tile kt - 1: its last reads were behind the previous barrier
+      if (more2) dtl_load_b(sb2, kt + 2);
 #pragma unroll
       for (int sub = 0; sub < kSub; ++sub) {
         if (sub + 1 < kSub) {
@@ -594,25 +535,9 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
           __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         }
       }
-      sa ^= 1;
       sb = sb1;
-      if (++kt == k_tiles) {
-        epilogue(n0);
-        if (!more) break;
-        kt = 0;
-        cur_vb = next_tile(cur_vb, tile_m, tile_n);
-        m0 = tile_m * BM;
-        n0 = tile_n * BN;
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
-        fetch_rows();
-        fetch_docs(n0);
-      }
     }
+    epilogue(n0);
   } else if constexpr (kStream) {
     // The workgroup's tiles form one sequence of steps (K tiles are even in number, so set tags and LDS buffers
     // alternate the same way in every tile); an epilogue sits where a tile's last step ends, with the next tile's
@@ -739,15 +664,6 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
       return MSA_EINVAL;
     }
     grid = std::min(tiles_n, compute_units() * std::max<int>(1, (int)(kLdsPerCu / lds)));
-  }
-  if (score_tile_is_direct<T, BM, BN, kSets, kStream>()) {
-    // persistent: one workgroup per compute unit (a multiple of 8 of them, so each stays on one XCD's range of the
-    // tile order) walks the positions blockIdx.x, + grid, ...; the loop needs at least two K tiles per tile
-    if (K * (int)sizeof(T) < 2 * kRowBytes) {
-      msa_set_error("score_gemm: K=%d too small for the direct-to-LDS form", K);
-      return MSA_EINVAL;
-    }
-    grid = std::min(grid, std::max(8, compute_units() / 8 * 8));
   }
   auto kern = score_gemm_kernel<T, BM, BN, WAVES_M, WAVES_N, kSets, kDocMax, kStream>;
   static std::atomic<int> lds_limit_raised{0};

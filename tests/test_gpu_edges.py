@@ -387,6 +387,23 @@ def test_score_epilogue_forms_on_a_dirty_workspace(ops, B, S):
     assert torch.isinf(s.cpu()[~live]).all()
 
 
+@pytest.mark.parametrize("B,S,Hkv", [(24, 100, 4), (9, 250, 8), (40, 33, 2)])
+def test_scores_many_query_tiles(ops, B, S, Hkv):
+    """More than eight 256-row query tiles (they are then walked in groups of eight per K_r tile, the last group
+    ragged), a ragged last K_r tile, and depths of 4 to 16 K steps per tile through the large-tile form; a masked
+    tail of one query and a query whose padded rows end inside a tile."""
+    say(f"many query tiles B={B} S={S} Hkv={Hkv}")
+    bank, kr, dco, _ = _bank(ops, [5, 1, 8, 2, 11, 3] * 37, Hkv, torch.bfloat16, 950 + B)
+    q = _randn((B, S, 4 * Hkv, 128), 951 + S, torch.bfloat16)
+    mask = torch.ones(B, S, dtype=torch.bool)
+    mask[1, S // 3:] = False
+    got = ops.chunk_scores(bank, 0, q.cuda(), mask.cuda()).cpu()
+    want = cf.chunk_scores(q, mask, kr, "cosine")
+    assert cf.rel_err(got, want) < 1e-2
+    s_, d, _ = ops.route_topk(bank, 0, q.cuda(), mask.cuda(), "cosine", 1.0, 8)
+    assert not cf.topk_acceptable(cf.doc_scores(want, dco), d.cpu().long(), 8)
+
+
 @pytest.mark.parametrize("topk", [1, 16, 64])
 def test_topk_windows_long_documents_and_filtering(ops, topk):
     """Documents longer than the top-k kernel's LDS window (2044 keys) among one-chunk documents, more documents

@@ -317,8 +317,9 @@ def main():
     ap.add_argument("--seq", type=int, default=128)
     ap.add_argument("--host-kv-layers", type=int, default=2,
                     help="distinct pinned host K/V layer buffers (routed layers share them round-robin)")
-    ap.add_argument("--gather", choices=["device", "memcpy"], default="device",
+    ap.add_argument("--gather", choices=["device", "fused", "memcpy"], default="fused",
                     help="device: plan + copy kernels read the pinned bank directly, no ids on the host; "
+                         "fused: the same plan + copy inside the next layer's scan launch (one workgroup of it); "
                          "memcpy: ids to the host, one hipMemcpyAsync per document run")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-sweep", action="store_true")
@@ -431,6 +432,17 @@ def main():
                                             gv[li & 1].data_ptr(), cap_chunks, cu_dev[li].data_ptr(), gws.data_ptr(),
                                             gws.numel(), side.cuda_stream), "msa_gather_kv_device")
 
+    def route_fused(li, prev):             # layer li's scan; one of its workgroups fetches layer prev's selection
+        t_r = time.perf_counter()
+        _lib.check(lib.msa_route_topk_gather(bank.handle, li, qs[li].data_ptr(), None, B, S, HQ, _lib.MODE_COSINE, 1.0,
+                                             TOPK, scores[li].data_ptr(), docs[li].data_ptr(), gids[li].data_ptr(),
+                                             ws.data_ptr(), ws.numel(), prev, docs[prev].data_ptr(), B, TOPK,
+                                             gk[prev & 1].data_ptr(), gv[prev & 1].data_ptr(), cap_chunks,
+                                             cu_dev[prev].data_ptr(), gws.data_ptr(), gws.numel(),
+                                             main_stream.cuda_stream), "msa_route_topk_gather")
+        scored[li].record(main_stream)
+        host_s["route_calls"] += time.perf_counter() - t_r
+
     pending = [None]                  # layer whose selected K / V have not been fetched yet
 
     def step():
@@ -438,6 +450,14 @@ def main():
             for li in range(L):
                 route(li)
                 gather_device(li)          # runs on the side stream under the next layer's scan
+            return
+        if args.gather == "fused":
+            for li in range(L):
+                if pending[0] is None:
+                    route(li)
+                else:
+                    route_fused(li, pending[0])
+                pending[0] = li
             return
         for li in range(L):
             route(li)                      # layer li is being scored ...
@@ -447,7 +467,7 @@ def main():
 
     def drain():                           # the last batch's last layer has no scan left to hide under
         if pending[0] is not None:
-            gather(pending[0])
+            gather_device(pending[0]) if args.gather == "fused" else gather(pending[0])
             pending[0] = None
 
     for _ in range(args.warmup):
@@ -483,7 +503,7 @@ def main():
     wk, wv, wcu, _ = cf.gather_selected(host_k[last % n_host], host_v[last % n_host], doc_chunk_off,
                                         torch.as_tensor(wants[last]))
     n_sel = int(wcu[-1])
-    if args.gather == "device":
+    if args.gather in ("device", "fused"):
         sel_chunks = [int(c[-1]) for c in cu_dev]
     if n_sel != sel_chunks[last] or not torch.equal(gk[last & 1][:n_sel].cpu(), wk) or \
             not torch.equal(gv[last & 1][:n_sel].cpu(), wv):

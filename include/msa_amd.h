@@ -162,6 +162,22 @@ int msa_gather_kv_device(const msa_bank* bank, int32_t layer, const int32_t* doc
                          int32_t k, void* k_out, void* v_out, int64_t out_capacity_chunks,
                          int32_t* cu_sel, void* workspace, size_t workspace_bytes, void* stream);
 
+/* msa_route_topk of one layer with the msa_gather_kv_device of an earlier selection inside the same launch (typically
+ * the previous router layer's documents: the reference fetches a layer's K / V right after routing it,
+ * src/msa_service.py:1203-1262; a pipelined caller can let that fetch ride under the next layer's scan).  One
+ * workgroup of the scan copies the rows from the pinned host bank while the others score, so the copy takes a compute
+ * unit of its own instead of slowing scoring workgroups that a separate copy kernel's wavefronts would sit beside.
+ * Arguments and results are those of the two calls (gather_* name the gathered layer and its selection [gather_B,
+ * gather_k]; gather_workspace is msa_gather_device_workspace_bytes(gather_B, gather_k)).  The large-tile form of the
+ * scan (bf16, more than 128 padded query rows) carries the copy; for other shapes the gather's own kernels run on the
+ * stream in front of the scan, with the same results. */
+int msa_route_topk_gather(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B, int32_t S,
+                          int32_t Hq, int32_t mode, float scale, int32_t topk, float* scores_out, int32_t* doc_out,
+                          int64_t* doc_global_out, void* workspace, size_t workspace_bytes, int32_t gather_layer,
+                          const int32_t* gather_doc_sel, int32_t gather_B, int32_t gather_k, void* k_out, void* v_out,
+                          int64_t out_capacity_chunks, int32_t* cu_sel, void* gather_workspace,
+                          size_t gather_workspace_bytes, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Context assembly.  Replaces the ragged scatter of src/msa/memory_sparse_attention.py:282-329
  * and the compact cache of :344-351: for every sample b writes

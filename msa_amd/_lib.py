@@ -38,6 +38,8 @@ SIGNATURES = {
     "msa_gather_kv": (C.c_int, [_vp, _i32, _vp, _i32, _i32, _vp, _vp, _i64, _vp]),
     "msa_gather_device_workspace_bytes": (_sz, [_i32, _i32]),
     "msa_gather_kv_device": (C.c_int, [_vp, _i32, _vp, _i32, _i32, _vp, _vp, _i64, _vp, _vp, _sz, _vp]),
+    "msa_route_topk_gather": (C.c_int, [_vp, _i32, _vp, _vp, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _vp, _vp, _vp, _sz,
+                                        _i32, _vp, _i32, _i32, _vp, _vp, _i64, _vp, _vp, _sz, _vp]),
     "msa_assemble_context": (C.c_int, [_vp, _vp, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _vp,
                                        _vp, _i32, _vp, _vp]),
     "msa_cache_append": (C.c_int, [_vp, _vp, _i32, _i32, _i32, _i32, _vp, _vp, _i32, _vp, _vp]),

@@ -7,9 +7,7 @@
 #include <unordered_map>
 #include <vector>
 
-#include "common.h"
-
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+#include "gather_device.h"
 
 namespace {
 
@@ -124,9 +122,9 @@ extern "C" int msa_gather_kv(const msa_bank* bank, int32_t layer, const int32_t*
 namespace {
 
 constexpr int kPlanWaves = 4;
-constexpr int kPlanInts = 4;            // ints per plan entry
-constexpr int kDedupMaxEntries = 2048;  // batch-wide de-duplication runs while B * k fits this many LDS slots
-constexpr int32_t kNoDoc = 0x7fffffff;
+using msa_gather::kPlanInts;
+using msa_gather::kDedupMaxEntries;
+using msa_gather::kCopyRowLanes;
 
 __global__ __launch_bounds__(kPlanWaves * 64) void gather_plan_kernel(const int32_t* __restrict__ doc_sel,
                                                                       const int32_t* __restrict__ doc_chunk_off,
@@ -134,129 +132,26 @@ __global__ __launch_bounds__(kPlanWaves * 64) void gather_plan_kernel(const int3
                                                                       int32_t capacity_rows, int32_t dedup,
                                                                       int32_t* __restrict__ cu_sel,
                                                                       int32_t* __restrict__ plan /* [B*k][4] */) {
-  extern __shared__ int32_t smem[];            // totals [B + 1] | sorted documents [B * k] | destination rows [B * k]
-  int32_t* totals = smem;
-  int32_t* s_doc = smem + (B + 1);
-  int32_t* s_dst = s_doc + (dedup ? B * k : 0);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  // pass 1 and 2 share this per-sample routine: sorted unique documents in lanes, chunk counts, in-sample offsets
-  auto sample = [&](int b, int32_t& d_out, int32_t& n_out, int32_t& off_out) -> int32_t {
-    int32_t d = kNoDoc;
-    if (lane < k) {
-      const int32_t x = doc_sel[(int64_t)b * k + lane];
-      if (x >= 0 && x < n_docs) d = x;
-    }
-#pragma unroll
-    for (int kk = 2; kk <= 64; kk <<= 1)
-#pragma unroll
-      for (int j = kk >> 1; j > 0; j >>= 1) {            // ascending bitonic sort
-        const int32_t o = __shfl_xor(d, j);
-        const bool asc = (lane & kk) == 0, lower = (lane & j) == 0;
-        d = (lower == asc) ? min(d, o) : max(d, o);
-      }
-    const int32_t prev = __shfl_up(d, 1);
-    const bool keep = d != kNoDoc && (lane == 0 || prev != d);
-    int32_t n = keep ? doc_chunk_off[d + 1] - doc_chunk_off[d] : 0;
-    int32_t incl = n;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const int32_t t = __shfl_up(incl, o);
-      if (lane >= o) incl += t;
-    }
-    d_out = keep ? d : -1; n_out = n; off_out = incl - n;
-    return __shfl(incl, 63);
-  };
-  for (int b = wave; b < B; b += kPlanWaves) {
-    int32_t d, n, off;
-    const int32_t total = sample(b, d, n, off);
-    if (lane == 0) totals[b + 1] = total;
-  }
-  if (threadIdx.x == 0) totals[0] = 0;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int32_t run = 0;
-    for (int b = 0; b < B; ++b) { run += totals[b + 1]; totals[b + 1] = run; }
-  }
-  __syncthreads();
-  // rows past the output's capacity are never written by the copy kernel: the prefix sums stop there too, so a
-  // consumer of cu_sel never addresses a row that was not filled
-  for (int i = threadIdx.x; i <= B; i += kPlanWaves * 64) cu_sel[i] = min(totals[i], capacity_rows);
-  for (int b = wave; b < B; b += kPlanWaves) {
-    int32_t d, n, off;
-    sample(b, d, n, off);
-    if (lane < k) {
-      int32_t* e = plan + ((int64_t)b * k + lane) * kPlanInts;
-      e[0] = d >= 0 ? doc_chunk_off[d] : 0;
-      e[1] = n;
-      e[2] = totals[b] + off;
-      e[3] = -1;
-      if (dedup) {                               // documents dropped as duplicates inside the sample sort last
-        s_doc[b * k + lane] = d >= 0 ? d : kNoDoc;
-        s_dst[b * k + lane] = totals[b] + off;
-      }
-    }
-  }
-  if (!dedup) return;                            // uniform over the workgroup
-  __syncthreads();
-  // an entry whose document an earlier sample also holds copies from that sample's rows instead of the host.
-  // s_doc rows are ascending except that in-sample duplicates were replaced by kNoDoc in place, so the search
-  // below is linear over the k slots (k <= 64).
-  for (int i = threadIdx.x; i < B * k; i += kPlanWaves * 64) {
-    const int32_t d = s_doc[i];
-    if (d == kNoDoc) continue;
-    const int b = i / k;
-    int32_t from = -1;
-    for (int b2 = 0; b2 < b && from < 0; ++b2)
-      for (int j = 0; j < k; ++j)
-        if (s_doc[b2 * k + j] == d) { from = s_dst[b2 * k + j]; break; }
-    if (from >= 0) plan[(int64_t)i * kPlanInts + 3] = from;
-  }
+  extern __shared__ int32_t smem[];
+  msa_gather::plan_body(doc_sel, doc_chunk_off, n_docs, B, k, capacity_rows, dedup, cu_sel, plan, smem, (int)threadIdx.x,
+                        (int)blockDim.x);
 }
 
-// grid.x = plan entry, grid.y = row group; 128 lanes move one row of K and of V per step.
-// kFromDevice = false: entries without an earlier copy, rows read from the pinned host bank;
-// kFromDevice = true: the others, rows read from the earlier copy inside the output itself.
-// The kernel stays within 16 vector registers (rows travel through buffer resources, i.e. scalar addresses and one
-// vector offset): a scoring workgroup of the routing scan takes 496 of a SIMD's 512, and only a wavefront that fits
-// beside it runs under the scan instead of taking a compute unit's turn between two of its workgroups (the copy is
-// PCIe-bound: it needs residency, not registers).
+// grid.x strides over plan entries, grid.y and the workgroup's groups of 128 lanes over an entry's rows.
 // Few workgroups: PCIe reads are slow to return and a compute unit's memory pipeline serves its wavefronts in order, so
 // every compute unit that hosts a copy wavefront slows the scoring workgroup beside it.  32 workgroups keep 128 KB in
 // flight, enough for the link, and leave the other compute units alone (scan under the copy 5.81 ms against 6.15 ms
 // with 2048 workgroups, 5.75 ms without a copy).
 constexpr int kCopyGridX = 16, kCopyGridY = 2, kCopyThreads = 128;
-constexpr int kCopyRowLanes = 128;      // lanes that share a row (a 2 KB bf16 row is 128 lanes x 16 bytes)
 template <bool kFromDevice>
 __global__ __launch_bounds__(1024) void gather_copy_kernel(const uint4* __restrict__ k_src, const uint4* __restrict__ v_src,
                                                           const int32_t* __restrict__ plan, int32_t n_entries,
                                                           int32_t row_vecs, int64_t capacity_rows, uint4* k_dst,
                                                           uint4* v_dst) {
-  const int row_bytes = row_vecs * 16;
-  for (int ent = blockIdx.x; ent < n_entries; ent += gridDim.x) {
-  const int32_t* e = plan + (int64_t)ent * kPlanInts;
-  const int32_t n = e[1], dst0 = e[2], from = e[3];
-  if ((from >= 0) != kFromDevice) continue;
-  const int32_t src0 = kFromDevice ? from : e[0];
-  for (int r = blockIdx.y * (blockDim.x / kCopyRowLanes) + threadIdx.x / kCopyRowLanes; r < n;
-       r += gridDim.y * (blockDim.x / kCopyRowLanes)) {
-    if ((int64_t)dst0 + r >= capacity_rows) break;
-    if (kFromDevice && (int64_t)src0 + r >= capacity_rows) break;
-    const uint4* ks = (kFromDevice ? k_dst : k_src) + ((int64_t)src0 + r) * row_vecs;
-    const uint4* vs = (kFromDevice ? v_dst : v_src) + ((int64_t)src0 + r) * row_vecs;
-    uint4* kd = k_dst + ((int64_t)dst0 + r) * row_vecs;
-    uint4* vd = v_dst + ((int64_t)dst0 + r) * row_vecs;
-    const __amdgpu_buffer_rsrc_t rks = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(ks), 0, row_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rvs = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(vs), 0, row_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rkd = __builtin_amdgcn_make_buffer_rsrc(kd, 0, row_bytes, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rvd = __builtin_amdgcn_make_buffer_rsrc(vd, 0, row_bytes, 0x00020000);
-    for (int off = (threadIdx.x % kCopyRowLanes) * 16; off < row_bytes; off += kCopyRowLanes * 16) {
-      const u32x4_t a = __builtin_amdgcn_raw_buffer_load_b128(rks, off, 0, 0);
-      const u32x4_t b = __builtin_amdgcn_raw_buffer_load_b128(rvs, off, 0, 0);
-      __builtin_amdgcn_raw_buffer_store_b128(a, rkd, off, 0, 0);
-      __builtin_amdgcn_raw_buffer_store_b128(b, rvd, off, 0, 0);
-    }
-  }
-  }
+  const int groups = (int)blockDim.x / kCopyRowLanes;
+  msa_gather::copy_body<kFromDevice>(k_src, v_src, plan, n_entries, row_vecs, capacity_rows, k_dst, v_dst, (int)blockIdx.x,
+                                     (int)gridDim.x, (int)blockIdx.y * groups + (int)threadIdx.x / kCopyRowLanes,
+                                     (int)gridDim.y * groups, (int)threadIdx.x % kCopyRowLanes);
 }
 
 }  // namespace
@@ -285,7 +180,7 @@ extern "C" int msa_gather_kv_device(const msa_bank* bank, int32_t layer, const i
   int32_t* plan = static_cast<int32_t*>(workspace);
   const int32_t dedup = B > 1 && B * k <= kDedupMaxEntries ? 1 : 0;
   const int32_t cap32 = (int32_t)std::min<int64_t>(out_capacity_chunks, 0x7fffffff);
-  const size_t lds = (size_t)(B + 1 + (dedup ? 2 * B * k : 0)) * sizeof(int32_t);
+  const size_t lds = msa_gather::plan_lds_ints(B, k, dedup) * sizeof(int32_t);
   gather_plan_kernel<<<1, kPlanWaves * 64, lds, st>>>(doc_sel, bank->doc_chunk_off_dev, (int32_t)bank->n_docs, B, k,
                                                       cap32, dedup, cu_sel, plan);
   MSA_LAUNCH_CHECK();

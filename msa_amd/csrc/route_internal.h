@@ -5,6 +5,21 @@
 constexpr int kTopkMax = 64;          // width of every candidate list (one wavefront)
 constexpr int kTopkDocsPerBlock = 2048;   // documents per top-k workgroup: 43 workgroups per query at 87k documents
 
+// A K / V gather (msa_gather_kv_device's work) that rides along with a routing scan: one workgroup of the scan's launch
+// runs it while the others score.  active = 0: none.
+struct GatherJob {
+  const int32_t* doc_sel;        // [B, k] selected documents (device)
+  const int32_t* doc_chunk_off;  // bank table (device)
+  int32_t* cu_sel;               // [B + 1] out
+  int32_t* plan;                 // [B * k][4] scratch
+  const uint4* k_src;            // pinned host K / V of the gathered layer
+  const uint4* v_src;
+  uint4* k_dst;                  // [capacity_rows, Hkv, D] out
+  uint4* v_dst;
+  int64_t capacity_rows;
+  int32_t n_docs, B, k, dedup, row_vecs, active;
+};
+
 struct RouteWorkspace {
   int32_t S_pad;        // query tokens padded to a multiple of 32 (one MFMA row block never spans two queries)
   int32_t M_rows;       // B * S_pad
@@ -26,7 +41,9 @@ RouteWorkspace route_workspace_layout(int32_t B, int32_t S, int32_t Hkv, int32_t
 
 // Runs prologue + scoring GEMM on `st`; on success the keys (per document with doc_max, else per chunk) sit at
 // layout_out->off_key and score = key_to_f32(key) * (*mul_out); key 0 = nothing scored.
+// `job`: an optional gather to run inside the scan's launch; *job_taken tells whether the launch form could carry it
+// (only the large-tile form can; the caller runs the gather's own kernels otherwise).
 int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
                          int32_t S, int32_t Hq, int32_t mode, float scale, bool doc_max, void* workspace,
                          size_t workspace_bytes, hipStream_t st, RouteWorkspace* layout_out, float* mul_out,
-                         const char* who);
+                         const char* who, const GatherJob* job = nullptr, bool* job_taken = nullptr);

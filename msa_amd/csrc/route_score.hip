@@ -12,7 +12,8 @@
 #include <mutex>
 #include <type_traits>
 
-#include "common.h"
+#include "gather_device.h"
+#include "route_internal.h"
 
 namespace {
 
@@ -178,7 +179,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     uint32_t* __restrict__ out_key,      // [B, n_docs] or [B, C], zeroed
     const int32_t* __restrict__ chunk_doc,  // [C] document of every chunk (kDocMax)
     int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t tiles_m, int32_t tiles_n,
-    int32_t m_group, int32_t n_docs) {
+    int32_t m_group, int32_t n_docs, GatherJob job) {
   constexpr int kThreads = WAVES_M * WAVES_N * 64;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -196,16 +197,69 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
   if constexpr (kStream) {
     tile_n = blockIdx.x;
     tile_m = 0;
-  } else {
-    const int n_per_xcd = (tiles_n + 7) / 8;
-    const int within = blockIdx.x / 8;
-    const int per_group = n_per_xcd * m_group;
+  }
+  // Position `vb` of the XCD-aware tile order -> (M tile, N tile); false for the padding positions of the order.
+  const int n_per_xcd = (tiles_n + 7) / 8, per_group = n_per_xcd * m_group;
+  auto decode_tile = [&](int vb, int& tm, int& tn) -> bool {
+    const int within = vb / 8;
     const int rem = within % per_group;
-    tile_n = (blockIdx.x % 8) * n_per_xcd + rem / m_group;
-    tile_m = (within / per_group) * m_group + rem % m_group;
+    tn = (vb % 8) * n_per_xcd + rem / m_group;
+    tm = (within / per_group) * m_group + rem % m_group;
+    return tn < tiles_n && tm < tiles_m;
+  };
+  // The direct-to-LDS form is persistent: the workgroups of an XCD share the XCD's tiles, position p of its dense
+  // order naming (group of M tiles by group) an N tile of the XCD's range with the group's M tiles side by side;
+  // workgroup w of the XCD takes positions w, w + (workgroups of the XCD), ...  With a gather job attached the last
+  // workgroup of the launch does not score: it fetches the K / V rows of an earlier selection from the pinned host bank
+  // while the others scan (a copy on a compute unit of its own disturbs no scoring workgroup, and no scoring
+  // workgroup's share of tiles depends on where a separate copy kernel's wavefronts would have landed).  The XCDs'
+  // N ranges are sized in proportion to their scoring workgroups.
+  const int xcd = blockIdx.x % 8, wg_in_xcd = blockIdx.x / 8;
+  const int wgs_all = (int)gridDim.x, scoring_wgs = wgs_all - (job.active ? 1 : 0);
+  const bool is_copy_wg = kDtl && job.active && (int)blockIdx.x == wgs_all - 1;
+  auto wgs_before = [&](int x) {      // scoring workgroups on XCDs 0 .. x - 1 (workgroup b sits on XCD b % 8)
+    int n = 0;
+    for (int y = 0; y < x; ++y) n += (scoring_wgs - y + 7) / 8;
+    return n;
+  };
+  const int wgs_in_xcd = (scoring_wgs - xcd + 7) / 8;
+  const int n_begin = (int)((int64_t)tiles_n * wgs_before(xcd) / max(scoring_wgs, 1));
+  const int n_stop = (int)((int64_t)tiles_n * (wgs_before(xcd) + wgs_in_xcd) / max(scoring_wgs, 1));
+  const int n_in_xcd = n_stop - n_begin;
+  const int dense_total = n_in_xcd * tiles_m;
+  auto decode_dense = [&](int p, int& tm, int& tn) {
+    const int full_groups = tiles_m / m_group, full = full_groups * n_in_xcd * m_group;
+    int g, rem, mg;
+    if (p < full) { g = p / (n_in_xcd * m_group); rem = p - g * n_in_xcd * m_group; mg = m_group; }
+    else { g = full_groups; rem = p - full; mg = tiles_m - full_groups * m_group; }
+    tn = n_begin + rem / mg;
+    tm = g * m_group + rem % mg;
+  };
+  if constexpr (kDtl) {
+    if (is_copy_wg) {
+      // plan (sorted, de-duplicated selection -> copy entries), host rows, then the documents an earlier sample
+      // already fetched; the workgroup barriers order the three steps' memory
+      msa_gather::plan_body(job.doc_sel, job.doc_chunk_off, job.n_docs, job.B, job.k,
+                            (int32_t)min(job.capacity_rows, (int64_t)0x7fffffff), job.dedup,
+                            job.cu_sel, job.plan, reinterpret_cast<int32_t*>(lds), (int)threadIdx.x, kThreads);
+      __syncthreads();
+      const int groups = kThreads / msa_gather::kCopyRowLanes;
+      const int group = (int)threadIdx.x / msa_gather::kCopyRowLanes, lane_in_row = (int)threadIdx.x % msa_gather::kCopyRowLanes;
+      msa_gather::copy_body<false, 8>(job.k_src, job.v_src, job.plan, job.B * job.k, job.row_vecs, job.capacity_rows,
+                                   job.k_dst, job.v_dst, 0, 1, group, groups, lane_in_row);
+      __syncthreads();
+      if (job.dedup)
+        msa_gather::copy_body<true, 8>(nullptr, nullptr, job.plan, job.B * job.k, job.row_vecs, job.capacity_rows,
+                                    job.k_dst, job.v_dst, 0, 1, group, groups, lane_in_row);
+      return;
+    }
+    if (wg_in_xcd >= dense_total) return;
+    decode_dense(wg_in_xcd, tile_m, tile_n);
+  } else if constexpr (!kStream) {
+    if (!decode_tile(blockIdx.x, tile_m, tile_n)) return;
   }
   if (tile_n >= tiles_n || tile_m >= tiles_m) return;
-  const int m0 = tile_m * BM, n0 = tile_n * BN;
+  int m0 = tile_m * BM, n0 = tile_n * BN;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
@@ -351,15 +405,16 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     const int row = (wave * 4 + i) * 8 + dtl_row;
     return row * (int)row_bytes_g + ((dtl_slot ^ ((row >> 1) & 7)) * 16);
   };
+  __amdgpu_buffer_rsrc_t rsrc_la = rsrc_a;      // direct-to-LDS form: the query tile the loads have reached (K_r: rsrc_ld)
   auto dtl_load_a = [&](int stage, int kt) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      MSA_LOAD_TO_LDS(rsrc_a, lds + stage * kDtlStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes, 0);
+      MSA_LOAD_TO_LDS(rsrc_la, lds + stage * kDtlStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes, 0);
   };
   auto dtl_load_b = [&](int stage, int kt) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      MSA_LOAD_TO_LDS(rsrc_b, lds + (2 + stage) * kDtlStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes,
+      MSA_LOAD_TO_LDS(rsrc_ld, lds + (2 + stage) * kDtlStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes,
                       kStreamHint);
   };
   auto dtl_frags = [&](int sa, int sb, int sub, int slot) {
@@ -488,10 +543,48 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     // is exactly the wait the third stage exists to avoid.  The explicit vmcnt wait in front of it covers the tiles
     // the next step reads; the LDS reads of this step are drained by lgkmcnt(0).
     auto dtl_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    // Persistent: the workgroup's tiles form one sequence of K steps.  The query loads run one step ahead of the MFMAs
+    // and the K_r loads two, across tile boundaries, so a tile's first operands are in LDS before the previous tile's
+    // epilogue starts and the compute unit does not idle while a tile ramps up.  Each of the three positions (K_r
+    // loads, query loads, MFMAs) steps through the same tile list; a position that reaches a tile end takes over the
+    // tile of the position ahead of it (the K_r loads decode the list).
+    int tm_b = tile_m, tn_b = tile_n, p_b = wg_in_xcd, kt_b = 0;   // K_r loads
+    int tm_a = tile_m, tn_a = tile_n, kt_a = 0;                    // query loads
+    bool valid_a = true, valid_b = true;
+    auto set_rsrc_b = [&]() {
+      rsrc_ld = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(gb) + (int64_t)tn_b * BN * row_bytes_g, 0,
+                                                  (int)(min(BN, C - tn_b * BN) * row_bytes_g), 0x00020000);
+    };
+    auto set_rsrc_a = [&]() {
+      rsrc_la = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(ga) + (int64_t)tm_a * BM * row_bytes_g, 0,
+                                                  (int)(min(BM, M_rows - tm_a * BM) * row_bytes_g), 0x00020000);
+    };
+    auto advance_b = [&]() {
+      if (++kt_b == k_tiles) {
+        kt_b = 0;
+        p_b += wgs_in_xcd;
+        valid_b = p_b < dense_total;
+        if (valid_b) {
+          decode_dense(p_b, tm_b, tn_b);
+          set_rsrc_b();
+        }
+      }
+    };
+    auto advance_a = [&]() {      // the K_r position is ahead by one step, so at a tile end it already names the next tile
+      if (++kt_a == k_tiles) {
+        kt_a = 0;
+        tm_a = tm_b; tn_a = tn_b;
+        valid_a = valid_b;                   // (at least two K tiles per tile: the K_r position is still in that tile)
+        if (valid_a) set_rsrc_a();
+      }
+    };
     dtl_load_a(0, 0);
+    advance_a();
     dtl_load_b(0, 0);
-    if (k_tiles > 1) {
-      dtl_load_b(1, 1);
+    advance_b();
+    if (valid_b) {
+      dtl_load_b(1, kt_b);
+      advance_b();
       __builtin_amdgcn_s_waitcnt(kWaitAllButNewestB);
     } else {
       __builtin_amdgcn_s_waitcnt(kWaitAll);
@@ -500,15 +593,20 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     dtl_frags(0, 0, 0, 0);
     fetch_rows();
     fetch_docs(n0);
-    // the prefetches above are four more loads in flight behind tile 0: they are older than every later tile load,
-    // so the waits below, which count from the newest, cover them
-    int sb = 0;
-    for (int kt = 0; kt < k_tiles; ++kt) {
-      const int sa = kt & 1;
-      const bool more = kt + 1 < k_tiles, more2 = kt + 2 < k_tiles;
+    // (the prefetches of a tile are issued before the tile loads of its first step: the waits, which count from the
+    // newest load, cover them)
+    int sa = 0, sb = 0, kt = 0;
+    for (;;) {
       const int sb1 = sb == 2 ? 0 : sb + 1, sb2 = sb1 == 2 ? 0 : sb1 + 1;
-      if (more) dtl_load_a(sa ^ 1, kt + 1);      // stage of tile kt - 1: its last reads were behind the previous barrier
-      if (more2) dtl_load_b(sb2, kt + 2);
+      const bool more = valid_a, more2 = valid_b;    // a next step exists / its successor exists
+      if (more) {
+        dtl_load_a(sa ^ 1, kt_a);      // stage of the step before this one: its last reads were behind the previous barrier
+        advance_a();
+      }
+      if (more2) {
+        dtl_load_b(sb2, kt_b);
+        advance_b();
+      }
 #pragma unroll
       for (int sub = 0; sub < kSub; ++sub) {
         if (sub + 1 < kSub) {
@@ -535,9 +633,26 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
           __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         }
       }
+      sa ^= 1;
       sb = sb1;
+      if (++kt == k_tiles) {
+        epilogue(n0);
+        if (!more) break;
+        kt = 0;
+        tile_m = tm_a;      // the query loads entered the next tile during this tile's last step
+        tile_n = tn_a;
+        m0 = tile_m * BM;
+        n0 = tile_n * BN;
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        fetch_rows();
+        fetch_docs(n0);
+      }
     }
-    epilogue(n0);
   } else if constexpr (kStream) {
     // The workgroup's tiles form one sequence of steps (K tiles are even in number, so set tags and LDS buffers
     // alternate the same way in every tile); an epilogue sits where a tile's last step ends, with the next tile's
@@ -647,7 +762,8 @@ int compute_units() {
 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool kDocMax, bool kStream>
 int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key, const int32_t* chunk_doc,
-                int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t n_docs, hipStream_t st) {
+                int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t n_docs, hipStream_t st,
+                const GatherJob* job, bool* job_taken) {
   const size_t lds = score_tile_is_direct<T, BM, BN, kSets, kStream>() ? (size_t)kDtlLdsBytes
                                                                         : (size_t)2 * (BM + BN) * kRowStride;
   const int tiles_m = (M_rows + BM - 1) / BM;
@@ -665,6 +781,21 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
     }
     grid = std::min(tiles_n, compute_units() * std::max<int>(1, (int)(kLdsPerCu / lds)));
   }
+  GatherJob no_job{};
+  const GatherJob* the_job = &no_job;
+  if (score_tile_is_direct<T, BM, BN, kSets, kStream>()) {
+    // persistent: one workgroup per compute unit walks its XCD's tiles; with a gather job the last one copies instead.
+    // The loop needs at least two K tiles per tile.
+    if (K * (int)sizeof(T) < 2 * kRowBytes) {
+      msa_set_error("score_gemm: K=%d too small for the direct-to-LDS form", K);
+      return MSA_EINVAL;
+    }
+    grid = std::max(16, compute_units() / 8 * 8);
+    if (job != nullptr && job->active) {
+      the_job = job;
+      if (job_taken) *job_taken = true;
+    }
+  }
   auto kern = score_gemm_kernel<T, BM, BN, WAVES_M, WAVES_N, kSets, kDocMax, kStream>;
   static std::atomic<int> lds_limit_raised{0};
   MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(kern), (int)lds));
@@ -676,7 +807,7 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
   if (slot >= 0) MSA_HIP(hipEventRecord(g_timer.start[slot], st));
   kern<<<grid, WAVES_M * WAVES_N * 64, lds, st>>>(static_cast<const T*>(qs), static_cast<const T*>(kr), row_bits, out_key,
                                                   chunk_doc, M_rows, C, K, blocks_per_query, tiles_m, tiles_n, m_group,
-                                                  n_docs);
+                                                  n_docs, *the_job);
   MSA_LAUNCH_CHECK();
   if (slot >= 0) MSA_HIP(hipEventRecord(g_timer.stop[slot], st));
   return MSA_OK;
@@ -690,14 +821,14 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
 template <bool kDocMax>
 int launch_gemm_for(int32_t dtype, const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key,
                     const int32_t* chunk_doc, int32_t M_rows, int32_t C, int32_t K, int32_t bpq, int32_t n_docs,
-                    hipStream_t st) {
+                    hipStream_t st, const GatherJob* job, bool* job_taken) {
   if (dtype != MSA_BF16)
-    return launch_gemm<float, 128, 128, 2, 2, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
+    return launch_gemm<float, 128, 128, 2, 2, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken);
   if (M_rows <= 64)
-    return launch_gemm<bf16_t, 64, 128, 2, 2, 2, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
+    return launch_gemm<bf16_t, 64, 128, 2, 2, 2, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken);
   if (M_rows <= 128)
-    return launch_gemm<bf16_t, 128, 384, 2, 4, 1, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
-  return launch_gemm<bf16_t, 256, 256, 2, 4, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
+    return launch_gemm<bf16_t, 128, 384, 2, 4, 1, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken);
+  return launch_gemm<bf16_t, 256, 256, 2, 4, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken);
 }
 
 }  // namespace
@@ -705,7 +836,6 @@ int launch_gemm_for(int32_t dtype, const void* qs, const void* kr, const uint32_
 // ------------------------------------------------------------------------------------------
 // Workspace layout (shared with topk.hip through route_internal.h)
 // ------------------------------------------------------------------------------------------
-#include "route_internal.h"
 
 RouteWorkspace route_workspace_layout(int32_t B, int32_t S, int32_t Hkv, int32_t D, int64_t plane_cols, int64_t n_docs,
                                       int32_t dtype) {
@@ -779,7 +909,8 @@ extern "C" size_t msa_route_topk_workspace_bytes(int32_t B, int32_t S, int32_t H
 int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
                          int32_t S, int32_t Hq, int32_t mode, float scale, bool doc_max, void* workspace,
                          size_t workspace_bytes, hipStream_t st, RouteWorkspace* layout_out, float* mul_out,
-                         const char* who) {
+                         const char* who, const GatherJob* job, bool* job_taken) {
+  if (job_taken) *job_taken = false;
   MSA_REQUIRE(bank != nullptr, "%s: null bank", who);
   MSA_REQUIRE(layer >= 0 && layer < bank->n_layers, "%s: layer %d out of range", who, layer);
   if (bank->kr_dev[layer] == nullptr) {
@@ -823,9 +954,10 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
   const int32_t K = bank->Hkv * bank->D;
   const int32_t bpq = w.S_pad / 32;
   const int rc = doc_max ? launch_gemm_for<true>(bank->dtype, qs, bank->kr_dev[layer], row_bits, key, bank->chunk_doc_dev,
-                                                 w.M_rows, (int32_t)bank->C, K, bpq, (int32_t)bank->n_docs, st)
+                                                 w.M_rows, (int32_t)bank->C, K, bpq, (int32_t)bank->n_docs, st, job,
+                                                 job_taken)
                          : launch_gemm_for<false>(bank->dtype, qs, bank->kr_dev[layer], row_bits, key, nullptr, w.M_rows,
-                                                  (int32_t)bank->C, K, bpq, (int32_t)bank->n_docs, st);
+                                                  (int32_t)bank->C, K, bpq, (int32_t)bank->n_docs, st, job, job_taken);
   if (rc != MSA_OK) return rc;
   *layout_out = w;
   *mul_out = sc / (float)Hq;

@@ -6,6 +6,7 @@
 // score descending, then document index ascending; 0 is the empty slot.
 #include <mutex>
 
+#include "gather_device.h"
 #include "route_internal.h"
 
 namespace {
@@ -169,17 +170,19 @@ __global__ __launch_bounds__(kMergeWaves * 64) void merge_topk_kernel(const uint
 
 }  // namespace
 
-extern "C" int msa_route_topk(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
-                              int32_t S, int32_t Hq, int32_t mode, float scale, int32_t topk, float* scores_out,
-                              int32_t* doc_out, int64_t* doc_global_out, void* workspace, size_t workspace_bytes,
-                              void* stream) {
-  MSA_REQUIRE(scores_out && doc_out, "msa_route_topk: null output");
-  MSA_REQUIRE(topk > 0 && topk <= kTopkMax, "msa_route_topk: topk=%d out of range (1..%d)", topk, kTopkMax);
+namespace {
+
+int route_topk_impl(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B, int32_t S,
+                    int32_t Hq, int32_t mode, float scale, int32_t topk, float* scores_out, int32_t* doc_out,
+                    int64_t* doc_global_out, void* workspace, size_t workspace_bytes, void* stream, const char* who,
+                    const GatherJob* job, bool* job_taken) {
+  MSA_REQUIRE(scores_out && doc_out, "%s: null output", who);
+  MSA_REQUIRE(topk > 0 && topk <= kTopkMax, "%s: topk=%d out of range (1..%d)", who, topk, kTopkMax);
   RouteWorkspace w;
   float mul;
   hipStream_t st = as_stream(stream);
   int rc = route_scores_to_keys(bank, layer, q, qmask_u8, B, S, Hq, mode, scale, true, workspace, workspace_bytes, st, &w,
-                                &mul, "msa_route_topk");
+                                &mul, who, job, job_taken);
   if (rc != MSA_OK) return rc;
   char* ws = static_cast<char*>(workspace);
   const uint32_t* key = reinterpret_cast<const uint32_t*>(ws + w.off_key);
@@ -190,6 +193,76 @@ extern "C" int msa_route_topk(const msa_bank* bank, int32_t layer, const void* q
   merge_topk_kernel<<<B, kMergeWaves * 64, 0, st>>>(cand, w.topk_blocks, bank->doc_global_id_dev, mul, topk, scores_out, doc_out,
                                       doc_global_out);
   MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
+
+}  // namespace
+
+extern "C" int msa_route_topk(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
+                              int32_t S, int32_t Hq, int32_t mode, float scale, int32_t topk, float* scores_out,
+                              int32_t* doc_out, int64_t* doc_global_out, void* workspace, size_t workspace_bytes,
+                              void* stream) {
+  return route_topk_impl(bank, layer, q, qmask_u8, B, S, Hq, mode, scale, topk, scores_out, doc_out, doc_global_out,
+                         workspace, workspace_bytes, stream, "msa_route_topk", nullptr, nullptr);
+}
+
+// Routing of one layer with the K / V gather of an earlier selection inside the same launch: one workgroup of the
+// scan copies while the others score.  When the scan's form cannot carry the copy (few query rows, fp32) the gather's
+// own kernels run on the same stream first; the results are the same either way.
+extern "C" int msa_route_topk_gather(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
+                                     int32_t S, int32_t Hq, int32_t mode, float scale, int32_t topk, float* scores_out,
+                                     int32_t* doc_out, int64_t* doc_global_out, void* workspace,
+                                     size_t workspace_bytes, int32_t gather_layer, const int32_t* gather_doc_sel,
+                                     int32_t gather_B, int32_t gather_k, void* k_out, void* v_out,
+                                     int64_t out_capacity_chunks, int32_t* cu_sel, void* gather_workspace,
+                                     size_t gather_workspace_bytes, void* stream) {
+  const char* who = "msa_route_topk_gather";
+  MSA_REQUIRE(bank && gather_doc_sel && k_out && v_out && cu_sel && gather_workspace, "%s: null pointer", who);
+  MSA_REQUIRE(gather_B > 0 && gather_B <= 8192 && gather_k > 0 && gather_k <= 64, "%s: gather B=%d k=%d out of range", who,
+              gather_B, gather_k);
+  MSA_REQUIRE(gather_layer >= 0 && gather_layer < bank->n_layers, "%s: gather layer %d out of range", who, gather_layer);
+  MSA_REQUIRE(out_capacity_chunks > 0, "%s: empty gather output", who);
+  if (!bank->k_host[gather_layer] || !bank->v_host[gather_layer]) {
+    msa_set_error("%s: layer %d has no host K / V set", who, gather_layer);
+    return MSA_ESTATE;
+  }
+  if (gather_workspace_bytes < msa_gather_device_workspace_bytes(gather_B, gather_k)) {
+    msa_set_error("%s: gather workspace of %zu bytes, need %zu", who, gather_workspace_bytes,
+                  msa_gather_device_workspace_bytes(gather_B, gather_k));
+    return MSA_ESIZE;
+  }
+  GatherJob job{};
+  job.doc_sel = gather_doc_sel;
+  job.doc_chunk_off = bank->doc_chunk_off_dev;
+  job.cu_sel = cu_sel;
+  job.plan = static_cast<int32_t*>(gather_workspace);
+  job.k_src = static_cast<const uint4*>(bank->k_host[gather_layer]);
+  job.v_src = static_cast<const uint4*>(bank->v_host[gather_layer]);
+  job.k_dst = static_cast<uint4*>(k_out);
+  job.v_dst = static_cast<uint4*>(v_out);
+  job.capacity_rows = out_capacity_chunks;
+  job.n_docs = (int32_t)bank->n_docs;
+  job.B = gather_B;
+  job.k = gather_k;
+  job.dedup = gather_B > 1 && gather_B * gather_k <= msa_gather::kDedupMaxEntries ? 1 : 0;
+  job.row_vecs = (int32_t)((size_t)bank->Hkv * bank->D * elem_bytes(bank->dtype) / 16);
+  job.active = 1;
+  bool taken = false;
+  // the scan's form is known only inside; if it cannot carry the job the gather runs by itself, in front of the scan
+  // (probed with the same routing arguments: the decision depends on the query rows and the dtype alone)
+  const bool fused = bank->dtype == MSA_BF16 && (int64_t)B * ((S + 31) / 32 * 32) > 128;
+  if (!fused) {
+    int rc = msa_gather_kv_device(bank, gather_layer, gather_doc_sel, gather_B, gather_k, k_out, v_out, out_capacity_chunks,
+                                  cu_sel, gather_workspace, gather_workspace_bytes, stream);
+    if (rc != MSA_OK) return rc;
+  }
+  int rc = route_topk_impl(bank, layer, q, qmask_u8, B, S, Hq, mode, scale, topk, scores_out, doc_out, doc_global_out,
+                           workspace, workspace_bytes, stream, who, fused ? &job : nullptr, &taken);
+  if (rc != MSA_OK) return rc;
+  if (fused && !taken) {
+    msa_set_error("%s: internal: the scan did not take the gather", who);
+    return MSA_ESTATE;
+  }
   return MSA_OK;
 }
 

@@ -241,6 +241,37 @@ def gather_kv_device(bank: Bank, layer: int, doc_sel: torch.Tensor, capacity_chu
     return k_out, v_out, cu
 
 
+def route_topk_gather(bank: Bank, layer: int, q: torch.Tensor, qmask: Optional[torch.Tensor], mode: str, scale: float,
+                      topk: int, gather_layer: int, gather_doc_sel: torch.Tensor, capacity_chunks: int,
+                      out: Optional[Tuple[torch.Tensor, torch.Tensor]] = None):
+    """``route_topk`` of ``layer`` with ``gather_kv_device`` of (``gather_layer``, ``gather_doc_sel``) in the same
+    launch (one workgroup of the scan copies while the others score).  Returns the two calls' results:
+    ``(scores, doc, doc_global), (K, V, cu_sel)``."""
+    B, S, Hq, qm = _route_args(bank, q, qmask, mode)
+    _need_cuda(gather_doc_sel)
+    if gather_doc_sel.dtype != torch.int32 or gather_doc_sel.dim() != 2:
+        raise ValueError("gather_doc_sel must be int32 [B, k]")
+    gB, gk = gather_doc_sel.shape
+    lib = _lib.load()
+    dev = q.device
+    ws = bank.workspace(B, S, Hq, topk, dev)
+    scores = torch.empty((B, topk), dtype=torch.float32, device=dev)
+    doc = torch.empty((B, topk), dtype=torch.int32, device=dev)
+    gid = torch.empty((B, topk), dtype=torch.int64, device=dev)
+    if out is None:
+        k_out = torch.empty((capacity_chunks, bank.Hkv, bank.D), dtype=bank.dtype, device=dev)
+        v_out = torch.empty_like(k_out)
+    else:
+        k_out, v_out = out
+    cu = torch.empty(gB + 1, dtype=torch.int32, device=dev)
+    gws = torch.empty(lib.msa_gather_device_workspace_bytes(gB, gk), dtype=torch.uint8, device=dev)
+    check(lib.msa_route_topk_gather(bank.handle, layer, ptr(q), ptr(qm), B, S, Hq, MODES[mode], scale, topk, ptr(scores),
+                                    ptr(doc), ptr(gid), ptr(ws), ws.numel(), gather_layer, ptr(gather_doc_sel), gB, gk,
+                                    ptr(k_out), ptr(v_out), capacity_chunks, ptr(cu), ptr(gws), gws.numel(), _stream()),
+          "msa_route_topk_gather")
+    return (scores, doc, gid), (k_out, v_out, cu)
+
+
 class _null_ctx:
     def __enter__(self):
         return None

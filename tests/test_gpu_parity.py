@@ -581,3 +581,45 @@ def test_by_hand_fixture_through_the_c_abi(ops, dtype):
     mk2, mv2, cu2 = ops.gather_kv_device(bank, 0, sel.cuda(), 8)
     torch.cuda.synchronize()
     assert cu2.cpu().tolist() == gth["cu_sel"] and torch.equal(mk2[:6].cpu(), mk.cpu())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("B,S,dtype", [(6, 128, torch.bfloat16), (3, 200, torch.bfloat16), (2, 40, torch.bfloat16),
+                                      (4, 96, torch.float32)])
+def test_route_topk_gather_equals_the_two_calls(B, S, dtype):
+    """msa_route_topk_gather (routing of one layer with the gather of another layer's selection inside the scan's
+    launch) returns exactly what msa_route_topk and msa_gather_kv_device return by themselves: for the large-tile
+    form of the scan, which carries the copy in one of its workgroups, and for the forms that cannot (few query rows,
+    fp32), where the gather's own kernels run first.  The gathered selection shares documents between samples and
+    holds a duplicate and an out-of-range id."""
+    from msa_amd import ops
+    rng = np.random.default_rng(77 + B)
+    doc_chunks = rng.integers(1, 9, size=300).tolist()
+    dco = np.concatenate([[0], np.cumsum(doc_chunks)])
+    C, Hkv, D = int(dco[-1]), 8, 128
+    g = torch.Generator().manual_seed(5 + S)
+    bank = ops.Bank(2, dco.tolist(), list(range(len(doc_chunks))), Hkv, D, dtype)
+    keep = []
+    for layer in range(2):
+        kr = torch.nn.functional.normalize(torch.randn((C, Hkv, D), generator=g), dim=-1).to(dtype).cuda()
+        kh = torch.randn((C, Hkv, D), generator=g).to(dtype).pin_memory()
+        vh = torch.randn((C, Hkv, D), generator=g).to(dtype).pin_memory()
+        bank.set_layer(layer, kr, kh, vh)
+        keep.append((kr, kh, vh))
+    q = torch.randn((B, S, 32, D), generator=g).to(dtype).cuda()
+    mask = torch.ones(B, S, dtype=torch.bool)
+    mask[0, S // 2:] = False
+    sel = torch.from_numpy(rng.integers(0, len(doc_chunks), size=(5, 7)).astype(np.int32))
+    sel[1, :3] = sel[0, :3]          # documents shared between samples
+    sel[2, 4] = sel[2, 3]            # a duplicate inside a sample
+    sel[3, 0] = -1                   # skipped
+    sel = sel.cuda()
+    cap = 5 * 7 * 8
+    want_r = ops.route_topk(bank, 1, q, mask.cuda(), "cosine", 1.0, 8)
+    want_g = ops.gather_kv_device(bank, 0, sel, cap)
+    (s_, d_, gid_), (k_, v_, cu_) = ops.route_topk_gather(bank, 1, q, mask.cuda(), "cosine", 1.0, 8, 0, sel, cap)
+    torch.cuda.synchronize()
+    assert torch.equal(d_, want_r[1]) and torch.equal(gid_, want_r[2]) and torch.equal(s_, want_r[0])
+    assert torch.equal(cu_, want_g[2])
+    n = int(cu_[-1])
+    assert n > 0 and torch.equal(k_[:n], want_g[0][:n]) and torch.equal(v_[:n], want_g[1][:n])

@@ -145,7 +145,7 @@ struct Mma<float> {
   }
 };
 
-// The MFMA-bound form (bf16, 256 x 256, one workgroup per tile) stages its operand tiles with buffer loads that write
+// The MFMA-bound form (bf16, 256 x 256, one workgroup per compute unit) stages its operand tiles with buffer loads that write
 // LDS directly: no staging registers, no ds_write, and room for a third stage of the operand that comes from HBM.
 // LDS then holds two stages of the query tile (2 x 32 KB) and three of the K_r tile (3 x 32 KB), 160 KB in all, in
 // un-padded 128-byte rows whose 16-byte units are XOR-swizzled by (row >> 1) & 7 (conflict-free operand reads; a
@@ -607,22 +607,31 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
         dtl_load_b(sb2, kt_b);
         advance_b();
       }
-#pragma unroll
-      for (int sub = 0; sub < kSub; ++sub) {
-        if (sub + 1 < kSub) {
+      // One sub-step: the operand reads of the next one, then this one's MFMAs.  A tile's first sub-step multiplies
+      // into zero (the constant operand of the instruction) instead of into accumulators cleared beforehand: 128
+      // register moves per wavefront and tile that nothing could overlap, since the first MFMAs wait for them.
+      auto substep = [&](auto sub_tag, auto fresh_tag) {
+        constexpr int sub = decltype(sub_tag)::value;
+        constexpr bool fresh = decltype(fresh_tag)::value;
+        if constexpr (sub + 1 < kSub) {
           dtl_frags(sa, sb, sub + 1, (sub + 1) & 1);
-        } else if (more) {
-          if (more2) __builtin_amdgcn_s_waitcnt(kWaitAllButNewestB);
-          else __builtin_amdgcn_s_waitcnt(kWaitAll);
-          dtl_barrier();
-          dtl_frags(sa ^ 1, sb1, 0, 0);
-          __builtin_amdgcn_sched_barrier(0);
+        } else {
+          if (more) {
+            if (more2) __builtin_amdgcn_s_waitcnt(kWaitAllButNewestB);
+            else __builtin_amdgcn_s_waitcnt(kWaitAll);
+            dtl_barrier();
+            dtl_frags(sa ^ 1, sb1, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+          }
         }
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j) acc[i][j] = Mma<T>::mma(fa[sub & 1][i], fb[sub & 1][j], acc[i][j]);
-        if (sub + 1 < kSub) {
+          for (int j = 0; j < TN; ++j) {
+            if constexpr (fresh) acc[i][j] = Mma<T>::mma(fa[sub & 1][i], fb[sub & 1][j], floatx16_t{});
+            else acc[i][j] = Mma<T>::mma(fa[sub & 1][i], fb[sub & 1][j], acc[i][j]);
+          }
+        if constexpr (sub + 1 < kSub) {
           // issue order of the sub-step: each of the six operand reads of the next sub-step behind one MFMA of this
           // one, the last two MFMAs behind them (2.5 % faster than the order the scheduler picks by itself)
 #pragma unroll
@@ -632,7 +641,12 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
           }
           __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
         }
-      }
+      };
+      if (kt == 0) substep(std::integral_constant<int, 0>{}, std::true_type{});
+      else substep(std::integral_constant<int, 0>{}, std::false_type{});
+      substep(std::integral_constant<int, 1>{}, std::false_type{});
+      substep(std::integral_constant<int, 2>{}, std::false_type{});
+      substep(std::integral_constant<int, 3>{}, std::false_type{});
       sa ^= 1;
       sb = sb1;
       if (++kt == k_tiles) {
@@ -643,12 +657,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
         tile_n = tn_a;
         m0 = tile_m * BM;
         n0 = tile_n * BN;
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j)
-#pragma unroll
-            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
         fetch_rows();
         fetch_docs(n0);
       }

@@ -224,6 +224,31 @@ def extra_decode(dev):
                                                           "frac_hbm": round(by / ms_fused / 1e6 / HBM_PEAK_GBS, 4)}}
 
 
+def extra_mfma_ceiling(dev):
+    """What the matrix cores sustain with nothing but MFMAs running (a register-only loop at the scoring kernel's
+    occupancy): the rate with operands that toggle is the ceiling the scoring kernel's fraction can be read against."""
+    from msa_amd import _lib
+    lib = _lib.load()
+    wgs, iters = 256 * 4, 40000
+    sink = torch.empty(wgs * 512, dtype=torch.float32, device=dev)
+    flops = C.c_double(0)
+    out = {"workload": f"register-only v_mfma_f32_32x32x16_bf16 loop, {wgs} workgroups x 8 wavefronts x {iters} x 8 MFMAs"}
+    for mode, name in ((0, "zero_operands"), (2, "toggling_operands")):
+        ms = []
+        for rep in range(4):
+            a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            _lib.check(lib.msa_diag_mfma_loop(wgs, iters, mode, sink.data_ptr(), C.byref(flops), torch.cuda.current_stream().cuda_stream),
+                       "msa_diag_mfma_loop")
+            b.record()
+            torch.cuda.synchronize()
+            ms.append(a.elapsed_time(b))
+        best = min(ms[1:])
+        out[name] = {"ms": round(best, 3), "TFLOP/s": round(flops.value / best / 1e9, 1),
+                     "frac_mfma_peak": round(flops.value / best / 1e9 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    return out
+
+
 def extra_decode_projections(dev):
     """configs[4] projection share: the four weight-streaming linears of a decode layer and the LM head at B=16
     (Qwen3-4B shapes, bf16), each replayed from a HIP graph over distinct weight copies so that neither the Python
@@ -330,6 +355,8 @@ def main():
     ap.add_argument("--no-e2e", action="store_true", help="skip the end-to-end sparse decode run among the extras")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (reference point for rocprof FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--ceiling-only", action="store_true",
+                    help="run only the register-only MFMA loop (other_kernels.mfma_ceiling) and print its figures")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no sharding, no collectives); use --gpus 1")
@@ -340,6 +367,9 @@ def main():
     lib = _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.ceiling_only:
+        print(json.dumps({"mfma_ceiling": extra_mfma_ceiling(dev)}), flush=True)
+        return
     B, S, L = args.batch, args.seq, args.layers
 
     t_setup = time.perf_counter()
@@ -573,7 +603,8 @@ def main():
     extras = None
     if not args.no_extras:
         extras = {"pooling": extra_pooling(dev), "routing_10M_bank": extra_routing_10m(dev), "decode_attention": extra_decode(dev),
-                  "prefill_attention": extra_prefill_attention(dev), "decode_projections": extra_decode_projections(dev)}
+                  "prefill_attention": extra_prefill_attention(dev), "decode_projections": extra_decode_projections(dev),
+                  "mfma_ceiling": extra_mfma_ceiling(dev)}
 
     cpu = None
     if not args.no_cpu_baseline:

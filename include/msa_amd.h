@@ -134,6 +134,15 @@ int msa_route_topk_static(const msa_bank* bank, int32_t layer, const void* q, co
 int msa_profile_enable(int32_t max_records);
 int msa_profile_collect(float* ms_host, int32_t cap, int32_t* n_out);
 
+/* Measurement aid (no counterpart in the reference): a register-only loop of v_mfma_f32_32x32x16_bf16, 8 wavefronts
+ * per workgroup with a 4 x 2 grid of accumulators each (the scoring kernel's shape and occupancy), `iters`
+ * iterations of 8 MFMAs per wavefront, enqueued on `stream`.  mode 0: zero operands; 1: operands of ones (every
+ * sink[thread] then holds 128 * iters exactly); 2: operands whose signs and mantissas change every iteration, which is
+ * what the shader clock under real data answers to.  sink: device float [workgroups * 512]; *flops_out (host, may be
+ * null) receives the launch's floating-point operations.  The rate of mode 2 is the ceiling of this GPU's matrix
+ * cores under load, below the published peak, which assumes the boost clock. */
+int msa_diag_mfma_loop(int32_t workgroups, int32_t iters, int32_t mode, float* sink, double* flops_out, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Gather of the selected documents' pooled K / V from pinned host memory.  Replaces the
  * index_select fetch and per-sample regroup of MSAService.doc_query

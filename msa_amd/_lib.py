@@ -34,6 +34,7 @@ SIGNATURES = {
     "msa_route_topk_static": (C.c_int, [_vp, _i32, _vp, _vp, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _vp, _vp, _vp]),
     "msa_profile_enable": (C.c_int, [_i32]),
     "msa_profile_collect": (C.c_int, [_vp, _i32, _vp]),
+    "msa_diag_mfma_loop": (C.c_int, [_i32, _i32, _i32, _vp, _vp, _vp]),
     "msa_gather_plan": (C.c_int, [_vp, _vp, _i32, _i32, _vp]),
     "msa_gather_kv": (C.c_int, [_vp, _i32, _vp, _i32, _i32, _vp, _vp, _i64, _vp]),
     "msa_gather_device_workspace_bytes": (_sz, [_i32, _i32]),

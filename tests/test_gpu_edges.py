@@ -455,3 +455,28 @@ def test_scores_at_most_64_query_rows(ops, Hq, Hkv, B, S):
     mask[0, ::3] = False
     got = ops.chunk_scores(bank, 0, q.cuda(), mask.cuda())
     assert cf.rel_err(got.cpu(), cf.chunk_scores(q, mask, kr, "cosine")) < 1e-2
+
+
+@pytest.mark.gpu
+def test_mfma_loop_diagnostic_counts_exactly():
+    """msa_diag_mfma_loop with operands of ones: every MFMA adds 16 to each accumulator element, eight accumulators per
+    thread are summed, so every thread reports 128 * iters; the reported operation count is workgroups x 8 wavefronts x
+    iters x 8 MFMAs x 2 * 32 * 32 * 16.  The other two modes (zero and toggling operands) run and stay finite."""
+    import ctypes as C
+    from msa_amd import _lib
+    lib = _lib.load()
+    wgs, iters = 8, 1000
+    sink = torch.full((wgs * 512,), -1.0, device="cuda")
+    flops = C.c_double(0)
+    st = torch.cuda.current_stream().cuda_stream
+    _lib.check(lib.msa_diag_mfma_loop(wgs, iters, 1, sink.data_ptr(), C.byref(flops), st), "msa_diag_mfma_loop")
+    torch.cuda.synchronize()
+    assert torch.equal(sink.cpu(), torch.full((wgs * 512,), 128.0 * iters))
+    assert flops.value == wgs * 8 * iters * 8 * 2 * 32 * 32 * 16
+    _lib.check(lib.msa_diag_mfma_loop(wgs, iters, 0, sink.data_ptr(), None, st), "msa_diag_mfma_loop")
+    torch.cuda.synchronize()
+    assert torch.equal(sink.cpu(), torch.zeros(wgs * 512))
+    _lib.check(lib.msa_diag_mfma_loop(wgs, iters, 2, sink.data_ptr(), None, st), "msa_diag_mfma_loop")
+    torch.cuda.synchronize()
+    assert torch.isfinite(sink).all() and (sink != 0).any()
+    assert lib.msa_diag_mfma_loop(0, iters, 1, sink.data_ptr(), None, st) != 0

@@ -29,6 +29,7 @@ struct RouteWorkspace {
   size_t off_row_bits;  // scored-row bitmask, one uint32 per 32 rows
   size_t off_key;       // uint32 [B, n_docs] (routing) or [B, C] (chunk scores): order-preserving keys of the unscaled scores
   size_t off_cand;      // uint64 [B, topk_blocks, kTopkMax] sorted candidates
+  size_t off_sched;     // tile pool words of the persistent scan (counter cleared by the prologue kernel)
   size_t bytes;
 };
 

@@ -37,11 +37,17 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // workgroup 0 the zero words that pad the mask to whole M tiles, and all workgroups together clear the
 // `clear_words` key words the scoring kernel merges into with atomicMax.
 // ------------------------------------------------------------------------------------------
+// Words behind the persistent scan's tile pool: the pool's counter, on a cache line of its own, then one word per
+// workgroup through which the wavefront that drew a tile tells the workgroup's others.
+constexpr int kSchedCounterWords = 32;
+constexpr int kSchedMaxWorkgroups = 1024;
+constexpr size_t kSchedBytes = (size_t)(kSchedCounterWords + kSchedMaxWorkgroups) * sizeof(uint32_t);
+
 template <typename TIn, typename TOut>
 __global__ void presum_queries_kernel(const TIn* __restrict__ q, const uint8_t* __restrict__ qmask, int32_t B,
                                       int32_t S, int32_t S_pad, int32_t Hq, int32_t Hkv, int32_t normalize,
                                       TOut* __restrict__ qs, uint32_t* __restrict__ row_bits, int32_t mask_words,
-                                      uint32_t* __restrict__ key_plane, int64_t clear_words) {
+                                      uint32_t* __restrict__ key_plane, int64_t clear_words, uint32_t* __restrict__ sched) {
   const int row = blockIdx.x;              // b * S_pad + s
   const int b = row / S_pad, s = row % S_pad;
   const int G = Hq / Hkv;
@@ -62,8 +68,10 @@ __global__ void presum_queries_kernel(const TIn* __restrict__ q, const uint8_t* 
     }
     if (threadIdx.x == 0) row_bits[row >> 5] = bits;
   }
-  if (blockIdx.x == 0)
+  if (blockIdx.x == 0) {
     for (int w = (int)(gridDim.x >> 5) + (int)threadIdx.x; w < mask_words; w += blockDim.x) row_bits[w] = 0u;
+    if (threadIdx.x == 0) sched[0] = 0u;        // the scan's pool counter
+  }
   float acc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) acc[i] = 0.f;
@@ -172,14 +180,14 @@ constexpr bool score_tile_is_direct() {
 // HBM stream never drains between tiles.  That is what the HBM-bound shapes need; the MFMA-bound ones keep one
 // workgroup per tile, which leaves compute units free for kernels of other streams.
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool kDocMax, bool kStream>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vgpr(251))) void score_gemm_kernel(
     const T* __restrict__ qs,            // [M_rows, K]  pre-summed queries, M_rows = B * S_pad
     const T* __restrict__ kr,            // [C, K]
     const uint32_t* __restrict__ row_bits,  // [ceil(M_alloc / 32)] scored-row bitmask
     uint32_t* __restrict__ out_key,      // [B, n_docs] or [B, C], zeroed
     const int32_t* __restrict__ chunk_doc,  // [C] document of every chunk (kDocMax)
     int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t tiles_m, int32_t tiles_n,
-    int32_t m_group, int32_t n_docs, GatherJob job) {
+    int32_t m_group, int32_t n_docs, GatherJob job, uint32_t* __restrict__ sched, int32_t pool_n) {
   constexpr int kThreads = WAVES_M * WAVES_N * 64;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -223,18 +231,22 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     return n;
   };
   const int wgs_in_xcd = (scoring_wgs - xcd + 7) / 8;
-  const int n_begin = (int)((int64_t)tiles_n * wgs_before(xcd) / max(scoring_wgs, 1));
-  const int n_stop = (int)((int64_t)tiles_n * (wgs_before(xcd) + wgs_in_xcd) / max(scoring_wgs, 1));
+  // the last pool_n N tiles belong to no XCD: they are the pool every workgroup draws from when its share is done
+  const int tiles_n_own = tiles_n - pool_n;
+  const int n_begin = (int)((int64_t)tiles_n_own * wgs_before(xcd) / max(scoring_wgs, 1));
+  const int n_stop = (int)((int64_t)tiles_n_own * (wgs_before(xcd) + wgs_in_xcd) / max(scoring_wgs, 1));
   const int n_in_xcd = n_stop - n_begin;
-  const int dense_total = n_in_xcd * tiles_m;
-  auto decode_dense = [&](int p, int& tm, int& tn) {
-    const int full_groups = tiles_m / m_group, full = full_groups * n_in_xcd * m_group;
+  const int dense_total = n_in_xcd * tiles_m, pool_total = pool_n * tiles_m;
+  // position p of the dense order over n_in N tiles from nb on (group of M tiles by group, a group's M tiles adjacent)
+  auto decode_range = [&](int p, int nb, int n_in, int& tm, int& tn) {
+    const int full_groups = tiles_m / m_group, full = full_groups * n_in * m_group;
     int g, rem, mg;
-    if (p < full) { g = p / (n_in_xcd * m_group); rem = p - g * n_in_xcd * m_group; mg = m_group; }
+    if (p < full) { g = p / (n_in * m_group); rem = p - g * n_in * m_group; mg = m_group; }
     else { g = full_groups; rem = p - full; mg = tiles_m - full_groups * m_group; }
-    tn = n_begin + rem / mg;
+    tn = nb + rem / mg;
     tm = g * m_group + rem % mg;
   };
+  auto decode_dense = [&](int p, int& tm, int& tn) { decode_range(p, n_begin, n_in_xcd, tm, tn); };
   if constexpr (kDtl) {
     if (is_copy_wg) {
       // plan (sorted, de-duplicated selection -> copy entries), host rows, then the documents an earlier sample
@@ -551,6 +563,27 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     int tm_b = tile_m, tn_b = tile_n, p_b = wg_in_xcd, kt_b = 0;   // K_r loads
     int tm_a = tile_m, tn_a = tile_n, kt_a = 0;                    // query loads
     bool valid_a = true, valid_b = true;
+    // Once the workgroup's own share is done it draws tiles from the pool.  During the first steps of the tile in front
+    // of a pool tile one lane draws the position (an atomic that returns), publishes it (an exchange that returns, so
+    // its arrival says the word is in L2) and every wavefront reads it back: one hop per K step, issued in front of the
+    // step's tile loads, so the waits that already close the step (all but the newest K_r loads) cover it and no
+    // wavefront waits for the hand-out itself.  The position is in use from step 3; the K_r loads leave the tile three
+    // steps before its end, hence at least 6 K tiles per tile (the host offers no pool otherwise).
+    // The three hops keep their operands in v251 - v254, above the registers the compiler may allocate in this kernel
+    // (amdgpu_num_vgpr on its declaration): a value on its way back from memory must not sit in a register the
+    // compiler may copy or reuse before the step's wait has passed, and the compiler, which does not see these
+    // instructions' results, adds no waits of its own for them.  Each memory instruction sits behind five wait states:
+    // its address registers may have been written by a lane read just in front of the statement (a restored spill),
+    // and the hazard between the two is not resolved inside an asm statement.
+    int own_left = (dense_total - wg_in_xcd + wgs_in_xcd - 1) / wgs_in_xcd - 1;   // own tiles behind the K_r loads' one
+    uint32_t* const pool_counter = sched;
+    uint32_t* const my_claim = sched + kSchedCounterWords + blockIdx.x;
+    const bool drawer = __builtin_amdgcn_readfirstlane(tid >> 6) == 0;
+    int p_next = 0;
+    const uint32_t zero_off = 0;
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("v_mov_b32 v253, 1" ::: "v251", "v252", "v253", "v254");
+#endif
     auto set_rsrc_b = [&]() {
       rsrc_ld = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(gb) + (int64_t)tn_b * BN * row_bytes_g, 0,
                                                   (int)(min(BN, C - tn_b * BN) * row_bytes_g), 0x00020000);
@@ -562,11 +595,17 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     auto advance_b = [&]() {
       if (++kt_b == k_tiles) {
         kt_b = 0;
-        p_b += wgs_in_xcd;
-        valid_b = p_b < dense_total;
-        if (valid_b) {
+        if (own_left > 0) {
+          --own_left;
+          p_b += wgs_in_xcd;
           decode_dense(p_b, tm_b, tn_b);
           set_rsrc_b();
+        } else {
+          valid_b = p_next < pool_total;            // (no pool: 0 < 0 ends the walk)
+          if (valid_b) {
+            decode_range(p_next, tiles_n_own, pool_n, tm_b, tn_b);
+            set_rsrc_b();
+          }
         }
       }
     };
@@ -599,6 +638,21 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     for (;;) {
       const int sb1 = sb == 2 ? 0 : sb + 1, sb2 = sb1 == 2 ? 0 : sb1 + 1;
       const bool more = valid_a, more2 = valid_b;    // a next step exists / its successor exists
+#if defined(__HIP_DEVICE_COMPILE__)
+      if (pool_n > 0 && own_left == 0 && more2 && kt < 4) {      // the tile behind this one comes from the pool
+        if (kt == 0) {
+          if (drawer && lane == 0)       // v252 = counter++ (back before this step's closing wait returns)
+            asm volatile("s_nop 4\n\tglobal_atomic_add v252, %0, v253, %1 sc0" ::"v"(zero_off), "s"(pool_counter) : "v252", "v254", "memory");
+        } else if (kt == 1) {
+          if (drawer && lane == 0)       // word = v252; its old value comes back in v254, which tells the word is in L2
+            asm volatile("s_nop 4\n\tglobal_atomic_swap v254, %0, v252, %1 sc0" ::"v"(zero_off), "s"(my_claim) : "v254", "memory");
+        } else if (kt == 2) {            // every wavefront reads the word back (past the L1: device scope)
+          asm volatile("s_nop 4\n\tglobal_load_dword v251, %0, %1 sc1" ::"v"(zero_off), "s"(my_claim) : "v251", "memory");
+        } else {                         // complete since step 2's closing wait
+          asm volatile("v_readfirstlane_b32 %0, v251" : "=s"(p_next));
+        }
+      }
+#endif
       if (more) {
         dtl_load_a(sa ^ 1, kt_a);      // stage of the step before this one: its last reads were behind the previous barrier
         advance_a();
@@ -771,7 +825,7 @@ int compute_units() {
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool kDocMax, bool kStream>
 int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key, const int32_t* chunk_doc,
                 int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t n_docs, hipStream_t st,
-                const GatherJob* job, bool* job_taken) {
+                const GatherJob* job, bool* job_taken, uint32_t* sched) {
   const size_t lds = score_tile_is_direct<T, BM, BN, kSets, kStream>() ? (size_t)kDtlLdsBytes
                                                                         : (size_t)2 * (BM + BN) * kRowStride;
   const int tiles_m = (M_rows + BM - 1) / BM;
@@ -790,6 +844,7 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
     grid = std::min(tiles_n, compute_units() * std::max<int>(1, (int)(kLdsPerCu / lds)));
   }
   GatherJob no_job{};
+  int pool_n = 0;
   const GatherJob* the_job = &no_job;
   if (score_tile_is_direct<T, BM, BN, kSets, kStream>()) {
     // persistent: one workgroup per compute unit walks its XCD's tiles; with a gather job the last one copies instead.
@@ -798,7 +853,12 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
       msa_set_error("score_gemm: K=%d too small for the direct-to-LDS form", K);
       return MSA_EINVAL;
     }
-    grid = std::max(16, compute_units() / 8 * 8);
+    grid = std::min(kSchedMaxWorkgroups, std::max(16, compute_units() / 8 * 8));
+    // The XCDs do not run at one speed (their ends lay up to 6 % apart with fixed ranges, in an order that changes from
+    // launch to launch): the last twelfth of the N tiles is a pool the workgroups draw from one tile at a time once
+    // their own share is done.  Worth it when a workgroup has tiles enough for the pool to even the ends out, and
+    // possible when a tile is deep enough for a draw to come back in time.
+    if ((int64_t)tiles_m * tiles_n >= (int64_t)48 * grid && K * (int)sizeof(T) >= 6 * kRowBytes) pool_n = tiles_n / 12;
     if (job != nullptr && job->active) {
       the_job = job;
       if (job_taken) *job_taken = true;
@@ -815,7 +875,7 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
   if (slot >= 0) MSA_HIP(hipEventRecord(g_timer.start[slot], st));
   kern<<<grid, WAVES_M * WAVES_N * 64, lds, st>>>(static_cast<const T*>(qs), static_cast<const T*>(kr), row_bits, out_key,
                                                   chunk_doc, M_rows, C, K, blocks_per_query, tiles_m, tiles_n, m_group,
-                                                  n_docs, *the_job);
+                                                  n_docs, *the_job, sched, pool_n);
   MSA_LAUNCH_CHECK();
   if (slot >= 0) MSA_HIP(hipEventRecord(g_timer.stop[slot], st));
   return MSA_OK;
@@ -829,14 +889,14 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
 template <bool kDocMax>
 int launch_gemm_for(int32_t dtype, const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key,
                     const int32_t* chunk_doc, int32_t M_rows, int32_t C, int32_t K, int32_t bpq, int32_t n_docs,
-                    hipStream_t st, const GatherJob* job, bool* job_taken) {
+                    hipStream_t st, const GatherJob* job, bool* job_taken, uint32_t* sched) {
   if (dtype != MSA_BF16)
-    return launch_gemm<float, 128, 128, 2, 2, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken);
+    return launch_gemm<float, 128, 128, 2, 2, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
   if (M_rows <= 64)
-    return launch_gemm<bf16_t, 64, 128, 2, 2, 2, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken);
+    return launch_gemm<bf16_t, 64, 128, 2, 2, 2, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
   if (M_rows <= 128)
-    return launch_gemm<bf16_t, 128, 384, 2, 4, 1, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken);
-  return launch_gemm<bf16_t, 256, 256, 2, 4, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken);
+    return launch_gemm<bf16_t, 128, 384, 2, 4, 1, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
+  return launch_gemm<bf16_t, 256, 256, 2, 4, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
 }
 
 }  // namespace
@@ -858,6 +918,7 @@ RouteWorkspace route_workspace_layout(int32_t B, int32_t S, int32_t Hkv, int32_t
   w.off_key = off;      off = align_up(off + (size_t)B * plane_cols * sizeof(uint32_t), 256);
   w.topk_blocks = topk_blocks_for(n_docs);
   w.off_cand = off;     off = align_up(off + (size_t)B * w.topk_blocks * kTopkMax * sizeof(uint64_t), 256);
+  w.off_sched = off;    off = align_up(off + kSchedBytes, 256);
   w.bytes = off;
   return w;
 }
@@ -945,6 +1006,7 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
   void* qs = ws + w.off_qs;
   uint32_t* row_bits = reinterpret_cast<uint32_t*>(ws + w.off_row_bits);
   uint32_t* key = reinterpret_cast<uint32_t*>(ws + w.off_key);
+  uint32_t* sched = reinterpret_cast<uint32_t*>(ws + w.off_sched);
 
   const int normalize = mode == MSA_MODE_COSINE ? 1 : 0;
   const int pthreads = bank->Hkv * 16;
@@ -952,20 +1014,20 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
   if (bank->dtype == MSA_BF16)
     presum_queries_kernel<bf16_t, bf16_t><<<w.M_rows, pthreads, 0, st>>>(
         static_cast<const bf16_t*>(q), qmask_u8, B, S, w.S_pad, Hq, bank->Hkv, normalize, static_cast<bf16_t*>(qs),
-        row_bits, w.mask_words, key, clear_words);
+        row_bits, w.mask_words, key, clear_words, sched);
   else
     presum_queries_kernel<float, float><<<w.M_rows, pthreads, 0, st>>>(
         static_cast<const float*>(q), qmask_u8, B, S, w.S_pad, Hq, bank->Hkv, normalize, static_cast<float*>(qs),
-        row_bits, w.mask_words, key, clear_words);
+        row_bits, w.mask_words, key, clear_words, sched);
   MSA_LAUNCH_CHECK();
 
   const int32_t K = bank->Hkv * bank->D;
   const int32_t bpq = w.S_pad / 32;
   const int rc = doc_max ? launch_gemm_for<true>(bank->dtype, qs, bank->kr_dev[layer], row_bits, key, bank->chunk_doc_dev,
                                                  w.M_rows, (int32_t)bank->C, K, bpq, (int32_t)bank->n_docs, st, job,
-                                                 job_taken)
+                                                 job_taken, sched)
                          : launch_gemm_for<false>(bank->dtype, qs, bank->kr_dev[layer], row_bits, key, nullptr, w.M_rows,
-                                                  (int32_t)bank->C, K, bpq, (int32_t)bank->n_docs, st, job, job_taken);
+                                                  (int32_t)bank->C, K, bpq, (int32_t)bank->n_docs, st, job, job_taken, sched);
   if (rc != MSA_OK) return rc;
   *layout_out = w;
   *mul_out = sc / (float)Hq;

@@ -140,6 +140,15 @@ def test_config3_hundred_million_token_bank(ops):
     assert cud.cpu().tolist() == wcu.tolist()
     assert torch.equal(Kd[:n].cpu(), _pattern_rows(_pattern_k, exp_chunks)) and torch.equal(Vd[:n].cpu(), _pattern_rows(_pattern_v, exp_chunks))
 
+    # the same gather carried by a scan's launch (one workgroup of it copies, the others score; at this size the
+    # scan's last N tiles are a pool the workgroups draw from): both calls' results, bit for bit
+    (s3, d3, g3), (Kf, Vf, cuf) = ops.route_topk_gather(bank, 0, q, None, "cosine", 1.0, TOPK, 0, doc, cap)
+    torch.cuda.synchronize()
+    assert torch.equal(d3, doc) and torch.equal(s3, scores) and torch.equal(g3, gid)
+    assert cuf.cpu().tolist() == wcu.tolist()
+    assert torch.equal(Kf[:n].cpu(), _pattern_rows(_pattern_k, exp_chunks)) and torch.equal(Vf[:n].cpu(), _pattern_rows(_pattern_v, exp_chunks))
+    del Kf, Vf, Kd, Vd
+
     # oracle parity of the chunk scores on a sample (random chunks plus every planted one)
     cs_all = ops.chunk_scores(bank, 0, q, None, "cosine", 1.0)
     torch.cuda.synchronize()

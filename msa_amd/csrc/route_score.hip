@@ -855,10 +855,11 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
     }
     grid = std::min(kSchedMaxWorkgroups, std::max(16, compute_units() / 8 * 8));
     // The XCDs do not run at one speed (their ends lay up to 6 % apart with fixed ranges, in an order that changes from
-    // launch to launch): the last twelfth of the N tiles is a pool the workgroups draw from one tile at a time once
-    // their own share is done.  Worth it when a workgroup has tiles enough for the pool to even the ends out, and
+    // launch to launch): the last eighth of the N tiles is a pool the workgroups draw from one tile at a time once
+    // their own share is done (a sixth to a twenty-fourth measured alike at 196 tiles per workgroup, the larger pools
+    // slightly better at 39).  Worth it when a workgroup has tiles enough for the pool to even the ends out, and
     // possible when a tile is deep enough for a draw to come back in time.
-    if ((int64_t)tiles_m * tiles_n >= (int64_t)48 * grid && K * (int)sizeof(T) >= 6 * kRowBytes) pool_n = tiles_n / 12;
+    if ((int64_t)tiles_m * tiles_n >= (int64_t)16 * grid && K * (int)sizeof(T) >= 6 * kRowBytes) pool_n = tiles_n / 8;
     if (job != nullptr && job->active) {
       the_job = job;
       if (job_taken) *job_taken = true;

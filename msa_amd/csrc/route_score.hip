@@ -168,6 +168,16 @@ constexpr bool score_tile_is_direct() {
   return sizeof(T) == 2 && BM == 256 && BN == 256 && kSets == 1 && !kStream;
 }
 
+// The HBM-bound form for up to 128 query rows (bf16, 128 x 256, streaming over N tiles) uses the same loads with three
+// stages of each operand (3 x 16 KB + 3 x 32 KB = 144 KB): both operands are requested two K steps ahead, which keeps
+// 96 KB per compute unit in flight (returns are in order, so the query tile has to run as far ahead as the K_r tile for
+// the K_r tile's lead to count).
+constexpr int kDtlStreamLdsBytes = 3 * (128 + 256) * 128;
+template <typename T, int BM, int BN, int kSets, bool kStream>
+constexpr bool score_tile_is_direct_stream() {
+  return sizeof(T) == 2 && BM == 128 && BN == 256 && kSets == 1 && kStream;
+}
+
 // Workgroup tile BM x BN, WAVES_M x WAVES_N wavefronts, each owning TM x TN blocks of 32 x 32.
 // kSets: register sets of global loads, i.e. K tiles in flight ahead of the one being multiplied.  One is enough when
 // a tile's MFMA work outlasts a load's latency (the MFMA-bound shapes); the HBM-bound shapes (few query rows) need
@@ -197,6 +207,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vg
   extern __shared__ __align__(16) char lds[];
   constexpr int kBufBytes = (BM + BN) * kRowStride;   // [A tile | B tile] per buffer, two buffers
   constexpr bool kDtl = score_tile_is_direct<T, BM, BN, kSets, kStream>();
+  constexpr bool kDtlStream = score_tile_is_direct_stream<T, BM, BN, kSets, kStream>();
 
   // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so each XCD gets one
   // contiguous range of K_r tiles.  Inside it the M tiles are walked in groups of m_group: a group's
@@ -715,6 +726,126 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vg
         fetch_docs(n0);
       }
     }
+  } else if constexpr (kDtlStream) {
+    static_assert(kThreads == 512 && kSub == 4 && TM == 2 && TN == 2, "laid out for 8 wavefronts of 64 x 64");
+    constexpr int kAStage = BM * 128, kBStage = BN * 128, kStages = 3;
+    constexpr int kALoads = BM / 64, kBLoads = BN / 64;      // 1 KB blocks (8 rows) per wavefront and stage
+    constexpr int kWaitAllButNewestStep = 0x0F70 + kALoads + kBLoads, kWaitAll = 0x0F70;
+    char* const lds_a = lds;
+    char* const lds_b = lds + kStages * kAStage;
+    auto dtl_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    auto voff_of = [&](int row) { return row * (int)row_bytes_g + ((dtl_slot ^ ((row >> 1) & 7)) * 16); };
+    auto load_a = [&](int stage, int kt) {
+#pragma unroll
+      for (int i = 0; i < kALoads; ++i) {
+        const int blk = wave * kALoads + i;
+        MSA_LOAD_TO_LDS(rsrc_a, lds_a + stage * kAStage + blk * 1024, voff_of(blk * 8 + dtl_row), kt * kRowBytes, 0);
+      }
+    };
+    auto load_b = [&](int stage, int kt) {
+#pragma unroll
+      for (int i = 0; i < kBLoads; ++i) {
+        const int blk = wave * kBLoads + i;
+        MSA_LOAD_TO_LDS(rsrc_ld, lds_b + stage * kBStage + blk * 1024, voff_of(blk * 8 + dtl_row), kt * kRowBytes,
+                        kStreamHint);
+      }
+    };
+    auto frags = [&](int stage, int sub, int slot) {
+      const int unit = sub * 2 + half;
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+        const int row = wm * WM + i * 32 + l32;
+        fa[slot][i] = *reinterpret_cast<const Frag*>(lds_a + stage * kAStage + row * 128 + ((unit ^ ((row >> 1) & 7)) * 16));
+      }
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int row = wn * WN + j * 32 + l32;
+        fb[slot][j] = *reinterpret_cast<const Frag*>(lds_b + stage * kBStage + row * 128 + ((unit ^ ((row >> 1) & 7)) * 16));
+      }
+    };
+    // The workgroup's N tiles (blockIdx.x, blockIdx.x + gridDim.x, ...) form one sequence of K steps; the loads run two
+    // steps ahead of the MFMAs across tile boundaries.
+    const int my_tiles = (tiles_n - tile_n + (int)gridDim.x - 1) / (int)gridDim.x;
+    int t_ld = 0, kt_ld = 0;                       // tile and K tile the loads have reached
+    auto advance_ld = [&]() {
+      if (++kt_ld == k_tiles) {
+        kt_ld = 0;
+        if (++t_ld < my_tiles) {
+          const int tn = tile_n + t_ld * (int)gridDim.x;
+          rsrc_ld = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(gb) + (int64_t)tn * BN * row_bytes_g, 0,
+                                                      (int)(min(BN, C - tn * BN) * row_bytes_g), 0x00020000);
+        }
+      }
+    };
+    fetch_rows();                                  // one M tile: the scored-row words serve every N tile
+    fetch_docs(n0);
+    load_a(0, 0);
+    load_b(0, 0);
+    advance_ld();
+    if (t_ld < my_tiles) {
+      load_a(1, kt_ld);
+      load_b(1, kt_ld);
+      advance_ld();
+      __builtin_amdgcn_s_waitcnt(kWaitAllButNewestStep);
+    } else {
+      __builtin_amdgcn_s_waitcnt(kWaitAll);
+    }
+    dtl_barrier();
+    frags(0, 0, 0);
+    int st = 0, t = 0, kt = 0;
+    for (;;) {
+      const int st1 = st == 2 ? 0 : st + 1, st2 = st1 == 2 ? 0 : st1 + 1;
+      const bool more = !(t == my_tiles - 1 && kt == k_tiles - 1);    // a next step exists
+      const bool more2 = t_ld < my_tiles;                              // the step behind it exists
+      if (more2) {
+        load_a(st2, kt_ld);      // stage of the step before this one: its last reads were behind the previous barrier
+        load_b(st2, kt_ld);
+        advance_ld();
+      }
+      auto substep = [&](auto sub_tag, auto fresh_tag) {
+        constexpr int sub = decltype(sub_tag)::value;
+        constexpr bool fresh = decltype(fresh_tag)::value;
+        if constexpr (sub + 1 < kSub) {
+          frags(st, sub + 1, (sub + 1) & 1);
+        } else {
+          if (more) {
+            if (more2) __builtin_amdgcn_s_waitcnt(kWaitAllButNewestStep);
+            else __builtin_amdgcn_s_waitcnt(kWaitAll);
+            dtl_barrier();
+            frags(st1, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) {
+            if constexpr (fresh) acc[i][j] = Mma<T>::mma(fa[sub & 1][i], fb[sub & 1][j], floatx16_t{});
+            else acc[i][j] = Mma<T>::mma(fa[sub & 1][i], fb[sub & 1][j], acc[i][j]);
+          }
+        if constexpr (sub + 1 < kSub) {
+#pragma unroll
+          for (int g = 0; g < TM + TN; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+          }
+        }
+      };
+      if (kt == 0) substep(std::integral_constant<int, 0>{}, std::true_type{});
+      else substep(std::integral_constant<int, 0>{}, std::false_type{});
+      substep(std::integral_constant<int, 1>{}, std::false_type{});
+      substep(std::integral_constant<int, 2>{}, std::false_type{});
+      substep(std::integral_constant<int, 3>{}, std::false_type{});
+      st = st1;
+      if (++kt == k_tiles) {
+        epilogue(n0);
+        if (!more) break;
+        kt = 0;
+        ++t;
+        n0 += (int)gridDim.x * BN;
+        fetch_docs(n0);
+      }
+    }
   } else if constexpr (kStream) {
     // The workgroup's tiles form one sequence of steps (K tiles are even in number, so set tags and LDS buffers
     // alternate the same way in every tile); an epilogue sits where a tile's last step ends, with the next tile's
@@ -826,8 +957,9 @@ template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool 
 int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key, const int32_t* chunk_doc,
                 int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t n_docs, hipStream_t st,
                 const GatherJob* job, bool* job_taken, uint32_t* sched) {
-  const size_t lds = score_tile_is_direct<T, BM, BN, kSets, kStream>() ? (size_t)kDtlLdsBytes
-                                                                        : (size_t)2 * (BM + BN) * kRowStride;
+  const size_t lds = score_tile_is_direct<T, BM, BN, kSets, kStream>()          ? (size_t)kDtlLdsBytes
+                     : score_tile_is_direct_stream<T, BM, BN, kSets, kStream>() ? (size_t)kDtlStreamLdsBytes
+                                                                                 : (size_t)2 * (BM + BN) * kRowStride;
   const int tiles_m = (M_rows + BM - 1) / BM;
   const int tiles_n = (C + BN - 1) / BN;
   // M tiles are walked in groups of 8 per K_r tile: a group's query rows (4 MiB in bf16) are what an XCD's L2
@@ -883,10 +1015,11 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
 }
 
 // Tile choice by query rows.  Up to 64 rows: narrow M tile, two workgroups per compute unit, two K tiles of global
-// loads ahead (3 % faster than one).  Up to 128 rows: the widest N tile that fits LDS, so the query tile a workgroup
-// re-reads from L2 per K_r tile is the smallest share of its intake (128 x 384 beats 128 x 256 by 3 % and 128 x 128
-// by 8 %; a second or third register set of loads in flight, or 16 wavefronts instead of 8, measured 0-6 % slower
-// here: the bytes in flight are not what limits this shape).  More rows are MFMA-bound: 256 x 256 tile.
+// loads ahead (3 % faster than one).  Up to 128 rows: 128 x 256 with both operands loaded straight into LDS two K steps
+// ahead (1.5 % faster than the register-staged 128 x 384 it replaced, which beat register-staged 128 x 256 by 3 % and
+// 128 x 128 by 8 %; more register sets of loads in flight or 16 wavefronts measured 0-6 % slower: the bytes in flight
+// are not what limits this shape, the query tile's own traffic and the MFMA work are - with a query tile of zeros the
+// same launch streams at the rate of the 64-row form).  More rows are MFMA-bound: 256 x 256 tile.
 template <bool kDocMax>
 int launch_gemm_for(int32_t dtype, const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key,
                     const int32_t* chunk_doc, int32_t M_rows, int32_t C, int32_t K, int32_t bpq, int32_t n_docs,
@@ -896,7 +1029,7 @@ int launch_gemm_for(int32_t dtype, const void* qs, const void* kr, const uint32_
   if (M_rows <= 64)
     return launch_gemm<bf16_t, 64, 128, 2, 2, 2, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
   if (M_rows <= 128)
-    return launch_gemm<bf16_t, 128, 384, 2, 4, 1, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
+    return launch_gemm<bf16_t, 128, 256, 2, 4, 1, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
   return launch_gemm<bf16_t, 256, 256, 2, 4, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
 }
 

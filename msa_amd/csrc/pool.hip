@@ -14,6 +14,7 @@
 namespace {
 
 constexpr int kThreads = 256;
+constexpr int kStreamHint = 2;   // non-temporal: every input row is read once
 
 struct PoolArgs {
   const void* in[3];
@@ -42,7 +43,7 @@ template <>
 struct Raw8<bf16_t> {
   u32x4_t w;
   __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t rs, int voff, int soff) {
-    w = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff, 0);
+    w = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff, kStreamHint);
   }
   __device__ __forceinline__ void unpack(float (&x)[8]) const {
     x[0] = bf16lo(w.x); x[1] = bf16hi(w.x); x[2] = bf16lo(w.y); x[3] = bf16hi(w.y);
@@ -53,8 +54,8 @@ template <>
 struct Raw8<float> {
   u32x4_t a, b;
   __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t rs, int voff, int soff) {
-    a = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff, 0);
-    b = __builtin_amdgcn_raw_buffer_load_b128(rs, voff + 16, soff, 0);
+    a = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, soff, kStreamHint);
+    b = __builtin_amdgcn_raw_buffer_load_b128(rs, voff + 16, soff, kStreamHint);
   }
   __device__ __forceinline__ void unpack(float (&x)[8]) const {
     x[0] = __uint_as_float(a.x); x[1] = __uint_as_float(a.y); x[2] = __uint_as_float(a.z); x[3] = __uint_as_float(a.w);

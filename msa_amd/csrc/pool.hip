@@ -78,7 +78,9 @@ __device__ __forceinline__ void store8<float>(float* p, const float (&x)[8]) {
   *reinterpret_cast<float4*>(p + 4) = make_float4(x[4], x[5], x[6], x[7]);
 }
 
-template <typename T>
+// kRope: the launch's tensors are rotated while read (a launch holds tensors of one kind, so the plain kind does not
+// carry the rotary state's registers: 3 - 4 workgroups per compute unit instead of 2).
+template <typename T, bool kRope>
 __global__ __launch_bounds__(kThreads, 2) void pool_chunks_kernel(PoolArgs a) {
   __shared__ float fold[kThreads * 16];
 
@@ -86,7 +88,7 @@ __global__ __launch_bounds__(kThreads, 2) void pool_chunks_kernel(PoolArgs a) {
   const int slot = blockIdx.y;
   const T* __restrict__ in = static_cast<const T*>(a.in[slot]);
   T* __restrict__ out = static_cast<T*>(a.out[slot]);
-  const bool rope = a.rope[slot] != 0;
+  constexpr bool rope = kRope;
 
   const int U = a.H * 8;          // lanes per token row
   const int R = kThreads / U;     // token rows per step (the host checks that U divides the workgroup)
@@ -130,7 +132,7 @@ __global__ __launch_bounds__(kThreads, 2) void pool_chunks_kernel(PoolArgs a) {
 
   // rotary state of this lane's 8 frequencies at its current token, advanced by R positions per step
   float rc[8], rs[8], sc[8], ss[8];
-  if (rope) {
+  if constexpr (rope) {
     const int32_t pos0 = t0 - a.doc_start[a.chunk_doc[c]] + r;
     const int32_t p = min(pos0, a.rope_rows - 1), st = min(R, a.rope_rows - 1);
 #pragma unroll
@@ -143,13 +145,13 @@ __global__ __launch_bounds__(kThreads, 2) void pool_chunks_kernel(PoolArgs a) {
   }
 
   auto consume = [&](auto rope_tag, const Raw8<T>(&lo)[kRows], const Raw8<T>(&hi)[kRows]) {
-    constexpr bool kRope = decltype(rope_tag)::value;
+    constexpr bool kRotate = decltype(rope_tag)::value;
 #pragma unroll
     for (int q = 0; q < kRows; ++q) {
       float xl[8], xh[8];
       lo[q].unpack(xl);
       hi[q].unpack(xh);
-      if constexpr (kRope) {
+      if constexpr (kRotate) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           acc_lo[i] += xl[i] * rc[i] - xh[i] * rs[i];
@@ -178,8 +180,7 @@ __global__ __launch_bounds__(kThreads, 2) void pool_chunks_kernel(PoolArgs a) {
       consume(rope_tag, lo_b, hi_b);
     }
   };
-  if (rope) stream(std::true_type{});
-  else stream(std::false_type{});
+  stream(std::integral_constant<bool, kRope>{});
 
   // fold the R partial rows: fold[(r * U + u) * 16 + i]
 #pragma unroll
@@ -246,28 +247,40 @@ extern "C" int msa_pool_chunks(const void* k, const void* v, const void* kr, int
   }
   if (C == 0) return MSA_OK;
 
-  PoolArgs a{};
-  int n = 0;
-  auto add = [&](const void* in, void* out, int rp, int nm) {
+  // two launches at most: the tensors read plain, and the one rotated while read
+  PoolArgs plain{}, rotated{};
+  auto add = [&](PoolArgs& a, const void* in, void* out, int nm) {
     if (!in) return;
-    a.in[n] = in; a.out[n] = out; a.rope[n] = rp; a.normalize[n] = nm; ++n;
+    const int n = a.n_tensors++;
+    a.in[n] = in; a.out[n] = out; a.rope[n] = &a == &rotated; a.normalize[n] = nm;
   };
-  add(k, k_out, rope ? 1 : 0, 0);
-  add(v, v_out, 0, 0);
-  add(kr, kr_out, 0, normalize_kr ? 1 : 0);
-  MSA_REQUIRE(n > 0, "msa_pool_chunks: nothing to pool");
-  for (int i = 0; i < n; ++i)
-    MSA_REQUIRE(((uintptr_t)a.in[i] & 15) == 0 && ((uintptr_t)a.out[i] & 15) == 0,
-                "msa_pool_chunks: tensors must be 16-byte aligned");
-  a.n_tensors = n; a.T = T; a.H = H;
-  a.chunk_start = chunk_start; a.chunk_len = chunk_len; a.chunk_doc = chunk_doc; a.doc_start = doc_start;
-  a.rope_cos = rope_cos; a.rope_sin = rope_sin; a.rope_rows = rope_rows;
-
-  dim3 grid((unsigned)C, (unsigned)n);
-  if (dtype == MSA_BF16)
-    pool_chunks_kernel<bf16_t><<<grid, kThreads, 0, as_stream(stream)>>>(a);
-  else
-    pool_chunks_kernel<float><<<grid, kThreads, 0, as_stream(stream)>>>(a);
-  MSA_LAUNCH_CHECK();
+  add(rope ? rotated : plain, k, k_out, 0);
+  add(plain, v, v_out, 0);
+  add(plain, kr, kr_out, normalize_kr ? 1 : 0);
+  MSA_REQUIRE(plain.n_tensors + rotated.n_tensors > 0, "msa_pool_chunks: nothing to pool");
+  for (PoolArgs* a : {&plain, &rotated}) {
+    for (int i = 0; i < a->n_tensors; ++i)
+      MSA_REQUIRE(((uintptr_t)a->in[i] & 15) == 0 && ((uintptr_t)a->out[i] & 15) == 0,
+                  "msa_pool_chunks: tensors must be 16-byte aligned");
+    a->T = T; a->H = H;
+    a->chunk_start = chunk_start; a->chunk_len = chunk_len; a->chunk_doc = chunk_doc; a->doc_start = doc_start;
+    a->rope_cos = rope_cos; a->rope_sin = rope_sin; a->rope_rows = rope_rows;
+  }
+  if (plain.n_tensors > 0) {
+    const dim3 grid((unsigned)C, (unsigned)plain.n_tensors);
+    if (dtype == MSA_BF16)
+      pool_chunks_kernel<bf16_t, false><<<grid, kThreads, 0, as_stream(stream)>>>(plain);
+    else
+      pool_chunks_kernel<float, false><<<grid, kThreads, 0, as_stream(stream)>>>(plain);
+    MSA_LAUNCH_CHECK();
+  }
+  if (rotated.n_tensors > 0) {
+    const dim3 grid((unsigned)C, (unsigned)rotated.n_tensors);
+    if (dtype == MSA_BF16)
+      pool_chunks_kernel<bf16_t, true><<<grid, kThreads, 0, as_stream(stream)>>>(rotated);
+    else
+      pool_chunks_kernel<float, true><<<grid, kThreads, 0, as_stream(stream)>>>(rotated);
+    MSA_LAUNCH_CHECK();
+  }
   return MSA_OK;
 }

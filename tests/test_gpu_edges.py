@@ -480,3 +480,54 @@ def test_mfma_loop_diagnostic_counts_exactly():
     torch.cuda.synchronize()
     assert torch.isfinite(sink).all() and (sink != 0).any()
     assert lib.msa_diag_mfma_loop(0, iters, 1, sink.data_ptr(), None, st) != 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_route_topk_mid_size_banks_with_the_tile_pool(seed):
+    """Random mid-size banks (130k - 300k chunks, 9 - 24 queries of 64 - 200 tokens, 4 or 8 KV heads, ragged masks, both
+    modes): large enough for the scan's tile pool (the last eighth of the N tiles, drawn dynamically) to be active with
+    ragged last tiles.  Checked against the whole-bank property the top-k must have, computed by plain fp32 torch
+    matmuls on the device from the same bf16 inputs: the returned scores are the documents' true scores, they come in
+    descending order, and no returned document scores below the true k-th score (beyond the tie tolerance)."""
+    from msa_amd import ops
+    rng = np.random.default_rng(seed)
+    g = torch.Generator(device="cuda").manual_seed(seed)
+    D = 128
+    Hkv = int(rng.choice([4, 8])); Hq = Hkv * 4
+    B = int(rng.integers(9, 25)); S = int(rng.integers(64, 200))
+    n_docs = int(rng.integers(9000, 16000))
+    doc_chunks = rng.integers(4, 33, size=n_docs)
+    dco = np.concatenate([[0], np.cumsum(doc_chunks)]); C = int(dco[-1])
+    mode = ["cosine", "scaled_dot"][seed % 2]
+    k = [4, 16, 32][seed % 3]
+    say(f"mid-size bank seed={seed} B={B} S={S} Hkv={Hkv} C={C} docs={n_docs} mode={mode} k={k}")
+    bank = ops.Bank(1, dco.tolist(), list(range(n_docs)), Hkv, D, torch.bfloat16)
+    kr = torch.randn((C, Hkv, D), generator=g, device="cuda")
+    if mode == "cosine":
+        kr = kr / kr.norm(dim=-1, keepdim=True)
+    kr = kr.to(torch.bfloat16)
+    bank.set_layer(0, kr)
+    q = torch.randn((B, S, Hq, D), generator=g, device="cuda").to(torch.bfloat16)
+    mask = torch.rand((B, S), generator=g, device="cuda") > 0.2
+    mask[:, 0] = True
+    scale = D ** -0.5
+    sc, doc, gid = ops.route_topk(bank, 0, q, mask, mode, scale, k)
+    torch.cuda.synchronize()
+    qf = q.float()
+    if mode == "cosine":
+        qf = qf / qf.norm(dim=-1, keepdim=True)
+    qs = qf.view(B, S, Hkv, 4, D).sum(3).to(torch.bfloat16).float()        # rounded as the kernel's pre-sum rounds them
+    krf = kr.float().view(C, Hkv * D)
+    seg = torch.repeat_interleave(torch.arange(n_docs, device="cuda"), torch.as_tensor(doc_chunks, device="cuda"))
+    mul = (1.0 if mode == "cosine" else scale) / Hq
+    for b in range(B):
+        s_bc = (qs[b].reshape(S, Hkv * D) @ krf.T) * mul
+        s_bc[~mask[b]] = float("-inf")
+        ds = torch.full((n_docs,), float("-inf"), device="cuda").scatter_reduce_(0, seg, s_bc.max(0).values, reduce="amax")
+        true_of_returned = ds[doc[b].long()]
+        kth = torch.topk(ds, k).values[-1]
+        assert torch.allclose(sc[b], true_of_returned, rtol=1e-2, atol=2e-3)
+        assert bool((true_of_returned >= kth - 1e-3).all())                  # the 1e-3 gap rule at the k boundary
+        assert bool((sc[b][:-1] >= sc[b][1:]).all())
+        assert torch.equal(gid[b], doc[b].long())

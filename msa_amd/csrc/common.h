@@ -77,6 +77,16 @@ __device__ __forceinline__ float row16_ror8(float v) {  // value of the lane 8 p
   return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), 0x128, 0xf, 0xf, false));
 }
 
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+// 16 bytes per lane from a buffer resource straight into LDS (lane l lands at byte 16 * l behind `lds_dst`, which must be
+// the same in every lane).  The compiler's host pass has no such instruction and only needs the kernel's signature.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define MSA_LOAD_TO_LDS(rsrc, lds_dst, voffset, soffset, aux) \
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(lds_dst), 16, voffset, soffset, 0, aux)
+#else
+#define MSA_LOAD_TO_LDS(rsrc, lds_dst, voffset, soffset, aux) ((void)(rsrc), (void)(lds_dst), (void)(voffset), (void)(soffset))
+#endif
+
 static inline hipStream_t as_stream(void* s) { return (hipStream_t)s; }
 static inline size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 static inline size_t elem_bytes(int dtype) { return dtype == MSA_F32 ? 4 : 2; }

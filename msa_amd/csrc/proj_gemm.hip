@@ -8,8 +8,9 @@
 // 128-wide head; after the main loop it parks the block in LDS and finishes it row-wise (16 lanes per token row), where
 // the norm's sum of squares is a 16-lane reduction and a rotary pair (d, d + 64) is the lane 8 places away.  The main
 // loop is the one of the
-// scoring kernel: global -> register -> LDS staging through buffer loads whose extent is the valid part of the tile,
-// two LDS buffers, operand fragments one sub-step ahead, one barrier per K tile.
+// scoring kernel's large-tile form: operand tiles loaded straight into LDS through buffer resources whose extent is the
+// valid part of the tile, two stages of the token tile and three of the weight tile, operand fragments one sub-step
+// ahead, one barrier per K tile.
 #include <algorithm>
 #include <type_traits>
 
@@ -22,13 +23,11 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kRowBytes = 128;                 // one K tile of a row: 64 bf16
-constexpr int kRowStride = kRowBytes + 16;     // padded LDS row: conflict-free 16-byte operand reads
 constexpr int BM = 256, BN = 256, WAVES_M = 4, WAVES_N = 2;
 constexpr int kThreads = WAVES_M * WAVES_N * 64;
 constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;      // 64 tokens x 128 columns (one head) per wavefront
 constexpr int TM = WM / 32, TN = WN / 32;
-constexpr int kVecA = BM * 8 / kThreads, kVecB = BN * 8 / kThreads;
-constexpr int kBufBytes = (BM + BN) * kRowStride;
+constexpr int kLdsBytes = 5 * 256 * 128;       // two stages of the token tile, three of the weight tile
 constexpr int kSub = 4;                        // 32x32x16 steps per K tile
 static_assert(WN == kHeadDim, "a wavefront owns whole heads");
 
@@ -75,28 +74,7 @@ __global__ __launch_bounds__(kThreads) void proj_gemm_kernel(ProjArgs a) {
       const_cast<char*>(reinterpret_cast<const char*>(a.x)) + (int64_t)m0 * row_bytes_g, 0, rows_a * row_bytes_g, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_b = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<char*>(reinterpret_cast<const char*>(a.w)) + (int64_t)n0 * row_bytes_g, 0, rows_b * row_bytes_g, 0x00020000);
-  const int voff = (tid >> 3) * row_bytes_g + (tid & 7) * 16;
-  const int vec_stride = (kThreads / 8) * row_bytes_g;
   const int k_tiles = row_bytes_g / kRowBytes;
-  u32x4_t ra[kVecA], rb[kVecB];
-  auto load_tile = [&](int kt) {
-#pragma unroll
-    for (int i = 0; i < kVecA; ++i) ra[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_a, voff + i * vec_stride, kt * kRowBytes, 0);
-#pragma unroll
-    for (int i = 0; i < kVecB; ++i) rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rsrc_b, voff + i * vec_stride, kt * kRowBytes, 0);
-  };
-  auto store_tile = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < kVecA; ++i) {
-      const int v = tid + i * kThreads, r = v >> 3, c = v & 7;
-      *reinterpret_cast<u32x4_t*>(lds + buf * kBufBytes + r * kRowStride + c * 16) = ra[i];
-    }
-#pragma unroll
-    for (int i = 0; i < kVecB; ++i) {
-      const int v = tid + i * kThreads, r = v >> 3, c = v & 7;
-      *reinterpret_cast<u32x4_t*>(lds + buf * kBufBytes + (BM + r) * kRowStride + c * 16) = rb[i];
-    }
-  };
 
   floatx16_t acc[TM][TN];
 #pragma unroll
@@ -106,49 +84,102 @@ __global__ __launch_bounds__(kThreads) void proj_gemm_kernel(ProjArgs a) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  const int a_row = (wm * WM + l32) * kRowStride, b_row = (BM + wn * WN + l32) * kRowStride;
-  bf16x8_t fa[2][TM], fb[2][TN];
-  auto load_frags = [&](int buf, int sub, int slot) {
-    const char* pa = lds + buf * kBufBytes + a_row + sub * 32 + half * 16;
-    const char* pb = lds + buf * kBufBytes + b_row + sub * 32 + half * 16;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) fa[slot][i] = *reinterpret_cast<const bf16x8_t*>(pa + i * 32 * kRowStride);
-#pragma unroll
-    for (int j = 0; j < TN; ++j) fb[slot][j] = *reinterpret_cast<const bf16x8_t*>(pb + j * 32 * kRowStride);
+  // Operand tiles go from global memory straight into LDS (buffer_load ... lds): two stages of the token tile, three of
+  // the weight tile, 32 KB each, in un-padded 128-byte rows whose 16-byte units are XOR-swizzled by (row >> 1) & 7 (a
+  // direct load cannot pad: its 64 lanes fill 1 KB of LDS in lane order, so the swizzle is applied to the global
+  // address each lane fetches; operand reads stay conflict-free).  Token tile kt + 1 and weight tile kt + 2 are
+  // requested at the start of step kt; the wait in front of the step's barrier leaves the newest weight tile in
+  // flight.  A wavefront's load i covers rows (wave * 4 + i) * 8 .. + 8 of a tile.
+  constexpr int kStageBytes = 256 * 128;
+  const int dtl_row = lane >> 3, dtl_slot = lane & 7;
+  auto dtl_voff = [&](int i) {
+    const int row = (wave * 4 + i) * 8 + dtl_row;
+    return row * row_bytes_g + ((dtl_slot ^ ((row >> 1) & 7)) * 16);
   };
-  // While tile kt is multiplied out of LDS buffer kt & 1, tile kt + 1 (already in registers) is written to the other
-  // buffer during sub-step 1 and the global loads of tile kt + 2 are issued behind it; the barrier sits before the
-  // last sub-step's MFMAs, after that sub-step's fragments were read.
-  auto k_tile = [&](auto more_tag, int kt) {
-    constexpr bool kMore = decltype(more_tag)::value;
-    const int buf = kt & 1;
+  auto load_a = [&](int stage, int kt) {
 #pragma unroll
-    for (int sub = 0; sub < kSub; ++sub) {
-      if (sub + 1 < kSub) {
-        load_frags(buf, sub + 1, (sub + 1) & 1);
-      } else if (kMore) {
-        __syncthreads();
-        load_frags(buf ^ 1, 0, 0);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      if (sub == 1 && kMore) {
-        store_tile(buf ^ 1);
-        if (kt + 2 < k_tiles) load_tile(kt + 2);
+    for (int i = 0; i < 4; ++i)
+      MSA_LOAD_TO_LDS(rsrc_a, lds + stage * kStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes, 0);
+  };
+  auto load_b = [&](int stage, int kt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      MSA_LOAD_TO_LDS(rsrc_b, lds + (2 + stage) * kStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes, 0);
+  };
+  bf16x8_t fa[2][TM], fb[2][TN];
+  auto load_frags = [&](int sa, int sb, int sub, int slot) {
+    const int unit = sub * 2 + half;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int row = wm * WM + i * 32 + l32;
+      fa[slot][i] = *reinterpret_cast<const bf16x8_t*>(lds + sa * kStageBytes + row * 128 + ((unit ^ ((row >> 1) & 7)) * 16));
+    }
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int row = wn * WN + j * 32 + l32;
+      fb[slot][j] = *reinterpret_cast<const bf16x8_t*>(lds + (2 + sb) * kStageBytes + row * 128 + ((unit ^ ((row >> 1) & 7)) * 16));
+    }
+  };
+  // vmcnt(4) / vmcnt(0) with the other counters left alone: the four newest loads are the weight tile two steps ahead.
+  // The barrier is written out: __syncthreads() carries a release fence for which the compiler drains every load that
+  // writes LDS, the tile two steps ahead included.
+  constexpr int kWaitAllButNewestB = 0x0F74, kWaitAll = 0x0F70;
+  auto barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+  load_a(0, 0);
+  load_b(0, 0);
+  if (k_tiles > 1) {
+    load_b(1, 1);
+    __builtin_amdgcn_s_waitcnt(kWaitAllButNewestB);
+  } else {
+    __builtin_amdgcn_s_waitcnt(kWaitAll);
+  }
+  barrier();
+  load_frags(0, 0, 0, 0);
+  int sa = 0, sb = 0;
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    const int sb1 = sb == 2 ? 0 : sb + 1, sb2 = sb1 == 2 ? 0 : sb1 + 1;
+    const bool more = kt + 1 < k_tiles, more2 = kt + 2 < k_tiles;
+    if (more) load_a(sa ^ 1, kt + 1);       // stage of the step before this one: its last reads were behind the previous barrier
+    if (more2) load_b(sb2, kt + 2);
+    auto substep = [&](auto sub_tag, auto fresh_tag) {
+      constexpr int sub = decltype(sub_tag)::value;
+      constexpr bool fresh = decltype(fresh_tag)::value;
+      if constexpr (sub + 1 < kSub) {
+        load_frags(sa, sb, sub + 1, (sub + 1) & 1);
+      } else {
+        if (more) {
+          if (more2) __builtin_amdgcn_s_waitcnt(kWaitAllButNewestB);
+          else __builtin_amdgcn_s_waitcnt(kWaitAll);
+          barrier();
+          load_frags(sa ^ 1, sb1, 0, 0);
+          __builtin_amdgcn_sched_barrier(0);
+        }
       }
 #pragma unroll
       for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[sub & 1][i], fb[sub & 1][j], acc[i][j], 0, 0, 0);
-    }
-  };
-  load_tile(0);
-  store_tile(0);
-  if (k_tiles > 1) load_tile(1);
-  __syncthreads();
-  load_frags(0, 0, 0);
-  for (int kt = 0; kt + 1 < k_tiles; ++kt) k_tile(std::true_type{}, kt);
-  k_tile(std::false_type{}, k_tiles - 1);
+        for (int j = 0; j < TN; ++j) {
+          if constexpr (fresh) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[sub & 1][i], fb[sub & 1][j], floatx16_t{}, 0, 0, 0);
+          else acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[sub & 1][i], fb[sub & 1][j], acc[i][j], 0, 0, 0);
+        }
+      if constexpr (sub + 1 < kSub) {
+        // issue order of the sub-step: each of the six operand reads of the next sub-step behind one MFMA of this one
+#pragma unroll
+        for (int g = 0; g < TM + TN; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, TM * TN - TM - TN, 0);
+      }
+    };
+    if (kt == 0) substep(std::integral_constant<int, 0>{}, std::true_type{});
+    else substep(std::integral_constant<int, 0>{}, std::false_type{});
+    substep(std::integral_constant<int, 1>{}, std::false_type{});
+    substep(std::integral_constant<int, 2>{}, std::false_type{});
+    substep(std::integral_constant<int, 3>{}, std::false_type{});
+    sa ^= 1;
+    sb = sb1;
+  }
 
   // Epilogue: this wavefront holds head `head` for 64 tokens.  acc[i][j][e] is token row 8*(e/4) + 4*half + e%4 of
   // row block i, column j*32 + l32 of the head.
@@ -276,7 +307,7 @@ extern "C" int msa_qkv_proj(const void* x, int64_t T, int32_t K, const void* w, 
   const int groups = (m_per_xcd + a.m_group - 1) / a.m_group;
   const int64_t grid = (int64_t)8 * groups * a.m_group * a.tiles_n;
   MSA_REQUIRE(grid < ((int64_t)1 << 31), "msa_qkv_proj: grid too large");
-  const size_t lds = (size_t)2 * kBufBytes;
+  const size_t lds = (size_t)kLdsBytes;
   static std::atomic<int> lds_limit_raised{0};
   MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(proj_gemm_kernel), (int)lds));
   proj_gemm_kernel<<<(unsigned)grid, kThreads, lds, as_stream(stream)>>>(a);

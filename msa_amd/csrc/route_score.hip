@@ -20,15 +20,6 @@ namespace {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) void* lds_ptr_t;
-// 16 bytes per lane from a buffer resource straight into LDS (lane l lands at byte 16 * l behind `lds_dst`, which must be
-// the same in every lane).  The compiler's host pass has no such instruction and only needs the kernel's signature.
-#if defined(__HIP_DEVICE_COMPILE__)
-#define MSA_LOAD_TO_LDS(rsrc, lds_dst, voffset, soffset, aux) \
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(lds_dst), 16, voffset, soffset, 0, aux)
-#else
-#define MSA_LOAD_TO_LDS(rsrc, lds_dst, voffset, soffset, aux) ((void)(rsrc), (void)(lds_dst), (void)(voffset), (void)(soffset))
-#endif
 
 // ------------------------------------------------------------------------------------------
 // Prologue: normalise (cosine mode), sum the G heads of each KV group, cast, build row masks, clear the key plane.

@@ -64,7 +64,10 @@ __global__ __launch_bounds__(kThreads) void proj_gemm_kernel(ProjArgs a) {
   if (tile_m >= a.tiles_m || tile_m >= (int)(blockIdx.x % 8 + 1) * m_per_xcd) return;
   const int m0 = tile_m * BM, n0 = tile_n * BN;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  // (wave-uniform by construction; said so, the LDS addresses of the direct loads stay in scalar registers instead of
+  // being read back from a lane in front of every load: 1.9 % on the large-tile scan)
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
   const int half = lane >> 5, l32 = lane & 31;
 

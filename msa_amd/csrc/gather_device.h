@@ -118,39 +118,43 @@ __device__ __forceinline__ void copy_body(const uint4* __restrict__ k_src, const
                                           int64_t capacity_rows, uint4* k_dst, uint4* v_dst, int ent0, int ent_step,
                                           int r0, int r_step, int lane_in_row) {
   const int row_bytes = row_vecs * 16;
+  // Everything that names a row is the same in all lanes of a wavefront (128 lanes share a row).  Said so, the rows'
+  // buffer resources are built in scalar registers; left as vector values every load and store sat in a loop that
+  // reads the resource back lane by lane.
+  const int r0s = __builtin_amdgcn_readfirstlane(r0), r_steps = __builtin_amdgcn_readfirstlane(r_step);
   for (int ent = ent0; ent < n_entries; ent += ent_step) {
     const int32_t* e = plan + (int64_t)ent * kPlanInts;
-    const int32_t n = e[1], dst0 = e[2], from = e[3];
+    const int32_t n = __builtin_amdgcn_readfirstlane(e[1]), dst0 = __builtin_amdgcn_readfirstlane(e[2]);
+    const int32_t from = __builtin_amdgcn_readfirstlane(e[3]);
     if ((from >= 0) != kFromDevice) continue;
-    const int32_t src0 = kFromDevice ? from : e[0];
-    for (int r = r0; r < n; r += r_step * kRows) {
-      __amdgpu_buffer_rsrc_t rks[kRows], rvs[kRows], rkd[kRows], rvd[kRows];
-#pragma unroll
-      for (int j = 0; j < kRows; ++j) {
-        const int64_t rj = (int64_t)r + (int64_t)j * r_step;
-        // a row past the entry's end, or past the capacity on either side, gets an empty extent: its loads return
-        // zeros without traffic and its stores are dropped
+    const int32_t src0 = kFromDevice ? from : __builtin_amdgcn_readfirstlane(e[0]);
+    for (int r = r0s; r < n; r += r_steps * kRows) {
+      // a row past the entry's end, or past the capacity on either side, gets an empty extent: its loads return zeros
+      // without traffic and its stores are dropped.  The resources are built where they are used (a handful of scalar
+      // instructions each) instead of being kept: 4 per row would not fit the scalar registers.
+      auto row_of = [&](int j, int64_t& rr, int& ext) {
+        const int64_t rj = (int64_t)r + (int64_t)j * r_steps;
         const bool live = rj < n && dst0 + rj < capacity_rows && (!kFromDevice || src0 + rj < capacity_rows);
-        const int64_t rr = live ? rj : 0;
-        const int ext = live ? row_bytes : 0;
-        const uint4* ks = (kFromDevice ? k_dst : k_src) + (src0 + rr) * row_vecs;
-        const uint4* vs = (kFromDevice ? v_dst : v_src) + (src0 + rr) * row_vecs;
-        rks[j] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(ks), 0, ext, 0x00020000);
-        rvs[j] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(vs), 0, ext, 0x00020000);
-        rkd[j] = __builtin_amdgcn_make_buffer_rsrc(k_dst + (dst0 + rr) * row_vecs, 0, ext, 0x00020000);
-        rvd[j] = __builtin_amdgcn_make_buffer_rsrc(v_dst + (dst0 + rr) * row_vecs, 0, ext, 0x00020000);
-      }
+        rr = live ? rj : 0;
+        ext = live ? row_bytes : 0;
+      };
       for (int off = lane_in_row * 16; off < row_bytes; off += kCopyRowLanes * 16) {
         u32x4_t a[kRows], b[kRows];
 #pragma unroll
         for (int j = 0; j < kRows; ++j) {
-          a[j] = __builtin_amdgcn_raw_buffer_load_b128(rks[j], off, 0, 0);
-          b[j] = __builtin_amdgcn_raw_buffer_load_b128(rvs[j], off, 0, 0);
+          int64_t rr; int ext;
+          row_of(j, rr, ext);
+          const uint4* ks = (kFromDevice ? k_dst : k_src) + (src0 + rr) * row_vecs;
+          const uint4* vs = (kFromDevice ? v_dst : v_src) + (src0 + rr) * row_vecs;
+          a[j] = __builtin_amdgcn_raw_buffer_load_b128(__builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(ks), 0, ext, 0x00020000), off, 0, 0);
+          b[j] = __builtin_amdgcn_raw_buffer_load_b128(__builtin_amdgcn_make_buffer_rsrc(const_cast<uint4*>(vs), 0, ext, 0x00020000), off, 0, 0);
         }
 #pragma unroll
         for (int j = 0; j < kRows; ++j) {
-          __builtin_amdgcn_raw_buffer_store_b128(a[j], rkd[j], off, 0, 0);
-          __builtin_amdgcn_raw_buffer_store_b128(b[j], rvd[j], off, 0, 0);
+          int64_t rr; int ext;
+          row_of(j, rr, ext);
+          __builtin_amdgcn_raw_buffer_store_b128(a[j], __builtin_amdgcn_make_buffer_rsrc(k_dst + (dst0 + rr) * row_vecs, 0, ext, 0x00020000), off, 0, 0);
+          __builtin_amdgcn_raw_buffer_store_b128(b[j], __builtin_amdgcn_make_buffer_rsrc(v_dst + (dst0 + rr) * row_vecs, 0, ext, 0x00020000), off, 0, 0);
         }
       }
     }

@@ -9,16 +9,25 @@
 //   O^T[128 dims x 32 cols] += V^T . P^T      (contraction over keys).
 // S^T's accumulator layout IS the B-operand layout of the second product (same lane, same
 // column), up to the order of keys inside a group of 16, which the V^T operand mirrors, so P never
-// leaves registers.  V goes into LDS as it lies in memory ([key][dim] rows, 16-byte stores) and the
-// V^T operand comes out of gfx950's transposing LDS read (ds_read_b64_tr_b16): sixteen lanes hand in
-// the sixteen 8-byte pieces of four key rows x 16 dims and lane j of them receives dim j of the four
-// keys, so the transpose costs no instruction and the key order is whatever rows the lanes name.
+// leaves registers.  V lies in LDS as it lies in memory ([key][dim] rows) and the V^T operand comes
+// out of gfx950's transposing LDS read (ds_read_b64_tr_b16): sixteen lanes hand in the sixteen
+// 8-byte pieces of four key rows x 16 dims and lane j of them receives dim j of the four keys, so
+// the transpose costs no instruction and the key order is whatever rows the lanes name.
+//
+// Tiles travel from memory straight into LDS (buffer loads with the LDS bit: no staging registers,
+// no LDS store instructions) through a ring of three K tiles and two V tiles (80 KB, so two
+// workgroups share a compute unit and one computes while the other starts or ends): iteration t
+// reads K(t + 1) and V(t) while K(t + 2) lands and V(t + 1) and K(t + 3) are loaded into the slots
+// iteration t - 1 read.  Such a load writes a wavefront's 64 x 16 bytes contiguously, so rows are
+// unpadded (256 bytes) and bank conflicts are avoided by which 16-byte piece a lane fetches: piece
+// c of K row r sits at position c ^ (r & 15) (the score product reads one piece of 16 consecutive
+// rows at a time), piece c of V row r at c ^ ((r & 3) << 2) (a transposing read takes 64 bytes of
+// four consecutive rows).
 //
 // The loop is software-pipelined inside the wavefront: the scores of tile t + 1 are produced in the
 // same straight-line block as the exponentials of tile t, and an explicit issue order (scheduling
 // groups) puts the LDS reads two products ahead of their use, so one wavefront keeps the matrix pipe,
-// the VALU and the LDS busy at once.  K and V are double-buffered out of phase (iteration t reads
-// K(t + 1) and V(t) and stores K(t + 2) and V(t + 1)), one barrier per tile.
+// the VALU and the LDS busy at once.  One barrier per tile.
 #include "attn_internal.h"
 
 namespace {
@@ -32,12 +41,14 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16_t;
 
 constexpr int kKeysPerTile = 64;
-constexpr int kTileStride = 2 * kHeadDim + 16;   // bytes per key row in LDS: 256 + 16 pad (conflict-free b128 reads)
-constexpr int kVStride = 2 * kHeadDim + 64;      // bytes per key row of the V tile: four consecutive keys x 64 bytes
-                                                  // (one transposing read of a half-wave) cover all 64 banks once
-constexpr int kStageBytes = kKeysPerTile * (kTileStride + kVStride);   // one K tile + one V tile
+constexpr int kRowBytes = 2 * kHeadDim;                    // a key row of one KV head
+constexpr int kTileBytes = kKeysPerTile * kRowBytes;       // 16 KB, rows unpadded (see the swizzles above)
+constexpr int kRingK = 3, kRingV = 2;                      // tiles of K and of V resident or in flight
+constexpr int kVBase = kRingK * kTileBytes;                // the V ring lies behind the K ring
 constexpr int kWaves = 4;
-constexpr int kLdsBytes = 2 * kStageBytes;
+constexpr int kLdsBytes = (kRingK + kRingV) * kTileBytes;  // 80 KB: two workgroups per compute unit
+// s_waitcnt immediates: vector-memory loads return in order, so "at most n outstanding" names the oldest ones done
+constexpr int kWaitVm0 = 0x0F70, kWaitVm4 = 0x0F74, kWaitVm12 = 0x0F7C;
 
 // max / sum of a value over the two half-waves (lane and lane ^ 32), by the half-wave swap instruction
 __device__ __forceinline__ float half_wave_max(float x) {
@@ -66,6 +77,23 @@ __device__ __forceinline__ shortx4_t lds_read_tr16(const char* p) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_shortx4_t*)(p));
 }
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) char lds_char_t;
+
+__device__ __forceinline__ uint32_t lds_address(char* p) { return (uint32_t)(uintptr_t)(lds_char_t*)p; }
+
+// 16 bytes per lane from a buffer resource straight into LDS: lane l lands at byte lds_dst + 16 l (lds_dst the same in
+// every lane, and handed over in a scalar register).  Written as an asm statement, not through the compiler's builtin,
+// so that the compiler does not know of a load in flight that writes LDS: it would drain all of them (vmcnt(0)) in
+// front of the first transposing LDS read of every iteration, whose address it cannot tell from the loads' targets.
+// The waits are the kernel's own (see the ring).  The wait states in front of the load cover a resource or an M0 that
+// the preceding instruction wrote.  Nothing else in this kernel depends on M0.
+__device__ __forceinline__ void load_to_lds(u32x4_t rsrc, uint32_t lds_dst, int voffset) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_dst), "v"(voffset), "s"(rsrc));
+#endif
+}
+
 // kSplit: blockIdx.z selects a range of split_keys keys; the un-normalised accumulators and the
 // (reference max, sum) pair of every column go to part_acc / part_ml for the combine kernel.
 template <int G, bool kSplit>
@@ -76,12 +104,17 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
     int32_t split_keys, float* __restrict__ part_ml, float* __restrict__ part_acc) {
   constexpr int kTokPerWave = 32 / G;
   constexpr int kTokPerBlock = kWaves * kTokPerWave;
-  constexpr int kLoads = kKeysPerTile * 16 / (kWaves * 64);   // 16-byte pieces of a K (or V) tile per thread
-  extern __shared__ __align__(16) char lds[];                  // 2 x [K tile | V tile]
-  constexpr int kVOffset = kKeysPerTile * kTileStride;
+  constexpr int kLoads = kTileBytes / (kWaves * 64 * 16);     // load instructions per wavefront, tile and tensor
+  extern __shared__ __align__(16) char lds[];                  // [K ring | V ring]
 
   // which (sample, token block) is this workgroup?  B is small; the scan is uniform.
-  int blk = blockIdx.x, b = 0;
+  // Workgroups go to the eight XCDs round-robin in launch order and each XCD has an L2 of its own (4 MiB).  With the
+  // KV head as the fastest index an XCD keeps to one head (eight of them) or a few, and the workgroups resident on
+  // it at one time are neighbouring token blocks of one sample: they stream the same 2 MB of K and V, which stay in
+  // that L2.  With the head as a grid dimension of its own every XCD held blocks of several samples at once, more
+  // K / V than its L2 takes, and most tile loads came from beyond it.
+  const int g = blockIdx.x % Hkv;
+  int blk = blockIdx.x / Hkv, b = 0;
   bool found = false;
   for (; b < B; ++b) {
     const int sq_b = cu_q ? cu_q[b + 1] - cu_q[b] : 1;
@@ -90,14 +123,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
     blk -= nb;
   }
   if (!found) return;
-  const int g = blockIdx.y;
   const int q_first = cu_q ? cu_q[b] : b;
   const int sq = cu_q ? cu_q[b + 1] - q_first : 1;
   const int t0 = blk * kTokPerBlock;
   const int L = kv_len[b];
   const int64_t base = kv_off[b];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int col = lane & 31, half = lane >> 5;
   const int tok = t0 + wave * kTokPerWave + col / G;       // token within the sample
   const int head = g * G + col % G;
@@ -135,58 +167,91 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
 #pragma unroll
   for (int x = 32; x > 0; x >>= 1) wave_min_limit = min(wave_min_limit, __shfl_xor(wave_min_limit, x));
 
-  uint4 rk[kLoads], rv[kLoads];
   // Tile loads through buffer resources rebuilt per tile (scalar work only): the extent covers the tile's valid
-  // keys, so rows past the last key read as zero in hardware and a thread's offset never changes.
+  // keys and a lane's offset never changes.  Load instruction i of a wavefront fills the 1 KB block of rows
+  // 4 (kLoads wave + i) .. + 4: lane l lands at row l / 16, position l % 16 and fetches the piece that belongs there.
+  // K rows past the last key may hold anything (their scores are masked by a select); V rows past it are multiplied
+  // by probabilities of zero and must be finite, so those lanes fetch the last valid row again.
   const int row_bytes = row_elems * 2;
-  const int voff0 = (tid >> 4) * row_bytes + (tid & 15) * 16;
-  auto gload_one = [&](const bf16_t* src, uint4 (&r)[kLoads], int t) {
-    const int rows = min(kKeysPerTile, kmax - t * kKeysPerTile);
-    const char* at = reinterpret_cast<const char*>(src) + ((base + (int64_t)t * kKeysPerTile) * row_elems + g * kHeadDim) * 2;
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<char*>(at), 0, max(0, (rows - 1) * row_bytes + 2 * kHeadDim), 0x00020000);   // 0 when no row is left
+  int tile_row[kLoads], k_piece[kLoads], v_piece[kLoads];
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) {
+    tile_row[i] = 4 * (kLoads * wave + i) + (lane >> 4);
+    k_piece[i] = ((lane & 15) ^ (tile_row[i] & 15)) * 16;
+    v_piece[i] = ((lane & 15) ^ ((tile_row[i] & 3) << 2)) * 16;
+  }
+  auto tile_rsrc = [&](const bf16_t* src, int t, int& rows) -> u32x4_t {
+    rows = min(kKeysPerTile, kmax - t * kKeysPerTile);
+    const uintptr_t at = reinterpret_cast<uintptr_t>(src) + ((base + (int64_t)t * kKeysPerTile) * row_elems + g * kHeadDim) * 2;
+    return u32x4_t{(uint32_t)at, (uint32_t)(at >> 32) & 0xffffu, (uint32_t)max(0, (rows - 1) * row_bytes + kRowBytes),
+                   0x00020000u};                                                            // extent 0 when no row is left
+  };
+  const uint32_t lds_wave = lds_address(lds) + kLoads * wave * 1024;     // this wavefront's first block of a tile
+  auto issue_k = [&](int t, int slot) {
+    int rows;
+    const u32x4_t rsrc = tile_rsrc(k, t, rows);
 #pragma unroll
     for (int i = 0; i < kLoads; ++i)
-      r[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, voff0 + i * (kWaves * 4) * row_bytes, 0, 0));
+      load_to_lds(rsrc, lds_wave + slot * kTileBytes + i * 1024, tile_row[i] * row_bytes + k_piece[i]);
   };
-  auto store_k = [&](int slot) {
+  auto issue_v = [&](int t, int slot) {
+    int rows;
+    const u32x4_t rsrc = tile_rsrc(v, t, rows);
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) {
-      const int vv = tid + i * kWaves * 64;
-      *reinterpret_cast<uint4*>(lds + slot * kStageBytes + (vv >> 4) * kTileStride + (vv & 15) * 16) = rk[i];
-    }
+    for (int i = 0; i < kLoads; ++i)
+      load_to_lds(rsrc, lds_wave + kVBase + slot * kTileBytes + i * 1024,
+                  min(tile_row[i], rows - 1) * row_bytes + v_piece[i]);                      // rows <= 0: out of range
   };
-  auto store_v = [&](int slot) {
+  // a barrier that waits for this wavefront's LDS reads but not for its loads in flight
+  auto ring_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+  // per-lane read positions inside a tile: K piece 2 ks + half of row col (+ 32 rb), V as the transposing read
+  // wants it (rows 4 half + r of a group of 8, 64 bytes at dims 32 d, r = (lane % 16) / 4)
+  int k_at[8], v_at[4];
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) {
-      const int vv = tid + i * kWaves * 64;
-      *reinterpret_cast<uint4*>(lds + slot * kStageBytes + kVOffset + (vv >> 4) * kVStride + (vv & 15) * 16) = rv[i];
-    }
-  };
-  const char* k_lane = lds + col * kTileStride + half * 16;
-  const char* v_lane = lds + kVOffset + (4 * half + ((lane & 15) >> 2)) * kVStride + (lane & 16) * 2 + (lane & 3) * 8;
+  for (int ks = 0; ks < 8; ++ks) k_at[ks] = col * kRowBytes + (((2 * ks + half) ^ (col & 15)) * 16);
+  {
+    const int r = (lane & 15) >> 2;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+      v_at[d] = kVBase + (4 * half + r) * kRowBytes + ((d ^ r) * 64) + (lane & 16) * 2 + (lane & 3) * 8;
+  }
 
-  auto step = [&](int t, floatx16_t (&sc)[2], floatx16_t (&sn)[2]) {
-    const int slot = (t - first_tile) & 1;
-    // (A) mask, column maximum
+  // masks the scores of tile t past the column's last visible key and returns their maximum; `between(i)`, i = 0..3,
+  // is called at four points spread over the work (the caller's matrix products, so that they issue among these
+  // VALU instructions whichever way the branch goes)
+  auto tile_max = [&](int t, floatx16_t (&sx)[2], auto between) -> float {
     const int key_base = t * kKeysPerTile + 4 * half;
-    float mx_raw = -INFINITY;
+    float mx_t = -INFINITY;
     if ((t + 1) * kKeysPerTile <= wave_min_limit) {
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) mx_raw = fmaxf(mx_raw, sc[rb][e]);
+        for (int e = 0; e < 16; ++e) {
+          if ((e & 7) == 0) { between(2 * rb + (e >> 3)); __builtin_amdgcn_sched_barrier(0); }
+          mx_t = fmaxf(mx_t, sx[rb][e]);
+        }
     } else {
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
         for (int e = 0; e < 16; ++e) {
+          if ((e & 7) == 0) { between(2 * rb + (e >> 3)); __builtin_amdgcn_sched_barrier(0); }
           const int key = key_base + 32 * rb + 8 * (e >> 2) + (e & 3);
-          const float x = key < limit ? sc[rb][e] : -INFINITY;
-          sc[rb][e] = x;
-          mx_raw = fmaxf(mx_raw, x);
+          const float x = key < limit ? sx[rb][e] : -INFINITY;
+          sx[rb][e] = x;
+          mx_t = fmaxf(mx_t, x);
         }
     }
+    return mx_t;
+  };
+  float mx_raw = -INFINITY;                  // of the tile the next step consumes
+  int ring = 0;                              // (t - first_tile) % kRingK: the slot of K(t)
+  auto step = [&](int t, floatx16_t (&sc)[2], floatx16_t (&sn)[2]) {
+    const int ring1 = ring == kRingK - 1 ? 0 : ring + 1;
+    const int vslot = (t - first_tile) & 1;  // the slot of V(t)
+    issue_v(t + 1, vslot ^ 1);               // V(t - 1)'s slot: last read before the previous barrier
+    issue_k(t + 3, ring);                    // K(t)'s slot: likewise
+    // (A) the column maximum of this tile's (masked) scores came with the scores: `mx_raw`
     float mx = fmaxf(m, mx_raw * scale_log2e);
     mx = half_wave_max(mx);
     const bool none = mx == -INFINITY;
@@ -203,102 +268,94 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
       m = mref;
     }
     const float neg_m = none ? 0.f : -m;
-    // (C) scores of tile t + 1 next to the exponentials of tile t (the K slot holds zeros past the last tile)
-    const char* kn = k_lane + (slot ^ 1) * kStageBytes;
+    // (C) / (D) the 16 products of the scores of tile t + 1 (the K slot holds anything past the last tile: never used),
+    // the 16 products O^T += V^T . P^T of tile t, and this tile's 32 exponentials in 16 pairs, in an issue order that
+    // is written out slot by slot and fenced (the scheduler may not move anything across a slot's end):
+    // (slots  0 .. 15: score product s, an exponential pair behind every second one; 16 .. 27: O product, the other
+    // pairs; 28 .. 31: O product, the column maximum of the new scores), so that a matrix product has at most VALU
+    // work of its own length issued behind it, and each LDS read is issued two products ahead of its use.
+    const char* kn = lds + ring1 * kTileBytes;
+    const char* vt = lds + vslot * kTileBytes;
     float psum = 0.f;
-    bf16x8_t pf[2][2];
-    bf16x8_t kf[3][2];                      // K operands, fetched two steps ahead of their products
+    uint32_t pw[2][2][4];                   // P as packed bf16 pairs: [key rows 32 rb ..][16 j ..][pair]
+    constexpr int kKAhead = 6, kKRing = 4;  // K operand reads issued this many products ahead; ring of score steps
+    constexpr int kVAhead = 4, kVRing = 5;  // V^T operands read this many products ahead; ring of operands
+    bf16x8_t kf[kKRing][2];
+    bf16x8_t va[kVRing];
+    auto k_read = [&](int i) {              // i = 2 ks + rb
+      kf[(i >> 1) % kKRing][i & 1] = *reinterpret_cast<const bf16x8_t*>(kn + k_at[i >> 1] + (i & 1) * 32 * kRowBytes);
+    };
+    auto qk = [&](int i) {
+      const int ks = i >> 1, rb = i & 1;
+      if (ks == 0) {
+        floatx16_t z;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-      for (int rb = 0; rb < 2; ++rb)
-        kf[ks][rb] = *reinterpret_cast<const bf16x8_t*>(kn + rb * 32 * kTileStride + ks * 32);
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      if (ks + 2 < 8) {
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-          kf[(ks + 2) % 3][rb] = *reinterpret_cast<const bf16x8_t*>(kn + rb * 32 * kTileStride + (ks + 2) * 32);
+        for (int e = 0; e < 16; ++e) z[e] = 0.f;
+        sn[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0][rb], qf[0], z, 0, 0, 0);
+      } else {
+        sn[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks % kKRing][rb], qf[ks], sn[rb], 0, 0, 0);
       }
+    };
+    auto exp_pair = [&](int gi) {           // elements 2 (gi % 8), + 1 of sc[gi / 8]
+      const int prb = gi >> 3, e0 = (gi & 7) * 2;
+      const float p0 = fast_exp2(fmaf(sc[prb][e0], scale_log2e, neg_m));
+      const float p1 = fast_exp2(fmaf(sc[prb][e0 + 1], scale_log2e, neg_m));
+      const uint32_t pk = pack_pair(p0, p1);
+      psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), psum, false);
+      pw[prb][(gi & 7) >> 2][gi & 3] = pk;
+    };
+    auto v_read = [&](int i) {              // i = (2 rb + j) * 4 + d
+      const char* at = vt + v_at[i & 3] + 16 * (i >> 2) * kRowBytes;
+      const shortx4_t lo = lds_read_tr16(at), hi = lds_read_tr16(at + 8 * kRowBytes);
+      va[i % kVRing] = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+    auto pv = [&](int i) {
+      const int rbj = i >> 2, d = i & 3;
+      const u32x4_t pwv = {pw[rbj >> 1][rbj & 1][0], pw[rbj >> 1][rbj & 1][1], pw[rbj >> 1][rbj & 1][2], pw[rbj >> 1][rbj & 1][3]};
+      o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[i % kVRing], __builtin_bit_cast(bf16x8_t, pwv), o[d], 0, 0, 0);
+    };
+    auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+    fence();
 #pragma unroll
-      for (int rb = 0; rb < 2; ++rb) {
-        if (ks == 0) {
-          floatx16_t z;
+    for (int i = 0; i < kKAhead; ++i) k_read(i);
+    fence();
 #pragma unroll
-          for (int e = 0; e < 16; ++e) z[e] = 0.f;
-          sn[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[0][rb], qf[0], z, 0, 0, 0);
-        } else {
-          sn[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[ks % 3][rb], qf[ks], sn[rb], 0, 0, 0);
-        }
-        // two of this tile's 32 probabilities per product
-        const int prb = ks >> 2, e0 = (ks & 3) * 4 + 2 * rb;
-        const float p0 = fast_exp2(fmaf(sc[prb][e0], scale_log2e, neg_m));
-        const float p1 = fast_exp2(fmaf(sc[prb][e0 + 1], scale_log2e, neg_m));
-        const uint32_t pk = pack_pair(p0, p1);
-        psum = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), psum, false);
-        pf[prb][e0 >> 3][e0 & 7] = __builtin_bit_cast(bf16x2_t, pk)[0];
-        pf[prb][e0 >> 3][(e0 & 7) + 1] = __builtin_bit_cast(bf16x2_t, pk)[1];
-      }
+    for (int sl = 0; sl < 16; ++sl) {
+      if (sl + kKAhead < 16) k_read(sl + kKAhead);
+      qk(sl);
+      if (sl & 1) exp_pair(sl >> 1);
+      if (sl >= 16 - kVAhead) v_read(sl - (16 - kVAhead));
+      fence();
     }
+#pragma unroll
+    for (int u = 0; u < 12; ++u) {
+      if (u + kVAhead < 16) v_read(u + kVAhead);
+      pv(u);
+      if (u < 8 && !(u & 1)) exp_pair(8 + (u >> 1));
+      if (u >= 8) exp_pair(4 + u);
+      fence();
+    }
+    // the last O products share their issue slots with the maximum of the scores just finished (the next tile's)
+    mx_raw = tile_max(t + 1, sn, [&](int i) {
+      if (i + 12 + kVAhead < 16) v_read(i + 12 + kVAhead);
+      pv(i + 12);
+    });
+    fence();
     l += half_wave_sum(psum);
-    // (D) O^T += V^T . P^T from this tile's V slot; refill the slots that are free
-    const char* vt = v_lane + slot * kStageBytes;
-#pragma unroll
-    for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int d = 0; d < 4; ++d) {
-          const char* at = vt + (32 * rb + 16 * j) * kVStride + 64 * d;
-          const shortx4_t lo = lds_read_tr16(at), hi = lds_read_tr16(at + 8 * kVStride);
-          const bf16x8_t a = __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
-          o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pf[rb][j], o[d], 0, 0, 0);
-        }
-    store_k(slot);           // K(t + 2): this slot's K was last read before the previous barrier
-    store_v(slot ^ 1);       // V(t + 1): that slot's V was last read before the previous barrier
-    gload_one(k, rk, t + 3);
-    gload_one(v, rv, t + 2);
-    // Issue order of the straight-line part above: every matrix product is followed by the LDS reads of operands
-    // two products ahead and by a share of the exponentials, so neither the reads' latency nor the VALU work
-    // leaves the matrix pipe idle; the tile stores and loads ride behind the last products.
-    __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
-#pragma unroll
-    for (int i = 0; i < 12; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
-    }
-#pragma unroll
-    for (int i = 0; i < 12; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
-      __builtin_amdgcn_sched_group_barrier(0x002, 1, 0);
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x200, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-    }
-    __syncthreads();
+    // K(t + 2), issued an iteration ago, and V(t + 1) have landed once only the loads of K(t + 3) are outstanding
+    __builtin_amdgcn_s_waitcnt(kWaitVm4);
+    ring_barrier();
+    ring = ring1;
   };
 
+  static_assert(kLoads == 4, "the wait counts assume four loads per wavefront, tile and tensor");
   if (first_tile < n_tiles) {
-    gload_one(k, rk, first_tile);
-    gload_one(v, rv, first_tile);
-    store_k(0);
-    store_v(0);
-    gload_one(k, rk, first_tile + 1);
-    store_k(1);
-    gload_one(k, rk, first_tile + 2);
-    gload_one(v, rv, first_tile + 1);
-    __syncthreads();
+    issue_k(first_tile, 0);
+    issue_v(first_tile, 0);
+    issue_k(first_tile + 1, 1);
+    issue_k(first_tile + 2, 2);
+    __builtin_amdgcn_s_waitcnt(kWaitVm12);     // K(first) has landed
+    ring_barrier();
     floatx16_t s0[2], s1[2];
 #pragma unroll
     for (int rb = 0; rb < 2; ++rb)
@@ -308,16 +365,19 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
     for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
       for (int rb = 0; rb < 2; ++rb) {
-        const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(k_lane + rb * 32 * kTileStride + ks * 32);
+        const bf16x8_t a = *reinterpret_cast<const bf16x8_t*>(lds + k_at[ks] + rb * 32 * kRowBytes);
         s0[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[ks], s0[rb], 0, 0, 0);
       }
-    // the first step overwrites K slot 0 (with tile first + 2) before its own barrier: every wavefront must have
-    // finished the reads of slot 0 above before any wavefront gets there
-    __syncthreads();
+    // the first step reads V(first) and K(first + 1), and loads K(first + 3) over K(first): every wavefront must
+    // have those two and be done with the reads above before any wavefront gets there
+    __builtin_amdgcn_s_waitcnt(kWaitVm4);
+    ring_barrier();
+    mx_raw = tile_max(first_tile, s0, [](int) {});
     for (int t = first_tile; t < n_tiles; t += 2) {
       step(t, s0, s1);
       if (t + 1 < n_tiles) step(t + 1, s1, s0);
     }
+    __builtin_amdgcn_s_waitcnt(kWaitVm0);      // nothing may still be writing LDS when the workgroup ends
   }
 
   if constexpr (kSplit) {
@@ -353,10 +413,10 @@ int flash_launch_g(const void* q, const int32_t* cu_q, const void* k, const void
                    int32_t causal, void* out, SplitPlan plan, float* part_ml, float* part_acc, hipStream_t st) {
   constexpr int kTokPerBlock = kWaves * 32 / G;
   const int64_t blocks = ((int64_t)total_q + kTokPerBlock - 1) / kTokPerBlock + B;   // upper bound over ragged samples
-  MSA_REQUIRE(blocks < (int64_t)1 << 31, "flash attention: too many query rows");
-  dim3 grid((unsigned)blocks, (unsigned)Hkv, kSplit ? (unsigned)plan.n_split : 1u);
+  MSA_REQUIRE(blocks * Hkv < (int64_t)1 << 31, "flash attention: too many query rows");
+  dim3 grid((unsigned)(blocks * Hkv), 1u, kSplit ? (unsigned)plan.n_split : 1u);
   auto kern = flash_attn_kernel<G, kSplit>;
-  static std::atomic<int> lds_limit_raised{0};   // two tiles of K and V exceed the default dynamic LDS limit
+  static std::atomic<int> lds_limit_raised{0};   // the K and V rings exceed the default dynamic LDS limit
   MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(kern), kLdsBytes));
   kern<<<grid, kWaves * 64, kLdsBytes, st>>>(static_cast<const bf16_t*>(q), cu_q, static_cast<const bf16_t*>(k),
                                              static_cast<const bf16_t*>(v), kv_off, kv_len, B, Hq, Hkv,

@@ -229,13 +229,17 @@ def extra_mfma_ceiling(dev):
     occupancy): the rate with operands that toggle is the ceiling the scoring kernel's fraction can be read against."""
     from msa_amd import _lib
     lib = _lib.load()
-    wgs, iters = 256 * 4, 40000
+    wgs, iters = 256 * 4, 20000
     sink = torch.empty(wgs * 512, dtype=torch.float32, device=dev)
     flops = C.c_double(0)
     out = {"workload": f"register-only v_mfma_f32_32x32x16_bf16 loop, {wgs} workgroups x 8 wavefronts x {iters} x 8 MFMAs"}
-    for mode, name in ((0, "zero_operands"), (2, "toggling_operands")):
+    # mode + 16 * extra: other VALU work per 8 MFMAs (what the attention kernel's softmax asks of the issue port)
+    for mode, name in ((0, "zero_operands"), (2, "toggling_operands"), (16, "zero_operands_plus_24_fma"),
+                       (32, "zero_operands_plus_48_fma"), (48, "zero_operands_plus_24_exp"), (64, "zero_operands_plus_48_exp"),
+                       (80, "zero_operands_plus_24_cvt_pk_bf16"), (96, "zero_operands_plus_24_dot2c_bf16"),
+                       (112, "zero_operands_plus_24_max3")):
         ms = []
-        for rep in range(4):
+        for rep in range(3):
             a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             a.record()
             _lib.check(lib.msa_diag_mfma_loop(wgs, iters, mode, sink.data_ptr(), C.byref(flops), torch.cuda.current_stream().cuda_stream),

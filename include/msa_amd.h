@@ -140,7 +140,11 @@ int msa_profile_collect(float* ms_host, int32_t cap, int32_t* n_out);
  * sink[thread] then holds 128 * iters exactly); 2: operands whose signs and mantissas change every iteration, which is
  * what the shader clock under real data answers to.  sink: device float [workgroups * 512]; *flops_out (host, may be
  * null) receives the launch's floating-point operations.  The rate of mode 2 is the ceiling of this GPU's matrix
- * cores under load, below the published peak, which assumes the boost clock. */
+ * cores under load, below the published peak, which assumes the boost clock.
+ * mode + 16 * extra adds other VALU work per iteration of 8 MFMAs, on registers of its own (sink is then not
+ * defined): extra 1 / 2: 24 / 48 v_fma_f32; 3 / 4: 24 / 48 v_exp_f32; 5: 24 v_cvt_pk_bf16_f32; 6: 24 v_dot2c_f32_bf16;
+ * 7: 24 v_max3_f32.  The rates tell what each instruction costs on the SIMD's issue port next to the products
+ * (the budget of a kernel that does softmax arithmetic between them). */
 int msa_diag_mfma_loop(int32_t workgroups, int32_t iters, int32_t mode, float* sink, double* flops_out, void* stream);
 
 /* ---------------------------------------------------------------------------------------------

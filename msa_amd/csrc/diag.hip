@@ -13,7 +13,11 @@ constexpr int kThreads = 512;          // 8 wavefronts, two per SIMD: the scorin
 constexpr int kMfmasPerIter = 8;       // a 4 x 2 grid of 32 x 32 accumulators per wavefront, as in the scoring kernel
 
 // mode 0: zero operands; 1: all ones (the result is known exactly: 16 per MFMA); 2: operands whose mantissas and signs
-// change from one iteration to the next (what a GEMM on real data presents to the multipliers)
+// change from one iteration to the next (what a GEMM on real data presents to the multipliers).
+// kExtra: other VALU work per iteration of 8 MFMAs, on registers of its own (what a kernel that does arithmetic on its
+// accumulators between the products, such as the softmax of an attention kernel, asks of the SIMD's issue port):
+// 0 none; 1 / 2: 24 / 48 v_fma_f32; 3 / 4: 24 / 48 v_exp_f32; 5: 24 v_cvt_pk_bf16_f32; 6: 24 v_dot2c_f32_bf16; 7: 24 v_max3_f32.
+template <int kExtra>
 __global__ __launch_bounds__(kThreads) void mfma_loop_kernel(int32_t iters, int32_t mode, float* __restrict__ sink) {
   const uint32_t tid = blockIdx.x * kThreads + threadIdx.x;
   u32x4_t a[4], b[2];
@@ -36,6 +40,11 @@ __global__ __launch_bounds__(kThreads) void mfma_loop_kernel(int32_t iters, int3
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float floatx2_t __attribute__((ext_vector_type(2)));
+  float x[24];
+#pragma unroll
+  for (int i = 0; i < 24; ++i) x[i] = (float)(tid & 7) * 0.125f - (float)i;
   for (int it = 0; it < iters; ++it) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
@@ -43,6 +52,23 @@ __global__ __launch_bounds__(kThreads) void mfma_loop_kernel(int32_t iters, int3
       for (int j = 0; j < 2; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a[i]),
                                                             __builtin_bit_cast(bf16x8_t, b[j]), acc[i][j], 0, 0, 0);
+    if constexpr (kExtra != 0) {
+#pragma unroll
+      for (int rep = 0; rep < ((kExtra == 2 || kExtra == 4) ? 2 : 1); ++rep)
+#pragma unroll
+        for (int i = 0; i < 24; ++i) {
+          if constexpr (kExtra == 1 || kExtra == 2) x[i] = fmaf(x[i], 1.0001f, 0.5f);
+          if constexpr (kExtra == 3 || kExtra == 4) x[i] = __builtin_amdgcn_exp2f(x[i]);
+          if constexpr (kExtra == 5) {
+            const floatx2_t f = {x[i], x[i]};
+            x[i] = __builtin_bit_cast(float, __builtin_convertvector(f, bf16x2_t));
+          }
+          if constexpr (kExtra == 6)
+            x[i] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, 0x3f803f80u),
+                                                   __builtin_bit_cast(bf16x2_t, __float_as_uint(x[(i + 1) % 24])), x[i], false);
+          if constexpr (kExtra == 7) x[i] = fmaxf(fmaxf(x[i], x[(i + 1) % 24]), x[(i + 2) % 24]);
+        }
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) a[i] ^= flip;
 #pragma unroll
@@ -53,6 +79,10 @@ __global__ __launch_bounds__(kThreads) void mfma_loop_kernel(int32_t iters, int3
   for (int i = 0; i < 4; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) s += acc[i][j][0];
+  if constexpr (kExtra != 0) {          // keeps the extra work alive; sink values are only defined for kExtra == 0
+#pragma unroll
+    for (int i = 0; i < 24; ++i) s += x[i] * 1e-30f;
+  }
   sink[tid] = s;
 }
 
@@ -61,8 +91,19 @@ __global__ __launch_bounds__(kThreads) void mfma_loop_kernel(int32_t iters, int3
 extern "C" int msa_diag_mfma_loop(int32_t workgroups, int32_t iters, int32_t mode, float* sink, double* flops_out,
                                   void* stream) {
   MSA_REQUIRE(workgroups > 0 && workgroups <= 65536 && iters > 0 && iters <= (1 << 24), "msa_diag_mfma_loop: bad sizes");
-  MSA_REQUIRE(mode >= 0 && mode <= 2 && sink != nullptr, "msa_diag_mfma_loop: bad mode / null sink");
-  mfma_loop_kernel<<<workgroups, kThreads, 0, as_stream(stream)>>>(iters, mode, sink);
+  const int operands = mode & 15, extra = mode >> 4;          // mode = operands + 16 * extra VALU work
+  MSA_REQUIRE(mode >= 0 && operands <= 2 && extra <= 7 && sink != nullptr, "msa_diag_mfma_loop: bad mode / null sink");
+  hipStream_t st = as_stream(stream);
+  switch (extra) {
+    case 0: mfma_loop_kernel<0><<<workgroups, kThreads, 0, st>>>(iters, operands, sink); break;
+    case 1: mfma_loop_kernel<1><<<workgroups, kThreads, 0, st>>>(iters, operands, sink); break;
+    case 2: mfma_loop_kernel<2><<<workgroups, kThreads, 0, st>>>(iters, operands, sink); break;
+    case 3: mfma_loop_kernel<3><<<workgroups, kThreads, 0, st>>>(iters, operands, sink); break;
+    case 4: mfma_loop_kernel<4><<<workgroups, kThreads, 0, st>>>(iters, operands, sink); break;
+    case 5: mfma_loop_kernel<5><<<workgroups, kThreads, 0, st>>>(iters, operands, sink); break;
+    case 6: mfma_loop_kernel<6><<<workgroups, kThreads, 0, st>>>(iters, operands, sink); break;
+    default: mfma_loop_kernel<7><<<workgroups, kThreads, 0, st>>>(iters, operands, sink); break;
+  }
   MSA_LAUNCH_CHECK();
   if (flops_out)
     *flops_out = (double)workgroups * (kThreads / 64) * (double)iters * kMfmasPerIter * (2.0 * 32 * 32 * 16);

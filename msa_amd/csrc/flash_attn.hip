@@ -173,12 +173,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
   // K rows past the last key may hold anything (their scores are masked by a select); V rows past it are multiplied
   // by probabilities of zero and must be finite, so those lanes fetch the last valid row again.
   const int row_bytes = row_elems * 2;
-  int tile_row[kLoads], k_piece[kLoads], v_piece[kLoads];
+  int tile_row[kLoads], k_piece[kLoads], v_piece[kLoads], v_full[kLoads];
 #pragma unroll
   for (int i = 0; i < kLoads; ++i) {
     tile_row[i] = 4 * (kLoads * wave + i) + (lane >> 4);
     k_piece[i] = ((lane & 15) ^ (tile_row[i] & 15)) * 16;
     v_piece[i] = ((lane & 15) ^ ((tile_row[i] & 3) << 2)) * 16;
+    v_full[i] = tile_row[i] * row_bytes + v_piece[i];          // the lane's offset in a tile whose 64 rows all exist
   }
   auto tile_rsrc = [&](const bf16_t* src, int t, int& rows) -> u32x4_t {
     rows = min(kKeysPerTile, kmax - t * kKeysPerTile);
@@ -197,10 +198,15 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
   auto issue_v = [&](int t, int slot) {
     int rows;
     const u32x4_t rsrc = tile_rsrc(v, t, rows);
+    if (rows == kKeysPerTile) {
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i)
-      load_to_lds(rsrc, lds_wave + kVBase + slot * kTileBytes + i * 1024,
-                  min(tile_row[i], rows - 1) * row_bytes + v_piece[i]);                      // rows <= 0: out of range
+      for (int i = 0; i < kLoads; ++i) load_to_lds(rsrc, lds_wave + kVBase + slot * kTileBytes + i * 1024, v_full[i]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < kLoads; ++i)
+        load_to_lds(rsrc, lds_wave + kVBase + slot * kTileBytes + i * 1024,
+                    min(tile_row[i], rows - 1) * row_bytes + v_piece[i]);                    // rows <= 0: out of range
+    }
   };
   // a barrier that waits for this wavefront's LDS reads but not for its loads in flight
   auto ring_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
@@ -278,8 +284,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
     const char* vt = lds + vslot * kTileBytes;
     float psum = 0.f;
     uint32_t pw[2][2][4];                   // P as packed bf16 pairs: [key rows 32 rb ..][16 j ..][pair]
-    constexpr int kKAhead = 6, kKRing = 4;  // K operand reads issued this many products ahead; ring of score steps
-    constexpr int kVAhead = 4, kVRing = 5;  // V^T operands read this many products ahead; ring of operands
+    constexpr int kKAhead = 4, kKRing = 3;  // K operand reads issued this many products ahead; ring of score steps
+    constexpr int kVAhead = 2, kVRing = 3;  // V^T operands read this many products ahead; ring of operands
     bf16x8_t kf[kKRing][2];
     bf16x8_t va[kVRing];
     auto k_read = [&](int i) {              // i = 2 ks + rb

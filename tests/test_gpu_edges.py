@@ -480,6 +480,13 @@ def test_mfma_loop_diagnostic_counts_exactly():
     torch.cuda.synchronize()
     assert torch.isfinite(sink).all() and (sink != 0).any()
     assert lib.msa_diag_mfma_loop(0, iters, 1, sink.data_ptr(), None, st) != 0
+    # the variants with other VALU work between the products (mode + 16 * extra) run; their sink is not defined
+    for extra in range(1, 8):
+        _lib.check(lib.msa_diag_mfma_loop(wgs, 50, 16 * extra, sink.data_ptr(), C.byref(flops), st), "msa_diag_mfma_loop")
+        assert flops.value == wgs * 8 * 50 * 8 * 2 * 32 * 32 * 16
+    torch.cuda.synchronize()
+    assert lib.msa_diag_mfma_loop(wgs, 50, 16 * 8, sink.data_ptr(), None, st) != 0
+    assert lib.msa_diag_mfma_loop(wgs, 50, 3, sink.data_ptr(), None, st) != 0
 
 
 @pytest.mark.gpu

@@ -86,11 +86,14 @@ __device__ __forceinline__ uint32_t lds_address(char* p) { return (uint32_t)(uin
 // every lane, and handed over in a scalar register).  Written as an asm statement, not through the compiler's builtin,
 // so that the compiler does not know of a load in flight that writes LDS: it would drain all of them (vmcnt(0)) in
 // front of the first transposing LDS read of every iteration, whose address it cannot tell from the loads' targets.
-// The waits are the kernel's own (see the ring).  The wait states in front of the load cover a resource or an M0 that
-// the preceding instruction wrote.  Nothing else in this kernel depends on M0.
+// The waits are the kernel's own (see the ring).  M0 (the LDS target) is put back as it was, so the statement is
+// transparent to whatever the compiler keeps there; the wait states in front of the load cover a resource or an M0
+// that the preceding instruction wrote.
 __device__ __forceinline__ void load_to_lds(u32x4_t rsrc, uint32_t lds_dst, int voffset) {
 #if defined(__HIP_DEVICE_COMPILE__)
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 4\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds" ::"s"(lds_dst), "v"(voffset), "s"(rsrc));
+  uint32_t saved_m0;
+  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 4\n\tbuffer_load_dwordx4 %2, %3, 0 offen lds\n\ts_mov_b32 m0, %0"
+               : "=&s"(saved_m0) : "s"(lds_dst), "v"(voffset), "s"(rsrc));
 #endif
 }
 

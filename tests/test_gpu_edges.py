@@ -293,7 +293,7 @@ def test_rmsnorm_and_silu_mul_widths(ops, dtype, H):
     assert cf.rel_err(ops.silu_mul(gu.cuda()).cpu(), want) < tol
 
 
-@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 8), (16, 2)])
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 8), (16, 2), (6, 3)])
 @pytest.mark.parametrize("causal", [True, False])
 def test_flash_kernel_through_the_c_abi(ops, Hq, Hkv, causal):
     """msa_flash_attn called directly (the host wrapper only picks it for large batches): every tile count parity of

@@ -512,7 +512,7 @@ def test_qk_norm_rope_rmsnorm_silu(ops, dtype):
     assert cf.rel_err(got.cpu(), g64 * torch.sigmoid(g64) * u64) < TOL[dtype]
 
 
-@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 8), (16, 2)])
+@pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 8), (16, 2), (6, 3)])
 @pytest.mark.parametrize("causal", [True, False])
 def test_flash_attention_blocks(ops, Hq, Hkv, causal):
     say(f"flash attention Hq={Hkv} Hkv={Hkv} causal={causal}")

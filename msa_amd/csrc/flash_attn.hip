@@ -122,7 +122,13 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
   for (; b < B; ++b) {
     const int sq_b = cu_q ? cu_q[b + 1] - cu_q[b] : 1;
     const int nb = (sq_b + kTokPerBlock - 1) / kTokPerBlock;
-    if (blk < nb) { found = true; break; }
+    if (blk < nb) {
+      // under the causal mask a sample's last token blocks see the most keys: they go first, so that the launch
+      // ends on short workgroups instead of waiting for a few long ones
+      if (causal) blk = nb - 1 - blk;
+      found = true;
+      break;
+    }
     blk -= nb;
   }
   if (!found) return;

@@ -147,6 +147,13 @@ int msa_profile_collect(float* ms_host, int32_t cap, int32_t* n_out);
  * (the budget of a kernel that does softmax arithmetic between them). */
 int msa_diag_mfma_loop(int32_t workgroups, int32_t iters, int32_t mode, float* sink, double* flops_out, void* stream);
 
+/* Test aid (no counterpart in the reference): `workgroups` workgroups that each claim a compute unit's whole LDS
+ * (160 KB) and fill it with `word`; check (device, [workgroups], may be null) receives one word read back per
+ * workgroup.  LDS is not cleared between kernels, so a launch of a few workgroups per compute unit leaves every unit's
+ * LDS holding `word` (a NaN pattern, say) for the next kernel to find: the tests use it to show that kernels whose
+ * tiles end in rows they did not load (ragged tails) never let stale LDS contents reach their results. */
+int msa_diag_fill_lds(uint32_t word, uint32_t* check, int32_t workgroups, void* stream);
+
 /* ---------------------------------------------------------------------------------------------
  * Gather of the selected documents' pooled K / V from pinned host memory.  Replaces the
  * index_select fetch and per-sample regroup of MSAService.doc_query

@@ -86,7 +86,26 @@ __global__ __launch_bounds__(kThreads) void mfma_loop_kernel(int32_t iters, int3
   sink[tid] = s;
 }
 
+// fills the workgroup's dynamic LDS with `word`
+__global__ __launch_bounds__(256) void fill_lds_kernel(uint32_t word, int32_t words, uint32_t* __restrict__ check) {
+  extern __shared__ uint32_t lds_words[];
+  for (int i = threadIdx.x; i < words; i += 256) lds_words[i] = word;
+  __syncthreads();
+  // read one word back so that the stores cannot be dropped
+  if (threadIdx.x == 0 && check != nullptr) check[blockIdx.x] = lds_words[(blockIdx.x * 61) % words];
+}
+
 }  // namespace
+
+extern "C" int msa_diag_fill_lds(uint32_t word, uint32_t* check, int32_t workgroups, void* stream) {
+  MSA_REQUIRE(workgroups > 0 && workgroups <= 65536, "msa_diag_fill_lds: bad workgroup count %d", workgroups);
+  constexpr int kBytes = 160 * 1024;                       // a compute unit's whole LDS: one workgroup per unit at a time
+  static std::atomic<int> lds_limit_raised{0};
+  MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(fill_lds_kernel), kBytes));
+  fill_lds_kernel<<<workgroups, 256, kBytes, as_stream(stream)>>>(word, kBytes / 4, check);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
 
 extern "C" int msa_diag_mfma_loop(int32_t workgroups, int32_t iters, int32_t mode, float* sink, double* flops_out,
                                   void* stream) {

@@ -331,6 +331,50 @@ def test_flash_kernel_through_the_c_abi(ops, Hq, Hkv, causal):
             assert cf.rel_err(out[rows][blind:], want) < 1e-2, (b, sq[b], L[b])
 
 
+@pytest.mark.parametrize("causal", [True, False])
+def test_flash_kernel_ignores_stale_lds(ops, causal):
+    """The flash kernel's K / V tiles arrive in LDS by direct loads; rows past a sample's last key are not loaded.
+    With every compute unit's LDS filled with NaN patterns beforehand (LDS is not cleared between kernels), ragged
+    samples whose last tile is partly or almost wholly empty must still give the oracle's result: scores of rows that
+    were not loaded are masked by a select, and V rows that were not loaded are never multiplied (0 x NaN)."""
+    say(f"flash kernel after an LDS fill of NaNs causal={causal}")
+    import ctypes as C
+    from msa_amd import _lib
+    lib = _lib.load()
+    Hq, Hkv, D = 32, 8, 128
+    sq = [1, 40, 64, 3, 100, 130]
+    L = [1, 65, 64, 127, 129, 200]
+    cu_q = np.concatenate([[0], np.cumsum(sq)])
+    cu_kv = np.concatenate([[0], np.cumsum(L)])
+    q = _randn((int(cu_q[-1]), Hq, D), 310, torch.bfloat16)
+    k = _randn((int(cu_kv[-1]), Hkv, D), 311, torch.bfloat16)
+    v = _randn((int(cu_kv[-1]), Hkv, D), 312, torch.bfloat16)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    kv_off = torch.as_tensor(cu_kv[:-1], dtype=torch.int64).cuda()
+    kv_len = torch.as_tensor(L, dtype=torch.int32).cuda()
+    cu_q_dev = torch.as_tensor(cu_q, dtype=torch.int32).cuda()
+    st = torch.cuda.current_stream().cuda_stream
+    check = torch.zeros(2048, dtype=torch.int32, device="cuda")
+    for word in (0x7fc07fc0, 0xffffffff):                    # bf16 NaN pairs; all ones (NaN as bf16 and as fp32)
+        _lib.check(lib.msa_diag_fill_lds(word, _lib.ptr(check), 2048, st), "msa_diag_fill_lds")
+        out = torch.full_like(qd, float("nan"))
+        _lib.check(lib.msa_flash_attn(_lib.ptr(qd), _lib.ptr(cu_q_dev), _lib.ptr(kd), _lib.ptr(vd), _lib.ptr(kv_off),
+                                      _lib.ptr(kv_len), len(sq), int(cu_q[-1]), Hq, Hkv, D, D ** -0.5, int(causal),
+                                      _lib.ptr(out), st), "msa_flash_attn")
+        torch.cuda.synchronize()
+        assert (check.cpu().view(torch.uint8).view(-1, 4) == torch.tensor(list(word.to_bytes(4, "little")), dtype=torch.uint8)).all()
+        out = out.cpu()
+        assert not torch.isnan(out).any()
+        for b in range(len(sq)):
+            rows = slice(int(cu_q[b]), int(cu_q[b + 1]))
+            keys = slice(int(cu_kv[b]), int(cu_kv[b + 1]))
+            blind = max(0, sq[b] - L[b]) if causal else 0
+            assert (out[rows][:blind] == 0).all()
+            want = cf.attention(q[rows][blind:], k[keys], v[keys], causal=causal)
+            assert cf.rel_err(out[rows][blind:], want) < 1e-2, (b, sq[b], L[b])
+    assert lib.msa_diag_fill_lds(0, None, 0, st) != 0
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("B,V", [(16, 151936), (3, 1000), (1, 31), (5, 65)])
 def test_greedy_sample_against_argmax(ops, dtype, B, V):

@@ -450,7 +450,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vg
 
   // Epilogue of the N tile starting at chunk `tile_n0`.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of
   // its 32x32 block.  Consecutive row blocks of one query are folded into `run` (each half of the wavefront over its
-  // own rows); emit() joins the halves and merges the query's 32 column maxima of this block into the key plane.
+  // own rows); emit() joins the halves and merges the query's column maxima of both blocks into the key plane.
   // Several wavefronts and workgroups hold parts of a query (and of a document), so the merge is an atomicMax into
   // a zeroed plane.  emit() is reached by whole wavefronts (q and any are uniform).
   //
@@ -479,9 +479,17 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vg
       }
     }
   };
-  auto emit = [&](int q, int n, int doc, float run_half, bool any) {
+  // Both column blocks of the wavefront at once: after the halves are joined (one half-wave swap: the upper half of
+  // block 0's partial maxima against the lower half of block 1's) the lower 32 lanes hold block 0's 32 column maxima
+  // and the upper 32 lanes block 1's, so the segmented scan and the atomics below run once per query for the
+  // wavefront's 64 columns instead of once per block with half the lanes idle.
+  static_assert(TN == 2, "the epilogue pairs the two column blocks of a wavefront");
+  auto emit = [&](int q, int tile_n0, const float (&run_half)[TN], bool any) {
     if (!any || q >= n_queries) return;
-    const float run = fmaxf(run_half, __shfl_xor(run_half, 32));
+    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(run_half[0]), __float_as_uint(run_half[1]), false, false);
+    const float run = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    const int n = tile_n0 + wn * WN + half * 32 + l32;
+    const int doc = kDocMax ? (half ? cdoc[1] : cdoc[0]) : 0;
     const bool ok = n < C;
     const uint32_t key = ok ? f32_to_key(run) : 0u;
     if constexpr (kDocMax) {
@@ -510,45 +518,50 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vg
 #undef MSA_SCAN_STEP
       const int low = __builtin_amdgcn_update_dpp(0, m, 0x142, 0xA, 0xF, false);          // row_bcast:15 into rows 1, 3
       if (dist > (l32 & 15)) m = (int)max((uint32_t)m, (uint32_t)low);
-      if (ok && half == 0 && last) atomicMax(&out_key[(int64_t)q * n_docs + doc], (uint32_t)m);
+      if (ok && last) atomicMax(&out_key[(int64_t)q * n_docs + doc], (uint32_t)m);
     } else {
-      if (ok && half == 0) atomicMax(&out_key[(int64_t)q * C + n], key);
+      if (ok) atomicMax(&out_key[(int64_t)q * C + n], key);
     }
   };
   auto epilogue = [&](int tile_n0) {
+    float run[TN];
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int n = tile_n0 + wn * WN + j * 32 + l32;
-      const int doc = kDocMax ? cdoc[j] : 0;
-      float run = -INFINITY;
-      bool any = false;
-      int run_q = q_first, r = r_first;                    // query of row block i, its block index inside the query
+    for (int j = 0; j < TN; ++j) run[j] = -INFINITY;
+    bool any = false;
+    int run_q = q_first, r = r_first;                      // query of row block i, its block index inside the query
 #pragma unroll
-      for (int i = 0; i < TM; ++i) {
-        const uint32_t bits = __builtin_amdgcn_readfirstlane(rbits[i]);
-        if (r == blocks_per_query) {                       // row block i opens the next query
-          emit(run_q, n, doc, run, any);
-          run = -INFINITY; any = false; ++run_q; r = 0;
-        }
-        ++r;
-        if (bits == 0xffffffffu) {                          // every row scored: no per-row tests
+    for (int i = 0; i < TM; ++i) {
+      const uint32_t bits = __builtin_amdgcn_readfirstlane(rbits[i]);
+      if (r == blocks_per_query) {                         // row block i opens the next query
+        emit(run_q, tile_n0, run, any);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) run[j] = -INFINITY;
+        any = false; ++run_q; r = 0;
+      }
+      ++r;
+      if (bits == 0xffffffffu) {                            // every row scored: no per-row tests
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
           float mx = acc[i][j][0];
 #pragma unroll
           for (int e = 1; e < 16; ++e) mx = fmaxf(mx, acc[i][j][e]);
-          run = fmaxf(run, mx);
-          any = true;
-        } else if (bits != 0) {
-          const uint32_t mine = bits >> (4 * half);         // this half's rows: bit 8*(e/4) + e%4
+          run[j] = fmaxf(run[j], mx);
+        }
+        any = true;
+      } else if (bits != 0) {
+        const uint32_t mine = bits >> (4 * half);           // this half's rows: bit 8*(e/4) + e%4
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
           float mx = -INFINITY;
 #pragma unroll
           for (int e = 0; e < 16; ++e)
             if (mine & (1u << (8 * (e >> 2) + (e & 3)))) mx = fmaxf(mx, acc[i][j][e]);
-          run = fmaxf(run, mx);
-          any = true;
+          run[j] = fmaxf(run[j], mx);
         }
+        any = true;
       }
-      emit(run_q, n, doc, run, any);
     }
+    emit(run_q, tile_n0, run, any);
   };
 
   if constexpr (kDtl) {

@@ -130,3 +130,49 @@ def test_routing_ten_million_token_bank(ops):
     bank2.set_layer(0, kr2)
     cs_perm = ops.chunk_scores(bank2, 0, q, mask, "cosine", 1.0)
     assert torch.equal(cs_perm, cs_all[:, perm])
+
+
+def test_prefill_attention_full_size_properties(ops):
+    """The stage-2 prefill attention of the end-to-end workload at its real shape (16 samples of 4096 query tokens over
+    291 memory rows + the 4096 tokens, bottom-right causal mask, 32 query / 8 KV heads), where the fp64 oracle cannot
+    run over everything.  Size-independent properties that pin the mask boundary and the normalisation of every row:
+    (1) values of ones: every row must come out as ones whatever the scores (the probabilities the kernel multiplies
+        sum to the denominator it divides by);
+    (2) queries of zeros: every visible key has the same weight, so row i of a sample is the mean of the first
+        M + i + 1 value rows, which a prefix sum gives exactly: one key too many or too few in any row shows;
+    (3) random rows of the random case against the fp64 oracle."""
+    say("full size: prefill attention B=16 S=4096 L=4387")
+    B, S, M, Hq, Hkv, D = 16, 4096, 291, 32, 8, 128
+    L = M + S
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(77)
+    q = torch.randn((B * S, Hq, D), generator=g, device=dev).to(torch.bfloat16)
+    k = torch.randn((B * L, Hkv, D), generator=g, device=dev).to(torch.bfloat16)
+    v = torch.randn((B * L, Hkv, D), generator=g, device=dev).to(torch.bfloat16)
+    kv_off = torch.arange(B, dtype=torch.int64, device=dev) * L
+    kv_len = torch.full((B,), L, dtype=torch.int32, device=dev)
+    cu_q = torch.arange(B + 1, dtype=torch.int32, device=dev) * S
+    run = lambda qq, vv: ops.sparse_attn(qq, k, vv, kv_off, kv_len, L, cu_q=cu_q, max_sq=S, causal=True)
+    # (1)
+    out = run(q, torch.ones_like(v))
+    torch.cuda.synchronize()
+    assert (out.float() - 1.0).abs().max().item() < 1e-2
+    # (2)
+    out = run(torch.zeros_like(q), v).float().view(B, S, Hq, D)
+    prefix = torch.cumsum(v.float().view(B, L, Hkv, D), dim=1)                      # fp32 sums of bf16 values
+    counts = (M + 1 + torch.arange(S, device=dev)).float().view(1, S, 1, 1)
+    want = (prefix[:, M:M + S] / counts).repeat_interleave(Hq // Hkv, dim=2)        # [B, S, Hq, D]
+    # the means are at most ~0.3 in size, so bf16 rounding of the output is at most 1e-3; a key too many or too few
+    # moves the first rows (292 keys) by up to |v| / 292 ~ 0.014
+    err = (out - want).abs().max().item()
+    assert err < 3e-3, err
+    first = (out[:, :64] - want[:, :64]).abs().max().item()                        # the rows with the fewest keys
+    assert first < 2e-3, first
+    # (3)
+    out = run(q, v).view(B, S, Hq, D)
+    rng = np.random.default_rng(5)
+    qh, kh, vh = q.view(B, S, Hq, D), k.view(B, L, Hkv, D), v.view(B, L, Hkv, D)
+    for _ in range(6):
+        b, i = int(rng.integers(B)), int(rng.integers(S))
+        want_row = cf.attention(qh[b, i:i + 1].cpu(), kh[b, :M + i + 1].cpu(), vh[b, :M + i + 1].cpu(), causal=True)
+        assert cf.rel_err(out[b, i:i + 1].cpu(), want_row) < 1e-2, (b, i)

@@ -231,7 +231,8 @@ int msa_cache_append_rows(const void* k_new, const void* v_new, const int32_t* c
  *   q: [sum Sq, Hq, D] with cu_q[B+1] (NULL = one row per sample); k / v: rows [Hkv, D];
  *   sample b's keys are rows kv_off[b] .. kv_off[b] + kv_len[b].  causal != 0: query row i of a
  *   sample with Sq rows sees the first kv_len - Sq + i + 1 keys (bottom-right aligned).
- *   out: [sum Sq, Hq, D].  max_sq / max_kv bound the per-sample sizes (grid sizing only). */
+ *   out: [sum Sq, Hq, D].  max_sq / max_kv bound the per-sample sizes (grid sizing only).
+ *   q, k, v and out must be 16-byte aligned (MSA_EINVAL otherwise): rows move in 16-byte pieces. */
 size_t msa_attn_workspace_bytes(int32_t total_q, int32_t Hq, int32_t Hkv, int32_t D, int32_t max_kv);
 int msa_sparse_attn(const void* q, const int32_t* cu_q, const void* k, const void* v,
                     const int64_t* kv_off, const int32_t* kv_len, int32_t B, int32_t total_q,

@@ -534,6 +534,8 @@ extern "C" int msa_sparse_attn(const void* q, const int32_t* cu_q, const void* k
   MSA_REQUIRE(Hkv > 0 && Hq % Hkv == 0 && Hq / Hkv <= kMaxG, "msa_sparse_attn: Hq=%d Hkv=%d unsupported", Hq, Hkv);
   MSA_REQUIRE(dtype == MSA_BF16 || dtype == MSA_F32, "msa_sparse_attn: bad dtype %d", dtype);
   MSA_REQUIRE(scale > 0.f, "msa_sparse_attn: scale must be positive");
+  MSA_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) == 0,
+              "msa_sparse_attn: q, k, v and out must be 16-byte aligned");
   MSA_REQUIRE((int64_t)total_q * Hq < (int64_t)1 << 31 && total_q < 65536 * 32, "msa_sparse_attn: too many rows");
   const bool mfma = dtype == MSA_BF16 && max_sq >= 8;
   const SplitPlan plan = mfma ? plan_splits(total_q, Hkv, max_kv) : plan_splits_valu(total_q, Hkv, max_kv);

@@ -464,6 +464,8 @@ extern "C" int msa_flash_attn(const void* q, const int32_t* cu_q, const void* k,
   MSA_REQUIRE(cu_q != nullptr || total_q == B, "msa_flash_attn: cu_q is required when total_q != B");
   MSA_REQUIRE(Hkv > 0 && Hkv <= 65535 && Hq % Hkv == 0, "msa_flash_attn: Hq=%d Hkv=%d unsupported", Hq, Hkv);
   MSA_REQUIRE(scale > 0.f, "msa_flash_attn: scale must be positive");
+  MSA_REQUIRE((((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)out) & 15) == 0,
+              "msa_flash_attn: q, k, v and out must be 16-byte aligned");
   const int G = Hq / Hkv;
   MSA_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, "msa_flash_attn: GQA group size %d unsupported (1, 2, 4, 8)", G);
   return flash_launch<false>(G, q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale,

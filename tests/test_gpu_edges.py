@@ -128,6 +128,17 @@ def test_error_codes(ops):
         ops.chunk_scores(two, 0, q, mode="l2")
     with pytest.raises(ValueError, match="pinned"):
         two.set_layer(1, kr_dev, kr.clone(), kr.clone())
+    # attention: rows move in 16-byte pieces, so a misaligned tensor is refused, not read
+    aq = _randn((64 * 32 * 128 + 8,), 354, torch.bfloat16).cuda()
+    ak = _randn((64 * 8 * 128 + 8,), 355, torch.bfloat16).cuda()
+    off = torch.zeros(1, dtype=torch.int64, device="cuda"); ln = torch.full((1,), 64, dtype=torch.int32, device="cuda")
+    cu = torch.tensor([0, 64], dtype=torch.int32, device="cuda")
+    rc = lib.msa_flash_attn(aq.data_ptr() + 2, cu.data_ptr(), ak.data_ptr(), ak.data_ptr(), off.data_ptr(), ln.data_ptr(),
+                            1, 64, 32, 8, 128, 128 ** -0.5, 1, aq.data_ptr(), None)
+    assert rc == -1 and b"16-byte aligned" in lib.msa_last_error()                # MSA_EINVAL
+    rc = lib.msa_sparse_attn(aq.data_ptr(), cu.data_ptr(), ak.data_ptr() + 2, ak.data_ptr(), off.data_ptr(), ln.data_ptr(),
+                             1, 64, 64, 64, 32, 8, 128, 0, 128 ** -0.5, 1, aq.data_ptr(), ws.data_ptr(), 1024, None)
+    assert rc == -1 and b"16-byte aligned" in lib.msa_last_error()
     with pytest.raises(_lib.MsaError, match="rotary table"):
         t = ops.chunk_table([300], 64)
         x = _randn((300, 8, 128), 353, torch.bfloat16).cuda()

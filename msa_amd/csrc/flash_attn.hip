@@ -89,11 +89,26 @@ __device__ __forceinline__ uint32_t lds_address(char* p) { return (uint32_t)(uin
 // The waits are the kernel's own (see the ring).  M0 (the LDS target) is put back as it was, so the statement is
 // transparent to whatever the compiler keeps there; the wait states in front of the load cover a resource or an M0
 // that the preceding instruction wrote.
-__device__ __forceinline__ void load_to_lds(u32x4_t rsrc, uint32_t lds_dst, int voffset) {
+// Four loads at once: the wavefront's four consecutive 1 KB blocks of a tile (offsets v0 .. v3).
+__device__ __forceinline__ void load4_to_lds(u32x4_t rsrc, uint32_t lds_dst, int v0, int v1, int v2, int v3) {
 #if defined(__HIP_DEVICE_COMPILE__)
   uint32_t saved_m0;
-  asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 4\n\tbuffer_load_dwordx4 %2, %3, 0 offen lds\n\ts_mov_b32 m0, %0"
-               : "=&s"(saved_m0) : "s"(lds_dst), "v"(voffset), "s"(rsrc));
+  asm volatile(
+      "s_mov_b32 %0, m0\n\t"
+      "s_mov_b32 m0, %1\n\t"
+      "s_nop 4\n\t"
+      "buffer_load_dwordx4 %2, %6, 0 offen lds\n\t"
+      "s_add_u32 m0, m0, 0x400\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %3, %6, 0 offen lds\n\t"
+      "s_add_u32 m0, m0, 0x400\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %4, %6, 0 offen lds\n\t"
+      "s_add_u32 m0, m0, 0x400\n\t"
+      "s_nop 0\n\t"
+      "buffer_load_dwordx4 %5, %6, 0 offen lds\n\t"
+      "s_mov_b32 m0, %0"
+      : "=&s"(saved_m0) : "s"(lds_dst), "v"(v0), "v"(v1), "v"(v2), "v"(v3), "s"(rsrc) : "scc");
 #endif
 }
 
@@ -200,21 +215,19 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
   auto issue_k = [&](int t, int slot) {
     int rows;
     const u32x4_t rsrc = tile_rsrc(k, t, rows);
-#pragma unroll
-    for (int i = 0; i < kLoads; ++i)
-      load_to_lds(rsrc, lds_wave + slot * kTileBytes + i * 1024, tile_row[i] * row_bytes + k_piece[i]);
+    load4_to_lds(rsrc, lds_wave + slot * kTileBytes, tile_row[0] * row_bytes + k_piece[0], tile_row[1] * row_bytes + k_piece[1],
+                 tile_row[2] * row_bytes + k_piece[2], tile_row[3] * row_bytes + k_piece[3]);
   };
   auto issue_v = [&](int t, int slot) {
     int rows;
     const u32x4_t rsrc = tile_rsrc(v, t, rows);
     if (rows == kKeysPerTile) {
-#pragma unroll
-      for (int i = 0; i < kLoads; ++i) load_to_lds(rsrc, lds_wave + kVBase + slot * kTileBytes + i * 1024, v_full[i]);
+      load4_to_lds(rsrc, lds_wave + kVBase + slot * kTileBytes, v_full[0], v_full[1], v_full[2], v_full[3]);
     } else {
+      int vo[kLoads];
 #pragma unroll
-      for (int i = 0; i < kLoads; ++i)
-        load_to_lds(rsrc, lds_wave + kVBase + slot * kTileBytes + i * 1024,
-                    min(tile_row[i], rows - 1) * row_bytes + v_piece[i]);                    // rows <= 0: out of range
+      for (int i = 0; i < kLoads; ++i) vo[i] = min(tile_row[i], rows - 1) * row_bytes + v_piece[i];   // rows <= 0: out of range
+      load4_to_lds(rsrc, lds_wave + kVBase + slot * kTileBytes, vo[0], vo[1], vo[2], vo[3]);
     }
   };
   // a barrier that waits for this wavefront's LDS reads but not for its loads in flight
@@ -363,7 +376,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
     ring = ring1;
   };
 
-  static_assert(kLoads == 4, "the wait counts assume four loads per wavefront, tile and tensor");
+  static_assert(kLoads == 4, "the wait counts and the load statement assume four loads per wavefront, tile and tensor");
   if (first_tile < n_tiles) {
     issue_k(first_tile, 0);
     issue_v(first_tile, 0);

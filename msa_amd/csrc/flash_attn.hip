@@ -205,22 +205,32 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
     v_piece[i] = ((lane & 15) ^ ((tile_row[i] & 3) << 2)) * 16;
     v_full[i] = tile_row[i] * row_bytes + v_piece[i];          // the lane's offset in a tile whose 64 rows all exist
   }
-  auto tile_rsrc = [&](const bf16_t* src, int t, int& rows) -> u32x4_t {
-    rows = min(kKeysPerTile, kmax - t * kKeysPerTile);
-    const uintptr_t at = reinterpret_cast<uintptr_t>(src) + ((base + (int64_t)t * kKeysPerTile) * row_elems + g * kHeadDim) * 2;
-    return u32x4_t{(uint32_t)at, (uint32_t)(at >> 32) & 0xffffu, (uint32_t)max(0, (rows - 1) * row_bytes + kRowBytes),
-                   0x00020000u};                                                            // extent 0 when no row is left
+  // Tiles are loaded in order, K and V each from its own running position (address of the next tile to load, keys
+  // left from its first row on): a load takes the position's tile and moves it on by one.
+  struct TilePos { uintptr_t at; int left; };
+  auto first_pos = [&](const bf16_t* src) {
+    return TilePos{reinterpret_cast<uintptr_t>(src) + ((base + (int64_t)first_tile * kKeysPerTile) * row_elems + g * kHeadDim) * 2,
+                   kmax - first_tile * kKeysPerTile};
+  };
+  TilePos k_pos = first_pos(k), v_pos = first_pos(v);
+  auto tile_rsrc = [&](TilePos& p, int& rows) -> u32x4_t {
+    rows = min(kKeysPerTile, p.left);
+    const u32x4_t r = {(uint32_t)p.at, (uint32_t)(p.at >> 32) & 0xffffu, (uint32_t)max(0, (rows - 1) * row_bytes + kRowBytes),
+                       0x00020000u};                                                        // extent 0 when no row is left
+    p.at += (uintptr_t)kKeysPerTile * row_bytes;
+    p.left -= kKeysPerTile;
+    return r;
   };
   const uint32_t lds_wave = lds_address(lds) + kLoads * wave * 1024;     // this wavefront's first block of a tile
-  auto issue_k = [&](int t, int slot) {
+  auto issue_k = [&](int slot) {
     int rows;
-    const u32x4_t rsrc = tile_rsrc(k, t, rows);
+    const u32x4_t rsrc = tile_rsrc(k_pos, rows);
     load4_to_lds(rsrc, lds_wave + slot * kTileBytes, tile_row[0] * row_bytes + k_piece[0], tile_row[1] * row_bytes + k_piece[1],
                  tile_row[2] * row_bytes + k_piece[2], tile_row[3] * row_bytes + k_piece[3]);
   };
-  auto issue_v = [&](int t, int slot) {
+  auto issue_v = [&](int slot) {
     int rows;
-    const u32x4_t rsrc = tile_rsrc(v, t, rows);
+    const u32x4_t rsrc = tile_rsrc(v_pos, rows);
     if (rows == kKeysPerTile) {
       load4_to_lds(rsrc, lds_wave + kVBase + slot * kTileBytes, v_full[0], v_full[1], v_full[2], v_full[3]);
     } else {
@@ -277,8 +287,8 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
   auto step = [&](int t, floatx16_t (&sc)[2], floatx16_t (&sn)[2]) {
     const int ring1 = ring == kRingK - 1 ? 0 : ring + 1;
     const int vslot = (t - first_tile) & 1;  // the slot of V(t)
-    issue_v(t + 1, vslot ^ 1);               // V(t - 1)'s slot: last read before the previous barrier
-    issue_k(t + 3, ring);                    // K(t)'s slot: likewise
+    issue_v(vslot ^ 1);                      // V(t + 1) into V(t - 1)'s slot: last read before the previous barrier
+    issue_k(ring);                           // K(t + 3) into K(t)'s slot: likewise
     // (A) the column maximum of this tile's (masked) scores came with the scores: `mx_raw`
     float mx = fmaxf(m, mx_raw * scale_log2e);
     mx = half_wave_max(mx);
@@ -378,10 +388,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
 
   static_assert(kLoads == 4, "the wait counts and the load statement assume four loads per wavefront, tile and tensor");
   if (first_tile < n_tiles) {
-    issue_k(first_tile, 0);
-    issue_v(first_tile, 0);
-    issue_k(first_tile + 1, 1);
-    issue_k(first_tile + 2, 2);
+    issue_k(0);                                // K(first), V(first), K(first + 1), K(first + 2)
+    issue_v(0);
+    issue_k(1);
+    issue_k(2);
     __builtin_amdgcn_s_waitcnt(kWaitVm12);     // K(first) has landed
     ring_barrier();
     floatx16_t s0[2], s1[2];

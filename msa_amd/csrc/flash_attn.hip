@@ -365,6 +365,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
       if (sl >= 16 - kVAhead) v_read(sl - (16 - kVAhead));
       fence();
     }
+    // The O products have little VALU work of their own: with the wavefront's priority raised for their length the
+    // SIMD's other wavefront (of the compute unit's other workgroup, usually in a different phase) yields the matrix
+    // pipe to them and fills the gaps with its own VALU work instead of the other way round (1.4 %).
+    __builtin_amdgcn_s_setprio(1);
 #pragma unroll
     for (int u = 0; u < 12; ++u) {
       if (u + kVAhead < 16) v_read(u + kVAhead);
@@ -379,6 +383,7 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
       pv(i + 12);
     });
     fence();
+    __builtin_amdgcn_s_setprio(0);
     l += half_wave_sum(psum);
     // K(t + 2), issued an iteration ago, and V(t + 1) have landed once only the loads of K(t + 3) are outstanding
     __builtin_amdgcn_s_waitcnt(kWaitVm4);

@@ -124,7 +124,11 @@ __global__ __launch_bounds__(kThreads, 2) void pool_chunks_kernel(PoolArgs a) {
       hi[q].load(group, voff + q * q_stride + 64 * (int)sizeof(T), 0);
     }
   };
+  // (loads are issued at raised priority: a wavefront that has requests to make goes ahead of those that are summing,
+  // which keeps more bytes in flight per compute unit: 0.9 %)
+  __builtin_amdgcn_s_setprio(3);
   issue(lo_a, hi_a, 0);
+  __builtin_amdgcn_s_setprio(0);
 
   float acc_lo[8], acc_hi[8];
 #pragma unroll
@@ -174,9 +178,13 @@ __global__ __launch_bounds__(kThreads, 2) void pool_chunks_kernel(PoolArgs a) {
   };
   auto stream = [&](auto rope_tag) {
     for (int base = 0; base < rows_valid; base += 2 * group_rows) {
+      __builtin_amdgcn_s_setprio(3);
       issue(lo_b, hi_b, base + group_rows);
+      __builtin_amdgcn_s_setprio(0);
       consume(rope_tag, lo_a, hi_a);
+      __builtin_amdgcn_s_setprio(3);
       issue(lo_a, hi_a, base + 2 * group_rows);   // empty once past the end
+      __builtin_amdgcn_s_setprio(0);
       consume(rope_tag, lo_b, hi_b);
     }
   };

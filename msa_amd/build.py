@@ -15,7 +15,7 @@ LIB = os.path.join(HERE, "libmsa_amd.so")
 ARCH = "gfx950"
 # packed fp32 VALU ops are switched off for all device code of this library
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
-         "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
+         "-packed-fp32-ops", "-Wall", "-Wno-unused-function", "-Wno-inline-asm"]
 
 
 def sources():

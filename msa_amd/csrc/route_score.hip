@@ -925,6 +925,314 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vg
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// The MFMA-bound form (bf16, more than 128 query rows): 256 x 256 tile, four wavefronts (one per SIMD) of 128 x 128,
+// the sixteen 32 x 32 accumulators of a wavefront in the 256 accumulation registers, and the K step written at the
+// instruction level (scan_asm.inc, generated by gen_scan_asm.py, which describes the schedule and the registers the
+// asm statements own: v128 - v255 and a0 - a255; the compiler-allocated code of this kernel is held below v128 by the
+// register limit on its declaration and uses no accumulation registers, which the build checks).  One wavefront per
+// SIMD has nobody to cover a wait, so every wait the step contains is met long before it is reached: operand
+// fragments are read a sub-step ahead, the query and K_r tiles are requested two K steps ahead (LDS: two stages of the
+// query tile, three of the K_r tile, filled by buffer loads that write LDS directly), and the one barrier per step
+// stands behind an MFMA.  Per 128 x 128 wavefront tile a sub-step reads eight operand fragments for sixteen MFMAs,
+// against six for eight in a 2 x 4 layout of eight wavefronts.
+//
+// Persistent: one workgroup per compute unit walks its share of the tile list (scan_walk.h) as one sequence of K
+// steps, the loads two steps ahead across tile boundaries.  With a gather job attached the last workgroup of the
+// launch copies the K / V rows of an earlier selection instead (gather_device.h).  The last pool_n N tiles are handed
+// out one at a time to workgroups that have finished their own share: during the first K steps of the tile in front of
+// a pool tile one lane draws a position from the pool's counter (an atomic that returns), publishes it through the
+// workgroup's claim word (an exchange that returns, so its arrival says the word is in L2) and every wavefront reads
+// it back, one hop per K step, each issued in front of the step's tile loads so that the step's own wait (all but the
+// eight newest loads) covers it.  The hops' values live in v217 - v219.
+// ------------------------------------------------------------------------------------------
+#include "scan_asm.inc"
+#include "scan_walk.h"
+
+constexpr int kScan4CompilerVgprs = 128;     // the compiler's share of the vector registers in score_scan4_kernel
+constexpr int kScan4LdsBytes = 5 * 256 * 128;
+
+#if defined(__HIP_DEVICE_COMPILE__)
+template <int N>
+__device__ __forceinline__ void scan4_read_acc(float (&x)[16]);
+#define MSA_SCAN4_READER(N)                                                                                          \
+  template <>                                                                                                       \
+  __device__ __forceinline__ void scan4_read_acc<N>(float (&x)[16]) {                                               \
+    asm volatile(MSA_SCAN4_ACC_READ_##N                                                                              \
+                 : "=v"(x[0]), "=v"(x[1]), "=v"(x[2]), "=v"(x[3]), "=v"(x[4]), "=v"(x[5]), "=v"(x[6]), "=v"(x[7]),    \
+                   "=v"(x[8]), "=v"(x[9]), "=v"(x[10]), "=v"(x[11]), "=v"(x[12]), "=v"(x[13]), "=v"(x[14]), "=v"(x[15])); \
+  }
+MSA_SCAN4_READER(0) MSA_SCAN4_READER(1) MSA_SCAN4_READER(2) MSA_SCAN4_READER(3) MSA_SCAN4_READER(4) MSA_SCAN4_READER(5)
+MSA_SCAN4_READER(6) MSA_SCAN4_READER(7) MSA_SCAN4_READER(8) MSA_SCAN4_READER(9) MSA_SCAN4_READER(10) MSA_SCAN4_READER(11)
+MSA_SCAN4_READER(12) MSA_SCAN4_READER(13) MSA_SCAN4_READER(14) MSA_SCAN4_READER(15)
+#undef MSA_SCAN4_READER
+#endif
+
+template <bool kDocMax>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerVgprs))) void score_scan4_kernel(
+    const bf16_t* __restrict__ qs,          // [M_rows, K]  pre-summed queries, M_rows = B * S_pad
+    const bf16_t* __restrict__ kr,          // [C, K]
+    const uint32_t* __restrict__ row_bits,  // [ceil(M_alloc / 32)] scored-row bitmask
+    uint32_t* __restrict__ out_key,         // [B, n_docs] or [B, C], zeroed
+    const int32_t* __restrict__ chunk_doc,  // [C] document of every chunk (kDocMax)
+    int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t tiles_m, int32_t tiles_n, int32_t m_group,
+    int32_t n_docs, GatherJob job, uint32_t* __restrict__ sched, int32_t pool_n) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int kThreads = 256, BM = 256, BN = 256;
+  extern __shared__ __align__(16) char lds[];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  if (job.active && (int)blockIdx.x == (int)gridDim.x - 1) {
+    // plan (sorted, de-duplicated selection -> copy entries), host rows, then the documents an earlier sample already
+    // fetched; the workgroup barriers order the three steps' memory
+    msa_gather::plan_body(job.doc_sel, job.doc_chunk_off, job.n_docs, job.B, job.k,
+                          (int32_t)min(job.capacity_rows, (int64_t)0x7fffffff), job.dedup, job.cu_sel, job.plan,
+                          reinterpret_cast<int32_t*>(lds), tid, kThreads);
+    __syncthreads();
+    const int groups = kThreads / msa_gather::kCopyRowLanes;
+    const int group = tid / msa_gather::kCopyRowLanes, lane_in_row = tid % msa_gather::kCopyRowLanes;
+    msa_gather::copy_body<false, 8>(job.k_src, job.v_src, job.plan, job.B * job.k, job.row_vecs, job.capacity_rows,
+                                    job.k_dst, job.v_dst, 0, 1, group, groups, lane_in_row);
+    __syncthreads();
+    if (job.dedup)
+      msa_gather::copy_body<true, 8>(nullptr, nullptr, job.plan, job.B * job.k, job.row_vecs, job.capacity_rows, job.k_dst,
+                                     job.v_dst, 0, 1, group, groups, lane_in_row);
+    return;
+  }
+  const ScanWalk walk = scan_walk_init((int)blockIdx.x, (int)gridDim.x, job.active ? 1 : 0, tiles_m, tiles_n, m_group, pool_n);
+  if (walk.own_count == 0) return;
+
+  const int wm = wave >> 1, wn = wave & 1;
+  const int half = lane >> 5, l32 = lane & 31;
+  const int row_bytes = K * (int)sizeof(bf16_t);
+  const int k_tiles = row_bytes / kRowBytes;
+  {
+    // per-lane constants of the asm statements: LDS offsets of the operand fragments of sub-steps 0 - 3 (the rows of a
+    // wavefront's blocks are 32 apart, which leaves the swizzle term alone) and the global offsets of the lanes' 16
+    // bytes in the wavefront's eight 1 KB blocks of a tile (lane l lands at byte 16 * l of its block, i.e. row l / 8,
+    // unit slot l % 8, and fetches the unit that belongs there)
+    int aa[4], ab[4], vo[8];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int sw = ((s * 2 + half) ^ ((l32 >> 1) & 7)) * 16;
+      aa[s] = (wm * 128 + l32) * 128 + sw;
+      ab[s] = (wn * 128 + l32) * 128 + sw;
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int row = (wave * 8 + i) * 8 + (lane >> 3);
+      vo[i] = row * row_bytes + (((lane & 7) ^ ((row >> 1) & 7)) * 16);
+    }
+    asm volatile(MSA_SCAN4_SET_ADDR ::"v"(aa[0]), "v"(aa[1]), "v"(aa[2]), "v"(aa[3]), "v"(ab[0]), "v"(ab[1]), "v"(ab[2]), "v"(ab[3])
+                 : MSA_SCAN4_CLOBBERS);
+    asm volatile(MSA_SCAN4_SET_VOFF ::"v"(vo[0]), "v"(vo[1]), "v"(vo[2]), "v"(vo[3]), "v"(vo[4]), "v"(vo[5]), "v"(vo[6]), "v"(vo[7])
+                 : MSA_SCAN4_CLOBBERS);
+    // v222: byte offset of a lane's column in a run of 64 document ids; v223: the pool counter's increment
+    asm volatile("v_lshlrev_b32 v222, 2, %0\n\tv_mov_b32 v223, 1" ::"v"(lane) : MSA_SCAN4_CLOBBERS);
+  }
+  const char* ga = reinterpret_cast<const char*>(qs);
+  const char* gb = reinterpret_cast<const char*>(kr);
+  // One resource per operand tile whose extent is the valid part of the tile: rows past M_rows / C read as zero in
+  // hardware (the range check is on the vector offset, where the row displacement rides; the K displacement is
+  // scalar and stays inside the row).  A tile that does not exist gets an empty extent: its loads fetch nothing.
+  auto make_a = [&](int tm, bool valid) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(ga) + (valid ? (int64_t)tm * BM * row_bytes : 0), 0,
+                                             valid ? min(BM, M_rows - tm * BM) * row_bytes : 0, 0x00020000);
+  };
+  auto make_b = [&](int tn, bool valid) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(gb) + (valid ? (int64_t)tn * BN * row_bytes : 0), 0,
+                                             valid ? min(BN, C - tn * BN) * row_bytes : 0, 0x00020000);
+  };
+  const __amdgpu_buffer_rsrc_t rsrc_docs =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t*>(kDocMax ? chunk_doc : nullptr), 0, kDocMax ? C * 4 : 0, 0x00020000);
+
+  // The workgroup's tiles: `cur` is multiplied, `nxt` is the one behind it (the loads enter it two K steps before the
+  // MFMAs do).  Own tiles first, then pool draws.
+  int tm_c, tn_c, tm_n = 0, tn_n = 0, own_idx = 0;
+  scan_walk_own(walk, 0, tm_c, tn_c);
+  __amdgpu_buffer_rsrc_t ra_c = make_a(tm_c, true), rb_c = make_b(tn_c, true), ra_n, rb_n;
+  bool nxt_valid = false, nxt_pending = false;
+  auto plan_next = [&]() {
+    nxt_valid = own_idx + 1 < walk.own_count;
+    nxt_pending = !nxt_valid && pool_n > 0;
+    if (nxt_valid) scan_walk_own(walk, ++own_idx, tm_n, tn_n);
+    ra_n = make_a(tm_n, nxt_valid);
+    rb_n = make_b(tn_n, nxt_valid);
+  };
+  plan_next();
+  uint32_t* const pool_counter = sched;
+  uint32_t* const my_claim = sched + kSchedCounterWords + blockIdx.x;
+  const bool drawer = wave == 0;
+  const uint32_t zero_off = 0;
+
+  // ---- epilogue state: see score_gemm_kernel's epilogue, of which this is the 4 x 4 block form ----
+  // acc block (i, j), element e: row 8 * (e / 4) + 4 * half + e % 4 of row block i, column l32 of column block j.
+  const int n_queries = M_rows / (blocks_per_query * 32);
+  typedef const __attribute__((address_space(4))) uint32_t* const_words_t;      // scalar loads
+  const const_words_t row_bits_c = (const_words_t)row_bits;
+  uint32_t rbits[4];
+  int q_first = 0, r_first = 0;
+  auto fetch_rows = [&](int m0) {
+    const int blk0 = (m0 + wm * 128) >> 5;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rbits[i] = row_bits_c[blk0 + i];          // 0 past M_rows (the buffer is padded)
+    q_first = blk0 / blocks_per_query;
+    r_first = blk0 - q_first * blocks_per_query;
+  };
+  // the documents of the wavefront's 128 columns, 64 per load, into v220 / v221 (v224: their offsets): requested in
+  // front of a tile's first K step (whose waits cover them), read in the tile's epilogue; columns past the bank read 0
+  // and are masked below
+  auto fetch_docs = [&](int n0) {
+    if constexpr (kDocMax) {
+      const int first = (n0 + wn * 128) * 4;      // (in the vector offset, which is what the extent is checked against)
+      asm volatile("s_nop 4\n\tv_add_u32 v224, %1, v222\n\tbuffer_load_dword v220, v224, %0, 0 offen\n\t"
+                   "buffer_load_dword v221, v224, %0, 0 offen offset:256"
+                   ::"s"(rsrc_docs), "s"(first) : MSA_SCAN4_CLOBBERS);
+    }
+  };
+  // One pair of column blocks (64 columns): after the half-wave swap the lower 32 lanes hold block 2p's column maxima
+  // and the upper 32 lanes block 2p + 1's; the segmented scan then leaves a document's maximum in the last lane of its
+  // run, which alone touches memory.
+  auto emit_pair = [&](int q, int n_first, float lo, float hi, int doc_raw) {
+    const auto sw = __builtin_amdgcn_permlane32_swap(__float_as_uint(lo), __float_as_uint(hi), false, false);
+    const float run = fmaxf(__uint_as_float(sw[0]), __uint_as_float(sw[1]));
+    const int n = n_first + lane;
+    const bool ok = n < C;
+    const uint32_t key = ok ? f32_to_key(run) : 0u;
+    if constexpr (kDocMax) {
+      const int doc = ok ? doc_raw : -1 - l32;
+      const int prev = __builtin_amdgcn_update_dpp(doc, doc, 0x138, 0xF, 0xF, false);      // wave_shr:1
+      const uint64_t heads64 = __ballot(l32 == 0 || prev != doc);
+      const uint32_t heads = half ? (uint32_t)(heads64 >> 32) : (uint32_t)heads64;
+      const uint32_t upto = heads & ((2u << l32) - 1u);                  // heads at or below this lane (never empty)
+      const int dist = l32 - (31 - __builtin_clz(upto));
+      const bool last = l32 == 31 || ((heads >> (l32 + 1)) & 1u);
+      int m = (int)key;
+#define MSA_SCAN_STEP(OFF, CTRL)                                                          \
+      {                                                                                   \
+        const int o = __builtin_amdgcn_update_dpp(0, m, CTRL, 0xF, 0xF, true);            \
+        if (dist >= OFF) m = (int)max((uint32_t)m, (uint32_t)o);                          \
+      }
+      MSA_SCAN_STEP(1, 0x111)   // row_shr:1
+      MSA_SCAN_STEP(2, 0x112)
+      MSA_SCAN_STEP(4, 0x114)
+      MSA_SCAN_STEP(8, 0x118)
+#undef MSA_SCAN_STEP
+      const int low = __builtin_amdgcn_update_dpp(0, m, 0x142, 0xA, 0xF, false);          // row_bcast:15 into rows 1, 3
+      if (dist > (l32 & 15)) m = (int)max((uint32_t)m, (uint32_t)low);
+      if (ok && last) atomicMax(&out_key[(int64_t)q * n_docs + doc], (uint32_t)m);
+    } else {
+      if (ok) atomicMax(&out_key[(int64_t)q * C + n], key);
+    }
+  };
+  auto epilogue = [&](int n0) {
+    int doc0 = 0, doc1 = 0;
+    // (the s_nops: an MFMA's result may be read 18 wait states after its issue at the earliest)
+    if constexpr (kDocMax) asm volatile("s_nop 15\n\ts_nop 7\n\tv_mov_b32 %0, v220\n\tv_mov_b32 %1, v221" : "=v"(doc0), "=v"(doc1));
+    else asm volatile("s_nop 15\n\ts_nop 7");
+    float run[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+    bool any = false;
+    int run_q = q_first, r = r_first;
+    auto emit = [&]() {
+      if (!any || run_q >= n_queries) return;
+      emit_pair(run_q, n0 + wn * 128, run[0], run[1], doc0);
+      emit_pair(run_q, n0 + wn * 128 + 64, run[2], run[3], doc1);
+    };
+    auto row_block = [&](auto i_tag) {
+      constexpr int i = decltype(i_tag)::value;
+      const uint32_t bits = rbits[i];
+      if (r == blocks_per_query) {                         // row block i opens the next query
+        emit();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) run[j] = -INFINITY;
+        any = false; ++run_q; r = 0;
+      }
+      ++r;
+      if (bits == 0) return;
+      any = true;
+      auto col_block = [&](auto j_tag) {
+        constexpr int j = decltype(j_tag)::value;
+        float x[16];
+        scan4_read_acc<i * 4 + j>(x);
+        float mx = -INFINITY;
+        if (bits == 0xffffffffu) {                          // every row scored: no per-row tests
+#pragma unroll
+          for (int e = 0; e < 16; ++e) mx = fmaxf(mx, x[e]);
+        } else {
+          const uint32_t mine = bits >> (4 * half);         // this half's rows: bit 8 * (e / 4) + e % 4
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            if (mine & (1u << (8 * (e >> 2) + (e & 3)))) mx = fmaxf(mx, x[e]);
+        }
+        run[j] = fmaxf(run[j], mx);
+      };
+      col_block(std::integral_constant<int, 0>{}); col_block(std::integral_constant<int, 1>{});
+      col_block(std::integral_constant<int, 2>{}); col_block(std::integral_constant<int, 3>{});
+    };
+    row_block(std::integral_constant<int, 0>{}); row_block(std::integral_constant<int, 1>{});
+    row_block(std::integral_constant<int, 2>{}); row_block(std::integral_constant<int, 3>{});
+    emit();
+  };
+
+  // ---- prologue: the first two K tiles of the first tile, the first fragments ----
+  const int woff = wave * 8192;
+  int sa = 0, sb = 0x10000;
+  asm volatile(MSA_SCAN4_LOAD8_NT ::[dst] "s"(0x10000 + woff), [r] "s"(rb_c), [k] "s"(0) : MSA_SCAN4_CLOBBERS);
+  asm volatile(MSA_SCAN4_LOAD8 ::[dst] "s"(0 + woff), [r] "s"(ra_c), [k] "s"(0) : MSA_SCAN4_CLOBBERS);
+  asm volatile(MSA_SCAN4_LOAD8_NT ::[dst] "s"(0x18000 + woff), [r] "s"(rb_c), [k] "s"(kRowBytes) : MSA_SCAN4_CLOBBERS);
+  asm volatile(MSA_SCAN4_LOAD8 ::[dst] "s"(0x8000 + woff), [r] "s"(ra_c), [k] "s"(kRowBytes) : MSA_SCAN4_CLOBBERS);
+  asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+  asm volatile(MSA_SCAN4_FRAGS0 ::[sa] "s"(sa), [sb] "s"(sb) : MSA_SCAN4_CLOBBERS);
+
+  for (;;) {
+    const int n0 = tn_c * BN;
+    fetch_rows(tm_c * BM);
+    fetch_docs(n0);
+    // Step kt requests K tile kt + 2: of this tile while it has one, of the next tile after that.  The steps are laid
+    // out so that between two of them the scalar unit has next to nothing to do (a wavefront that is alone on its SIMD
+    // pays for every instruction between two MFMAs): the resources a step reads are fixed per loop, and the tile
+    // pool's hops ride in front of four peeled steps.
+#define MSA_SCAN4_STEP(TEXT, RA, RB, KOFF)                                                                   \
+    asm volatile(TEXT : [sa] "+s"(sa), [sb] "+s"(sb)                                                         \
+                 : [ra] "s"(RA), [rb] "s"(RB), [k] "s"(KOFF), [woff] "s"(woff) : MSA_SCAN4_CLOBBERS)
+    int kt;
+    if (nxt_pending) {                   // the tile behind this one comes from the pool (k_tiles >= 6 then)
+      if (drawer && lane == 0)           // v217 = counter++
+        asm volatile("s_nop 4\n\tglobal_atomic_add v217, %0, v223, %1 sc0" ::"v"(zero_off), "s"(pool_counter) : "memory");
+      MSA_SCAN4_STEP(MSA_SCAN4_KSTEP_FRESH, ra_c, rb_c, 2 * kRowBytes);
+      if (drawer && lane == 0)           // claim word = v217; its old value comes back in v218
+        asm volatile("s_nop 4\n\tglobal_atomic_swap v218, %0, v217, %1 sc0" ::"v"(zero_off), "s"(my_claim) : "memory");
+      MSA_SCAN4_STEP(MSA_SCAN4_KSTEP, ra_c, rb_c, 3 * kRowBytes);
+      // every wavefront reads the word back (past the L1: device scope)
+      asm volatile("s_nop 4\n\tglobal_load_dword v219, %0, %1 sc1" ::"v"(zero_off), "s"(my_claim) : "memory");
+      MSA_SCAN4_STEP(MSA_SCAN4_KSTEP, ra_c, rb_c, 4 * kRowBytes);
+      int p_next;                        // complete since the last step's wait
+      asm volatile("v_readfirstlane_b32 %0, v219" : "=s"(p_next));
+      nxt_pending = false;
+      nxt_valid = p_next < walk.pool_total;
+      if (nxt_valid) scan_walk_pool(walk, p_next, tm_n, tn_n);
+      ra_n = make_a(tm_n, nxt_valid);
+      rb_n = make_b(tn_n, nxt_valid);
+      MSA_SCAN4_STEP(MSA_SCAN4_KSTEP, ra_c, rb_c, 5 * kRowBytes);
+      kt = 4;
+    } else {
+      if (k_tiles > 2) MSA_SCAN4_STEP(MSA_SCAN4_KSTEP_FRESH, ra_c, rb_c, 2 * kRowBytes);
+      else MSA_SCAN4_STEP(MSA_SCAN4_KSTEP_FRESH, ra_n, rb_n, 0);
+      kt = 1;
+    }
+    for (int k_l = (kt + 2) * kRowBytes; k_l < row_bytes; k_l += kRowBytes) MSA_SCAN4_STEP(MSA_SCAN4_KSTEP, ra_c, rb_c, k_l);
+    for (int k_l = k_tiles > 2 ? 0 : kRowBytes; k_l < 2 * kRowBytes; k_l += kRowBytes) MSA_SCAN4_STEP(MSA_SCAN4_KSTEP, ra_n, rb_n, k_l);
+#undef MSA_SCAN4_STEP
+    epilogue(n0);
+    if (!nxt_valid) break;
+    tm_c = tm_n; tn_c = tn_n;
+    ra_c = ra_n; rb_c = rb_n;
+    plan_next();
+  }
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+#endif
+}
+
 // chunk_key -> fp32 scores (times scale / Hq); key 0 (query without a scored token) -> -inf.
 __global__ void decode_scores_kernel(const uint32_t* __restrict__ key, int64_t n, float mul,
                                      float* __restrict__ out) {
@@ -1021,6 +1329,58 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
   return MSA_OK;
 }
 
+// Launch of the MFMA-bound form (score_scan4_kernel): one workgroup per compute unit, persistent.
+std::atomic<int> g_tile_pool_enabled{1};
+
+template <bool kDocMax>
+int launch_scan4(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key, const int32_t* chunk_doc,
+                 int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t n_docs, hipStream_t st,
+                 const GatherJob* job, bool* job_taken, uint32_t* sched) {
+  constexpr int BM = 256, BN = 256;
+  const int tiles_m = (M_rows + BM - 1) / BM;
+  const int tiles_n = (C + BN - 1) / BN;
+  const int k_tiles = K * (int)sizeof(bf16_t) / kRowBytes;
+  // the loop requests K tiles two steps ahead: at least two K tiles per tile
+  if (K * (int)sizeof(bf16_t) % kRowBytes != 0 || k_tiles < 2) {
+    msa_set_error("score_scan4: K=%d is not a multiple of 64 of at least 128", K);
+    return MSA_EINVAL;
+  }
+  // M tiles are walked in groups of 8 per K_r tile: a group's query rows (4 MiB in bf16) are what an XCD's L2 holds.
+  // At 8 M tiles that is all of them (groups of 1, 2, 4 lose 2-14 % there); with 16 M tiles groups of 8 measured
+  // 1.4 % faster than one group, with 256 (a 64k-row prefill batch) 4 %.
+  const int m_group = std::min(tiles_m, 8);
+  const int grid = std::min(kSchedMaxWorkgroups, std::max(16, compute_units() / 8 * 8));
+  // The XCDs do not run at one speed (their ends lay up to 6 % apart with fixed ranges, in an order that changes from
+  // launch to launch): the last eighth of the N tiles is a pool the workgroups draw from one tile at a time once
+  // their own share is done.  Worth it when a workgroup has tiles enough for the pool to even the ends out, and
+  // possible when a tile is deep enough for a draw to come back in time (three hops, one per K step, in front of the
+  // step in which the loads leave the tile).
+  int pool_n = 0;
+  if (g_tile_pool_enabled.load(std::memory_order_relaxed) && (int64_t)tiles_m * tiles_n >= (int64_t)16 * grid && k_tiles >= 6)
+    pool_n = tiles_n / 8;
+  GatherJob no_job{};
+  const GatherJob* the_job = &no_job;
+  if (job != nullptr && job->active) {
+    the_job = job;
+    if (job_taken) *job_taken = true;
+  }
+  auto kern = score_scan4_kernel<kDocMax>;
+  static std::atomic<int> lds_limit_raised{0};
+  MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(kern), kScan4LdsBytes));
+  int slot = -1;
+  if (g_timer.on.load(std::memory_order_acquire)) {
+    std::lock_guard<std::mutex> lock(g_timer.mu);
+    if (g_timer.n < g_timer.cap) slot = g_timer.n++;
+  }
+  if (slot >= 0) MSA_HIP(hipEventRecord(g_timer.start[slot], st));
+  kern<<<grid, 256, kScan4LdsBytes, st>>>(static_cast<const bf16_t*>(qs), static_cast<const bf16_t*>(kr), row_bits, out_key,
+                                          chunk_doc, M_rows, C, K, blocks_per_query, tiles_m, tiles_n, m_group, n_docs,
+                                          *the_job, sched, pool_n);
+  MSA_LAUNCH_CHECK();
+  if (slot >= 0) MSA_HIP(hipEventRecord(g_timer.stop[slot], st));
+  return MSA_OK;
+}
+
 // Tile choice by query rows.  Up to 64 rows: narrow M tile, two workgroups per compute unit, two K tiles of global
 // loads ahead (3 % faster than one).  Up to 128 rows: 128 x 256 with both operands loaded straight into LDS two K steps
 // ahead (1.5 % faster than the register-staged 128 x 384 it replaced, which beat register-staged 128 x 256 by 3 % and
@@ -1037,7 +1397,7 @@ int launch_gemm_for(int32_t dtype, const void* qs, const void* kr, const uint32_
     return launch_gemm<bf16_t, 64, 128, 2, 2, 2, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
   if (M_rows <= 128)
     return launch_gemm<bf16_t, 128, 256, 2, 4, 1, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
-  return launch_gemm<bf16_t, 256, 256, 2, 4, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
+  return launch_scan4<kDocMax>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
 }
 
 }  // namespace

@@ -24,8 +24,11 @@ typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 // ------------------------------------------------------------------------------------------
 // Prologue: normalise (cosine mode), sum the G heads of each KV group, cast, build row masks, clear the key plane.
 // One workgroup of Hkv*16 lanes per (b, padded token); lane (g, j) owns 8 contiguous d of group g.
-// The workgroup of every 32nd row also writes the scored-row bitmask word of its 32 rows (a ballot, no atomics),
-// workgroup 0 the zero words that pad the mask to whole M tiles, and all workgroups together clear the
+// A row that is not scored (a masked token, or the padding of a query to a multiple of 32 rows) repeats the query's
+// first scored row: a repeated row changes no maximum, so the scoring epilogues fold whole 32-row blocks without
+// per-row tests.  A query without any scored token keeps rows of zeros and mask words of zero: its row blocks are
+// skipped and its keys stay 0.  The workgroup of every 32nd row writes the mask word of its 32 rows (all ones or
+// zero), workgroup 0 the zero words that pad the mask to whole M tiles, and all workgroups together clear the
 // `clear_words` key words the scoring kernel merges into with atomicMax.
 // ------------------------------------------------------------------------------------------
 // Words behind the persistent scan's tile pool: the pool's counter, on a cache line of its own, then one word per
@@ -40,24 +43,36 @@ __global__ void presum_queries_kernel(const TIn* __restrict__ q, const uint8_t* 
                                       TOut* __restrict__ qs, uint32_t* __restrict__ row_bits, int32_t mask_words,
                                       uint32_t* __restrict__ key_plane, int64_t clear_words, uint32_t* __restrict__ sched) {
   const int row = blockIdx.x;              // b * S_pad + s
-  const int b = row / S_pad, s = row % S_pad;
+  const int b = row / S_pad;
+  int s = row % S_pad;
   const int G = Hq / Hkv;
   const int g = threadIdx.x >> 4, j = threadIdx.x & 15;
-  auto scored = [&](int r) {
-    const int rb = r / S_pad, rs = r % S_pad;
-    return rs < S && (qmask == nullptr || qmask[(int64_t)rb * S + rs] != 0);
-  };
-  const bool valid = scored(row);
+  bool valid = s < S && (qmask == nullptr || qmask[(int64_t)b * S + s] != 0);
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words; i += (int64_t)gridDim.x * blockDim.x)
     key_plane[i] = 0u;
-  if ((row & 31) == 0 && threadIdx.x < 64) {          // rows are padded per query to a multiple of 32
-    const int nl = min((int)blockDim.x, 32);
-    uint32_t bits = 0;
-    for (int base = 0; base < 32; base += nl) {
-      const bool v = (int)threadIdx.x < nl && scored(row + base + (int)threadIdx.x);
-      bits |= (uint32_t)__ballot(v) << base;
+  const bool writes_word = (row & 31) == 0;           // rows are padded per query to a multiple of 32
+  if (!valid || writes_word) {                        // (uniform over the workgroup)
+    // the query's first scored token, found by the workgroup's first wavefront
+    __shared__ int first_scored;
+    if (threadIdx.x < 64) {
+      const int nl = min((int)blockDim.x, 64);
+      int found = qmask == nullptr ? 0 : -1;
+      for (int base = 0; base < S && found < 0; base += nl) {
+        const int t = base + (int)threadIdx.x;
+        const bool v = (int)threadIdx.x < nl && t < S && qmask[(int64_t)b * S + t] != 0;
+        const uint64_t m = __ballot(v);
+        if (m != 0) found = base + __builtin_ctzll(m);
+      }
+      if (threadIdx.x == 0) {
+        first_scored = found;
+        if (writes_word) row_bits[row >> 5] = found >= 0 ? 0xffffffffu : 0u;
+      }
     }
-    if (threadIdx.x == 0) row_bits[row >> 5] = bits;
+    __syncthreads();
+    if (!valid && first_scored >= 0) {
+      s = first_scored;
+      valid = true;
+    }
   }
   if (blockIdx.x == 0) {
     for (int w = (int)(gridDim.x >> 5) + (int)threadIdx.x; w < mask_words; w += blockDim.x) row_bits[w] = 0u;
@@ -952,22 +967,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vg
 constexpr int kScan4CompilerVgprs = 128;     // the compiler's share of the vector registers in score_scan4_kernel
 constexpr int kScan4LdsBytes = 5 * 256 * 128;
 
-#if defined(__HIP_DEVICE_COMPILE__)
-template <int N>
-__device__ __forceinline__ void scan4_read_acc(float (&x)[16]);
-#define MSA_SCAN4_READER(N)                                                                                          \
-  template <>                                                                                                       \
-  __device__ __forceinline__ void scan4_read_acc<N>(float (&x)[16]) {                                               \
-    asm volatile(MSA_SCAN4_ACC_READ_##N                                                                              \
-                 : "=v"(x[0]), "=v"(x[1]), "=v"(x[2]), "=v"(x[3]), "=v"(x[4]), "=v"(x[5]), "=v"(x[6]), "=v"(x[7]),    \
-                   "=v"(x[8]), "=v"(x[9]), "=v"(x[10]), "=v"(x[11]), "=v"(x[12]), "=v"(x[13]), "=v"(x[14]), "=v"(x[15])); \
-  }
-MSA_SCAN4_READER(0) MSA_SCAN4_READER(1) MSA_SCAN4_READER(2) MSA_SCAN4_READER(3) MSA_SCAN4_READER(4) MSA_SCAN4_READER(5)
-MSA_SCAN4_READER(6) MSA_SCAN4_READER(7) MSA_SCAN4_READER(8) MSA_SCAN4_READER(9) MSA_SCAN4_READER(10) MSA_SCAN4_READER(11)
-MSA_SCAN4_READER(12) MSA_SCAN4_READER(13) MSA_SCAN4_READER(14) MSA_SCAN4_READER(15)
-#undef MSA_SCAN4_READER
-#endif
-
 template <bool kDocMax>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerVgprs))) void score_scan4_kernel(
     const bf16_t* __restrict__ qs,          // [M_rows, K]  pre-summed queries, M_rows = B * S_pad
@@ -1029,6 +1028,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerV
                  : MSA_SCAN4_CLOBBERS);
     // v222: byte offset of a lane's column in a run of 64 document ids; v223: the pool counter's increment
     asm volatile("v_lshlrev_b32 v222, 2, %0\n\tv_mov_b32 v223, 1" ::"v"(lane) : MSA_SCAN4_CLOBBERS);
+    asm volatile(MSA_SCAN4_SET_FOLD ::"v"(l32) : MSA_SCAN4_CLOBBERS);
   }
   const char* ga = reinterpret_cast<const char*>(qs);
   const char* gb = reinterpret_cast<const char*>(kr);
@@ -1070,7 +1070,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerV
   const int n_queries = M_rows / (blocks_per_query * 32);
   typedef const __attribute__((address_space(4))) uint32_t* const_words_t;      // scalar loads
   const const_words_t row_bits_c = (const_words_t)row_bits;
-  uint32_t rbits[4];
+  uint32_t rbits[4] = {0u, 0u, 0u, 0u};
   int q_first = 0, r_first = 0;
   auto fetch_rows = [&](int m0) {
     const int blk0 = (m0 + wm * 128) >> 5;
@@ -1079,14 +1079,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerV
     q_first = blk0 / blocks_per_query;
     r_first = blk0 - q_first * blocks_per_query;
   };
-  // the documents of the wavefront's 128 columns, 64 per load, into v220 / v221 (v224: their offsets): requested in
-  // front of a tile's first K step (whose waits cover them), read in the tile's epilogue; columns past the bank read 0
+  // the documents of the wavefront's 128 columns, 64 per load, into v220 / v221 (v216: their offsets): requested in
+  // front of a K step (whose waits cover them), read when the tile's maxima are folded; columns past the bank read 0
   // and are masked below
   auto fetch_docs = [&](int n0) {
     if constexpr (kDocMax) {
       const int first = (n0 + wn * 128) * 4;      // (in the vector offset, which is what the extent is checked against)
-      asm volatile("s_nop 4\n\tv_add_u32 v224, %1, v222\n\tbuffer_load_dword v220, v224, %0, 0 offen\n\t"
-                   "buffer_load_dword v221, v224, %0, 0 offen offset:256"
+      asm volatile("s_nop 4\n\tv_add_u32 v216, %1, v222\n\tbuffer_load_dword v220, v216, %0, 0 offen\n\t"
+                   "buffer_load_dword v221, v216, %0, 0 offen offset:256"
                    ::"s"(rsrc_docs), "s"(first) : MSA_SCAN4_CLOBBERS);
     }
   };
@@ -1125,11 +1125,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerV
       if (ok) atomicMax(&out_key[(int64_t)q * C + n], key);
     }
   };
-  auto epilogue = [&](int n0) {
+  // Folds the finished tile's block maxima (v224 - v239, left by the reduction that rides in the next tile's first K
+  // step or by the stand-alone one): row blocks of one query are joined, and at a query's end the two pairs of column
+  // blocks are merged into the key plane.  Every row of a scored block counts (the prologue kernel made unscored rows
+  // repeat a scored one); a block whose mask word is zero belongs to a query without scored tokens or to the padding
+  // past M_rows and is skipped.
+  auto fold_tile = [&](int n0) {
+    float mx[16];
+    asm volatile(MSA_SCAN4_MAX_READ
+                 : "=v"(mx[0]), "=v"(mx[1]), "=v"(mx[2]), "=v"(mx[3]), "=v"(mx[4]), "=v"(mx[5]), "=v"(mx[6]), "=v"(mx[7]),
+                   "=v"(mx[8]), "=v"(mx[9]), "=v"(mx[10]), "=v"(mx[11]), "=v"(mx[12]), "=v"(mx[13]), "=v"(mx[14]), "=v"(mx[15]));
     int doc0 = 0, doc1 = 0;
-    // (the s_nops: an MFMA's result may be read 18 wait states after its issue at the earliest)
-    if constexpr (kDocMax) asm volatile("s_nop 15\n\ts_nop 7\n\tv_mov_b32 %0, v220\n\tv_mov_b32 %1, v221" : "=v"(doc0), "=v"(doc1));
-    else asm volatile("s_nop 15\n\ts_nop 7");
+    if constexpr (kDocMax) asm volatile("v_mov_b32 %0, v220\n\tv_mov_b32 %1, v221" : "=v"(doc0), "=v"(doc1));
     float run[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
     bool any = false;
     int run_q = q_first, r = r_first;
@@ -1138,9 +1145,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerV
       emit_pair(run_q, n0 + wn * 128, run[0], run[1], doc0);
       emit_pair(run_q, n0 + wn * 128 + 64, run[2], run[3], doc1);
     };
-    auto row_block = [&](auto i_tag) {
-      constexpr int i = decltype(i_tag)::value;
-      const uint32_t bits = rbits[i];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
       if (r == blocks_per_query) {                         // row block i opens the next query
         emit();
 #pragma unroll
@@ -1148,29 +1154,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerV
         any = false; ++run_q; r = 0;
       }
       ++r;
-      if (bits == 0) return;
-      any = true;
-      auto col_block = [&](auto j_tag) {
-        constexpr int j = decltype(j_tag)::value;
-        float x[16];
-        scan4_read_acc<i * 4 + j>(x);
-        float mx = -INFINITY;
-        if (bits == 0xffffffffu) {                          // every row scored: no per-row tests
+      if (rbits[i] != 0) {
+        any = true;
 #pragma unroll
-          for (int e = 0; e < 16; ++e) mx = fmaxf(mx, x[e]);
-        } else {
-          const uint32_t mine = bits >> (4 * half);         // this half's rows: bit 8 * (e / 4) + e % 4
-#pragma unroll
-          for (int e = 0; e < 16; ++e)
-            if (mine & (1u << (8 * (e >> 2) + (e & 3)))) mx = fmaxf(mx, x[e]);
-        }
-        run[j] = fmaxf(run[j], mx);
-      };
-      col_block(std::integral_constant<int, 0>{}); col_block(std::integral_constant<int, 1>{});
-      col_block(std::integral_constant<int, 2>{}); col_block(std::integral_constant<int, 3>{});
-    };
-    row_block(std::integral_constant<int, 0>{}); row_block(std::integral_constant<int, 1>{});
-    row_block(std::integral_constant<int, 2>{}); row_block(std::integral_constant<int, 3>{});
+        for (int j = 0; j < 4; ++j) run[j] = fmaxf(run[j], mx[i * 4 + j]);
+      }
+    }
     emit();
   };
 
@@ -1184,10 +1173,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerV
   asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
   asm volatile(MSA_SCAN4_FRAGS0 ::[sa] "s"(sa), [sb] "s"(sb) : MSA_SCAN4_CLOBBERS);
 
+  // A tile's accumulators are reduced inside the next tile's first K step and folded right behind it, so the fold of
+  // tile t uses the row words and the documents fetched for t; those of t + 1 are requested once it is done.
+  bool have_prev = false;
+  int prev_n0 = 0;
   for (;;) {
-    const int n0 = tn_c * BN;
-    fetch_rows(tm_c * BM);
-    fetch_docs(n0);
     // Step kt requests K tile kt + 2: of this tile while it has one, of the next tile after that.  The steps are laid
     // out so that between two of them the scalar unit has next to nothing to do (a wavefront that is alone on its SIMD
     // pays for every instruction between two MFMAs): the resources a step reads are fixed per loop, and the tile
@@ -1195,11 +1185,36 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerV
 #define MSA_SCAN4_STEP(TEXT, RA, RB, KOFF)                                                                   \
     asm volatile(TEXT : [sa] "+s"(sa), [sb] "+s"(sb)                                                         \
                  : [ra] "s"(RA), [rb] "s"(RB), [k] "s"(KOFF), [woff] "s"(woff) : MSA_SCAN4_CLOBBERS)
-    int kt;
-    if (nxt_pending) {                   // the tile behind this one comes from the pool (k_tiles >= 6 then)
-      if (drawer && lane == 0)           // v217 = counter++
-        asm volatile("s_nop 4\n\tglobal_atomic_add v217, %0, v223, %1 sc0" ::"v"(zero_off), "s"(pool_counter) : "memory");
-      MSA_SCAN4_STEP(MSA_SCAN4_KSTEP_FRESH, ra_c, rb_c, 2 * kRowBytes);
+    const bool pending = nxt_pending;      // the tile behind this one comes from the pool (k_tiles >= 6 then)
+    if (pending && drawer && lane == 0)    // v217 = counter++
+      asm volatile("s_nop 4\n\tglobal_atomic_add v217, %0, v223, %1 sc0" ::"v"(zero_off), "s"(pool_counter) : "memory");
+    // What the finished tile left is reduced inside this tile's first step.  Usually the wavefront's four row blocks
+    // are one query whose rows all count (blocks_per_query a multiple of 4: queries of 128, 256, ... padded tokens) and
+    // the tile lies inside the bank: then the step also folds the maxima into the key plane.  Otherwise it leaves one
+    // maximum per block and fold_tile() does the rest; a wavefront whose rows are all padding has nothing to fold.
+    const bool fold_any = have_prev && (rbits[0] | rbits[1] | rbits[2] | rbits[3]) != 0;
+    const bool fold_fast = kDocMax && fold_any && (blocks_per_query & 3) == 0 && rbits[0] != 0 && prev_n0 + BN <= C;
+    if (fold_fast) {
+      const uint32_t* okey = out_key + (int64_t)q_first * n_docs;
+      if (k_tiles > 2)
+        asm volatile(MSA_SCAN4_KSTEP_FRESH_FOLD : [sa] "+s"(sa), [sb] "+s"(sb)
+                     : [ra] "s"(ra_c), [rb] "s"(rb_c), [k] "s"(2 * kRowBytes), [woff] "s"(woff), [okey] "s"(okey) : MSA_SCAN4_CLOBBERS);
+      else
+        asm volatile(MSA_SCAN4_KSTEP_FRESH_FOLD : [sa] "+s"(sa), [sb] "+s"(sb)
+                     : [ra] "s"(ra_n), [rb] "s"(rb_n), [k] "s"(0), [woff] "s"(woff), [okey] "s"(okey) : MSA_SCAN4_CLOBBERS);
+    } else if (fold_any) {
+      if (k_tiles > 2) MSA_SCAN4_STEP(MSA_SCAN4_KSTEP_FRESH_REDUCE, ra_c, rb_c, 2 * kRowBytes);
+      else MSA_SCAN4_STEP(MSA_SCAN4_KSTEP_FRESH_REDUCE, ra_n, rb_n, 0);
+      fold_tile(prev_n0);
+    } else {
+      if (k_tiles > 2) MSA_SCAN4_STEP(MSA_SCAN4_KSTEP_FRESH, ra_c, rb_c, 2 * kRowBytes);
+      else MSA_SCAN4_STEP(MSA_SCAN4_KSTEP_FRESH, ra_n, rb_n, 0);
+    }
+    const int n0 = tn_c * BN;
+    fetch_rows(tm_c * BM);
+    fetch_docs(n0);
+    int kt = 1;
+    if (pending) {
       if (drawer && lane == 0)           // claim word = v217; its old value comes back in v218
         asm volatile("s_nop 4\n\tglobal_atomic_swap v218, %0, v217, %1 sc0" ::"v"(zero_off), "s"(my_claim) : "memory");
       MSA_SCAN4_STEP(MSA_SCAN4_KSTEP, ra_c, rb_c, 3 * kRowBytes);
@@ -1215,20 +1230,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerV
       rb_n = make_b(tn_n, nxt_valid);
       MSA_SCAN4_STEP(MSA_SCAN4_KSTEP, ra_c, rb_c, 5 * kRowBytes);
       kt = 4;
-    } else {
-      if (k_tiles > 2) MSA_SCAN4_STEP(MSA_SCAN4_KSTEP_FRESH, ra_c, rb_c, 2 * kRowBytes);
-      else MSA_SCAN4_STEP(MSA_SCAN4_KSTEP_FRESH, ra_n, rb_n, 0);
-      kt = 1;
     }
     for (int k_l = (kt + 2) * kRowBytes; k_l < row_bytes; k_l += kRowBytes) MSA_SCAN4_STEP(MSA_SCAN4_KSTEP, ra_c, rb_c, k_l);
     for (int k_l = k_tiles > 2 ? 0 : kRowBytes; k_l < 2 * kRowBytes; k_l += kRowBytes) MSA_SCAN4_STEP(MSA_SCAN4_KSTEP, ra_n, rb_n, k_l);
 #undef MSA_SCAN4_STEP
-    epilogue(n0);
+    have_prev = true;
+    prev_n0 = n0;
     if (!nxt_valid) break;
     tm_c = tm_n; tn_c = tn_n;
     ra_c = ra_n; rb_c = rb_n;
     plan_next();
   }
+  asm volatile(MSA_SCAN4_REDUCE ::: MSA_SCAN4_CLOBBERS);
+  fold_tile(prev_n0);
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
 #endif
 }

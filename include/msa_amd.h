@@ -147,6 +147,21 @@ int msa_profile_collect(float* ms_host, int32_t cap, int32_t* n_out);
  * (the budget of a kernel that does softmax arithmetic between them). */
 int msa_diag_mfma_loop(int32_t workgroups, int32_t iters, int32_t mode, float* sink, double* flops_out, void* stream);
 
+/* Test aid (no counterpart in the reference; runs on the host, no GPU needed): replays the tile order of the
+ * persistent large-tile scan (more than 128 query rows) for a launch of `grid` workgroups over tiles_m x tiles_n
+ * tiles of 256 x 256, with or without the workgroup that copies K / V rows instead of scoring, the last pool_n N
+ * tiles handed out from the shared pool.  visits (host, [tiles_m * tiles_n], M-major) receives how often each tile is
+ * scored: all ones for a correct order.  Fails if the kernel's incremental tile cursor and the closed form of the
+ * order disagree anywhere. */
+int msa_diag_scan_walk(int32_t tiles_m, int32_t tiles_n, int32_t grid, int32_t has_copy_workgroup, int32_t pool_n,
+                       int32_t* visits);
+
+/* Switch (no counterpart in the reference): the large-tile scan hands the last eighth of its tiles out dynamically,
+ * from a counter in the workspace, to even out the ends of the eight XCDs.  enabled = 0 gives every tile a fixed
+ * workgroup (a few percent slower on large banks; no atomics on the hand-out path); 1 is the default.  Process-wide,
+ * takes effect at the next call. */
+int msa_route_set_tile_pool(int32_t enabled);
+
 /* Test aid (no counterpart in the reference): `workgroups` workgroups that each claim a compute unit's whole LDS
  * (160 KB) and fill it with `word`; check (device, [workgroups], may be null) receives one word read back per
  * workgroup.  LDS is not cleared between kernels, so a launch of a few workgroups per compute unit leaves every unit's

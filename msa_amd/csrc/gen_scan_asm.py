@@ -197,23 +197,20 @@ def kstep(fresh, reduce=None):
         (a0, at0), (a1, at1) = fold_pair(0), fold_pair(1)
         fillers = interleave(a0, a1)
         atomics = at0 + at1
-        e("s_mov_b32 s86, 0")
-        e("s_mov_b32 s87, -1")
     per_slot = -(-len(fillers) // 32)
-    e(f"s_mov_b32 {S_M0}, m0")
-    e(f"s_add_u32 {S_BN}, %[sb], 0x8000")
-    e(f"s_cmp_eq_u32 {S_BN}, {BEND:#x}")
-    e(f"s_cselect_b32 {S_BN}, {B0:#x}, {S_BN}")
-    e(f"s_sub_u32 {S_BLD}, %[sb], 0x8000")
-    e(f"s_cmp_lt_u32 {S_BLD}, {B0:#x}")
-    e(f"s_cselect_b32 {S_BLD}, {BEND - 0x8000:#x}, {S_BLD}")
-    e(f"s_xor_b32 {S_AN}, %[sa], 0x8000")
-    for s in (1, 2, 3):
-        e(f"v_add_u32 v{VT + 2 * (s - 1)}, %[sa], v{VADDR_A + s}")
-        e(f"v_add_u32 v{VT + 2 * (s - 1) + 1}, %[sb], v{VADDR_B + s}")
-    e(f"v_add_u32 v{VT + 6}, {S_AN}, v{VADDR_A}")
-    e(f"v_add_u32 v{VT + 7}, {S_BN}, v{VADDR_B}")
-    e(f"s_add_u32 {S_BLD}, {S_BLD}, %[woff]")
+    # The step's scalar and address arithmetic stands behind its first MFMAs, not in front of them (a wavefront that
+    # is alone on its SIMD pays for every instruction the matrix pipe does not run under): `early` is what the first
+    # LDS read and the first tile load need, `later` the rest, three instructions per MFMA.
+    early = [f"s_mov_b32 {S_M0}, m0",
+             f"v_add_u32 v{VT}, %[sa], v{VADDR_A + 1}", f"v_add_u32 v{VT + 1}, %[sb], v{VADDR_B + 1}",
+             f"s_sub_u32 {S_BLD}, %[sb], 0x8000", f"s_cmp_lt_u32 {S_BLD}, {B0:#x}",
+             f"s_cselect_b32 {S_BLD}, {BEND - 0x8000:#x}, {S_BLD}", f"s_add_u32 {S_BLD}, {S_BLD}, %[woff]"]
+    later = [f"s_add_u32 {S_BN}, %[sb], 0x8000", f"s_cmp_eq_u32 {S_BN}, {BEND:#x}", f"s_cselect_b32 {S_BN}, {B0:#x}, {S_BN}",
+             f"s_xor_b32 {S_AN}, %[sa], 0x8000", f"v_add_u32 v{VT + 2}, %[sa], v{VADDR_A + 2}", f"v_add_u32 v{VT + 3}, %[sb], v{VADDR_B + 2}",
+             f"v_add_u32 v{VT + 4}, %[sa], v{VADDR_A + 3}", f"v_add_u32 v{VT + 5}, %[sb], v{VADDR_B + 3}", f"v_add_u32 v{VT + 6}, {S_AN}, v{VADDR_A}",
+             f"v_add_u32 v{VT + 7}, {S_BN}, v{VADDR_B}"]
+    if reduce == "fold":
+        later += ["s_mov_b32 s86, 0", "s_mov_b32 s87, -1"]
     for sub in range(4):
         slot, nslot = sub & 1, (sub & 1) ^ 1
         va, vb = (VT + 2 * sub, VT + 2 * sub + 1) if sub < 3 else (VT + 6, VT + 7)
@@ -234,6 +231,12 @@ def kstep(fresh, reduce=None):
             e(f"v_mfma_f32_32x32x16_bf16 {acc(i, j)}, {fa(slot, i)}, {fb(slot, j)}, {c}")
             if sub == 3 and n == 0:
                 e("s_barrier")
+            if sub == 0 and n == 0:
+                out.extend(early)
+            if sub == 0 and n >= 1:
+                for _ in range(3):
+                    if later:
+                        e(later.pop(0))
             if sub in (1, 2):
                 for _ in range(per_slot):
                     if fillers:
@@ -257,7 +260,7 @@ def kstep(fresh, reduce=None):
     e(f"s_mov_b32 %[sa], {S_AN}")
     e(f"s_mov_b32 %[sb], {S_BN}")
     e(f"s_mov_b32 m0, {S_M0}")
-    assert not fillers and not atomics
+    assert not fillers and not atomics and not later
     return fix_lane_move_hazards(out)
 
 

@@ -11,6 +11,7 @@
 #include <algorithm>
 #include <mutex>
 #include <type_traits>
+#include <vector>
 
 #include "gather_device.h"
 #include "route_internal.h"
@@ -1049,13 +1050,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerV
   // The workgroup's tiles: `cur` is multiplied, `nxt` is the one behind it (the loads enter it two K steps before the
   // MFMAs do).  Own tiles first, then pool draws.
   int tm_c, tn_c, tm_n = 0, tn_n = 0, own_idx = 0;
-  scan_walk_own(walk, 0, tm_c, tn_c);
+  ScanWalkCursor cursor = scan_walk_cursor(walk);
+  scan_walk_cursor_tile(walk, cursor, tm_c, tn_c);
   __amdgpu_buffer_rsrc_t ra_c = make_a(tm_c, true), rb_c = make_b(tn_c, true), ra_n, rb_n;
   bool nxt_valid = false, nxt_pending = false;
   auto plan_next = [&]() {
     nxt_valid = own_idx + 1 < walk.own_count;
     nxt_pending = !nxt_valid && pool_n > 0;
-    if (nxt_valid) scan_walk_own(walk, ++own_idx, tm_n, tn_n);
+    if (nxt_valid) {
+      ++own_idx;
+      scan_walk_cursor_next(walk, cursor);
+      scan_walk_cursor_tile(walk, cursor, tm_n, tn_n);
+    }
     ra_n = make_a(tm_n, nxt_valid);
     rb_n = make_b(tn_n, nxt_valid);
   };
@@ -1070,13 +1076,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kScan4CompilerV
   const int n_queries = M_rows / (blocks_per_query * 32);
   typedef const __attribute__((address_space(4))) uint32_t* const_words_t;      // scalar loads
   const const_words_t row_bits_c = (const_words_t)row_bits;
+  // floor(2^32 / d) + 1 divides exactly while n * d < 2^32 (row blocks < 2^19, blocks per query <= 2^11)
+  const uint32_t bpq_magic = (uint32_t)(0x100000000ull / (uint32_t)blocks_per_query) + 1u;
   uint32_t rbits[4] = {0u, 0u, 0u, 0u};
   int q_first = 0, r_first = 0;
   auto fetch_rows = [&](int m0) {
     const int blk0 = (m0 + wm * 128) >> 5;
 #pragma unroll
     for (int i = 0; i < 4; ++i) rbits[i] = row_bits_c[blk0 + i];          // 0 past M_rows (the buffer is padded)
-    q_first = blk0 / blocks_per_query;
+    q_first = blocks_per_query == 1 ? blk0 : (int)__umulhi((uint32_t)blk0, bpq_magic);     // blk0 / blocks_per_query
     r_first = blk0 - q_first * blocks_per_query;
   };
   // the documents of the wavefront's 128 columns, 64 per load, into v220 / v221 (v216: their offsets): requested in
@@ -1436,6 +1444,61 @@ RouteWorkspace route_workspace_layout(int32_t B, int32_t S, int32_t Hkv, int32_t
   w.off_sched = off;    off = align_up(off + kSchedBytes, 256);
   w.bytes = off;
   return w;
+}
+
+// Host-side replay of the large-tile scan's tile order (scan_walk.h): every scoring workgroup walks its own tiles
+// with the cursor the kernel uses, then the workgroups draw the pool's tiles in turn from one counter.
+extern "C" int msa_diag_scan_walk(int32_t tiles_m, int32_t tiles_n, int32_t grid, int32_t has_copy_workgroup,
+                                  int32_t pool_n, int32_t* visits) {
+  MSA_REQUIRE(visits != nullptr, "msa_diag_scan_walk: null output");
+  MSA_REQUIRE(tiles_m > 0 && tiles_n > 0 && grid >= 16 && grid <= kSchedMaxWorkgroups && pool_n >= 0 && pool_n <= tiles_n,
+              "msa_diag_scan_walk: tiles %d x %d, grid %d, pool %d out of range", tiles_m, tiles_n, grid, pool_n);
+  const int m_group = std::min(tiles_m, 8);
+  for (int64_t i = 0; i < (int64_t)tiles_m * tiles_n; ++i) visits[i] = 0;
+  const int scoring = grid - (has_copy_workgroup ? 1 : 0);
+  std::vector<int> draws;
+  for (int b = 0; b < scoring; ++b) {
+    const ScanWalk w = scan_walk_init(b, grid, has_copy_workgroup, tiles_m, tiles_n, m_group, pool_n);
+    if (w.own_count == 0) continue;
+    ScanWalkCursor c = scan_walk_cursor(w);
+    for (int idx = 0; idx < w.own_count; ++idx) {
+      int tm, tn, tm2, tn2;
+      scan_walk_cursor_tile(w, c, tm, tn);
+      scan_walk_own(w, idx, tm2, tn2);
+      if (tm != tm2 || tn != tn2 || tm < 0 || tm >= tiles_m || tn < 0 || tn >= tiles_n) {
+        msa_set_error("msa_diag_scan_walk: workgroup %d tile %d: cursor (%d, %d), closed form (%d, %d)", b, idx, tm, tn, tm2, tn2);
+        return MSA_ESTATE;
+      }
+      ++visits[(int64_t)tm * tiles_n + tn];
+      if (idx + 1 < w.own_count) scan_walk_cursor_next(w, c);
+    }
+    draws.push_back(b);
+  }
+  int counter = 0;
+  while (pool_n > 0 && !draws.empty()) {
+    std::vector<int> still;
+    for (int b : draws) {
+      const ScanWalk w = scan_walk_init(b, grid, has_copy_workgroup, tiles_m, tiles_n, m_group, pool_n);
+      const int p = counter++;
+      if (p >= w.pool_total) continue;
+      int tm, tn;
+      scan_walk_pool(w, p, tm, tn);
+      if (tm < 0 || tm >= tiles_m || tn < 0 || tn >= tiles_n) {
+        msa_set_error("msa_diag_scan_walk: pool position %d -> (%d, %d)", p, tm, tn);
+        return MSA_ESTATE;
+      }
+      ++visits[(int64_t)tm * tiles_n + tn];
+      still.push_back(b);
+    }
+    draws.swap(still);
+  }
+  return MSA_OK;
+}
+
+// The tile pool of the large-tile scan can be switched off (every tile then belongs to a fixed workgroup).
+extern "C" int msa_route_set_tile_pool(int32_t enabled) {
+  g_tile_pool_enabled.store(enabled ? 1 : 0, std::memory_order_relaxed);
+  return MSA_OK;
 }
 
 extern "C" int msa_profile_enable(int32_t max_records) {

@@ -66,3 +66,47 @@ MSA_WALK_FN void scan_walk_own(const ScanWalk& w, int idx, int& tm, int& tn) {
 MSA_WALK_FN void scan_walk_pool(const ScanWalk& w, int p, int& tm, int& tn) {
   scan_walk_decode(w.tiles_m, w.m_group, p, w.tiles_n - w.pool_n, w.pool_n, tm, tn);
 }
+
+// The workgroup's own tiles in order, without a division per tile: the cursor steps by the XCD's workgroup count
+// through the dense order, keeping (group of M tiles, N offset, M offset) and the step split into whole N tiles and a
+// remainder of M tiles; only a step that crosses into the next group of M tiles divides.
+struct ScanWalkCursor {
+  int g, mg, tn_off, tm_off, dq, dr;
+};
+
+MSA_WALK_FN int scan_walk_group_size(const ScanWalk& w, int g) {
+  const int full_groups = w.tiles_m / w.m_group;
+  return g < full_groups ? w.m_group : w.tiles_m - full_groups * w.m_group;
+}
+
+MSA_WALK_FN void scan_walk_cursor_place(const ScanWalk& w, ScanWalkCursor& c, int g, int rem) {
+  int mg = scan_walk_group_size(w, g);
+  while (mg > 0 && rem >= w.n_in_xcd * mg) {      // (past the last group the cursor is never read)
+    rem -= w.n_in_xcd * mg;
+    mg = scan_walk_group_size(w, ++g);
+  }
+  if (mg <= 0) mg = 1;
+  c.g = g; c.mg = mg;
+  c.tn_off = rem / mg; c.tm_off = rem % mg;
+  c.dq = w.wgs_in_xcd / mg; c.dr = w.wgs_in_xcd % mg;
+}
+
+// cursor on the workgroup's first own tile
+MSA_WALK_FN ScanWalkCursor scan_walk_cursor(const ScanWalk& w) {
+  ScanWalkCursor c;
+  scan_walk_cursor_place(w, c, 0, w.wg_in_xcd);
+  return c;
+}
+
+MSA_WALK_FN void scan_walk_cursor_tile(const ScanWalk& w, const ScanWalkCursor& c, int& tm, int& tn) {
+  tm = c.g * w.m_group + c.tm_off;
+  tn = w.n_begin + c.tn_off;
+}
+
+// on to the workgroup's next own tile (the caller counts them: own_count)
+MSA_WALK_FN void scan_walk_cursor_next(const ScanWalk& w, ScanWalkCursor& c) {
+  c.tm_off += c.dr;
+  c.tn_off += c.dq;
+  if (c.tm_off >= c.mg) { c.tm_off -= c.mg; ++c.tn_off; }
+  if (c.tn_off >= w.n_in_xcd) scan_walk_cursor_place(w, c, c.g + 1, (c.tn_off - w.n_in_xcd) * c.mg + c.tm_off);
+}

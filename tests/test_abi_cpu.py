@@ -74,3 +74,26 @@ def test_product_does_not_import_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 src = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in src.replace("ORACLE", ""), f"{f} mentions the oracle"
+
+
+@pytest.mark.parametrize("tiles_m,tiles_n,grid,copy_wg,pool_n", [
+    (8, 6271, 256, 1, 783), (8, 6271, 256, 0, 783), (8, 6271, 256, 1, 0),      # the 100M-token bank, B = 16 x 128
+    (16, 628, 256, 0, 78), (16, 628, 256, 1, 0),                                # the 10M-token bank, B = 32 x 128
+    (1, 40, 256, 0, 0), (2, 3, 16, 1, 0), (3, 100, 64, 1, 12), (11, 37, 256, 0, 4), (11, 37, 24, 1, 18),
+    (20, 999, 248, 1, 124), (256, 628, 256, 0, 78), (9, 5, 1024, 1, 0), (5, 1, 16, 0, 0), (7, 200, 16, 1, 25),
+])
+def test_scan_tile_order_covers_every_tile_once(tiles_m, tiles_n, grid, copy_wg, pool_n):
+    """The persistent scan's tile order (fixed shares per XCD walked by an incremental cursor, then the pool):
+    every tile exactly once, for grids with and without the copying workgroup and with and without a pool."""
+    lib = _lib.load()
+    visits = (C.c_int32 * (tiles_m * tiles_n))()
+    rc = lib.msa_diag_scan_walk(tiles_m, tiles_n, grid, copy_wg, pool_n, C.addressof(visits))
+    assert rc == 0, lib.msa_last_error()
+    v = list(visits)
+    assert min(v) == 1 and max(v) == 1, f"{v.count(0)} tiles unvisited, {sum(1 for x in v if x > 1)} visited twice"
+
+
+def test_tile_pool_switch_is_exported():
+    lib = _lib.load()
+    assert lib.msa_route_set_tile_pool(0) == 0
+    assert lib.msa_route_set_tile_pool(1) == 0

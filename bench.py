@@ -53,6 +53,21 @@ def measured_traffic(kernel: str, workload: str):
     return None
 
 
+def traffic_source(kernel: str, workload: str):
+    """Where measured_traffic()'s figure comes from: the committed profile summary (an earlier rocprofv3 --pmc run,
+    not this run) that holds the matching TRAFFIC line, or None."""
+    try:
+        names = sorted(os.listdir(PROFILES))
+    except OSError:
+        return None
+    for name in names:
+        if name.endswith((".txt", ".md")):
+            for line in open(os.path.join(PROFILES, name), errors="replace"):
+                if line.startswith("TRAFFIC ") and f"kernel={kernel} " in line and f"workload={workload} " in line:
+                    return f"profiles/{name} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of an earlier run, scaled by a plain copy)"
+    return None
+
+
 def cpu_model() -> str:
     try:
         for line in open("/proc/cpuinfo"):
@@ -100,11 +115,9 @@ def plant_needles(kr, q, doc_chunk_off, n_docs, seed):
     g = np.random.default_rng(seed)
     want = np.zeros((B, TOPK), dtype=np.int64)
     used = set()
+    toks, cs = [], []
     for b in range(B):
-        tok = int(g.integers(0, S))
-        qt = q[b, tok].float()
-        qn = (qt / qt.norm(dim=-1, keepdim=True)).view(HKV, HQ // HKV, D).sum(1)
-        direction = qn / qn.norm(dim=-1, keepdim=True)
+        toks.append(int(g.integers(0, S)))
         docs = []
         while len(docs) < TOPK:
             d = int(g.integers(0, n_docs))
@@ -112,13 +125,19 @@ def plant_needles(kr, q, doc_chunk_off, n_docs, seed):
                 used.add(d)
                 docs.append(d)
         for r, d in enumerate(docs):
-            c = (int(doc_chunk_off[d]) + int(doc_chunk_off[d + 1])) // 2
-            cos = 0.98 - 0.025 * r
-            noise = kr[c].float()
-            perp = noise - (noise * direction).sum(-1, keepdim=True) * direction
-            perp = perp / perp.norm(dim=-1, keepdim=True)
-            kr[c] = (cos * direction + (1 - cos * cos) ** 0.5 * perp).to(torch.bfloat16)
+            cs.append((int(doc_chunk_off[d]) + int(doc_chunk_off[d + 1])) // 2)
             want[b, r] = d
+    # all B * TOPK chunks in one batch of device operations (the planted chunks are distinct)
+    dev = kr.device
+    qt = q[torch.arange(B, device=dev), torch.tensor(toks, device=dev)].float()                 # [B, HQ, D]
+    qn = (qt / qt.norm(dim=-1, keepdim=True)).view(B, HKV, HQ // HKV, D).sum(2)
+    direction = (qn / qn.norm(dim=-1, keepdim=True)).repeat_interleave(TOPK, dim=0)           # [B * TOPK, HKV, D]
+    cos = (0.98 - 0.025 * torch.arange(TOPK, device=dev, dtype=torch.float32)).repeat(B).view(-1, 1, 1)
+    idx = torch.tensor(cs, device=dev)
+    noise = kr[idx].float()
+    perp = noise - (noise * direction).sum(-1, keepdim=True) * direction
+    perp = perp / perp.norm(dim=-1, keepdim=True)
+    kr[idx] = (cos * direction + (1 - cos * cos).sqrt() * perp).to(torch.bfloat16)
     return want
 
 
@@ -344,8 +363,10 @@ def main():
     ap.add_argument("--layers", type=int, default=18, help="routed layers resident in HBM")
     ap.add_argument("--batch", type=int, default=16)
     ap.add_argument("--seq", type=int, default=128)
-    ap.add_argument("--host-kv-layers", type=int, default=2,
-                    help="distinct pinned host K/V layer buffers (routed layers share them round-robin)")
+    ap.add_argument("--host-kv-layers", type=int, default=0,
+                    help="distinct pinned host K/V layer buffers (routed layers share them round-robin); 0: as many as "
+                         "the box pins, up to 8 (the boxes of this pool refuse pinned memory past about 56 GB, i.e. the "
+                         "17th 3.3 GB buffer at the 100M-token bank)")
     ap.add_argument("--gather", choices=["device", "fused", "memcpy"], default="fused",
                     help="device: plan + copy kernels read the pinned bank directly, no ids on the host; "
                          "fused: the same plan + copy inside the next layer's scan launch (one workgroup of it); "
@@ -385,21 +406,39 @@ def main():
         f"{C_total * HKV * D * 2 * L / 1e9:.1f} GB of K_r")
     bank = ops.Bank(L, doc_chunk_off.tolist(), list(range(n_docs)), HKV, D, torch.bfloat16)
 
-    # pinned host K / V: a few distinct layer buffers, filled from the device
-    n_host = max(1, min(args.host_kv_layers, L))
-    host_k, host_v = [], []
+    # Pinned host K / V: distinct layer buffers, filled from the device.  The configuration names pinned K / V for
+    # every routed layer; this pool's boxes refuse pinned allocations past about 56 GB, so the bench takes as many
+    # layer buffers as the box pins (each K + V pair is allocated before it counts; one buffer of head room is kept
+    # below the point of refusal), up to 8 by default, and the routed layers share them round-robin.
+    auto = args.host_kv_layers <= 0
+    n_want = max(1, min(8 if auto else args.host_kv_layers, L))
+    buf_gb = C_total * HKV * D * 2 / 1e9
+    host_k, host_v, refused_at_gb = [], [], None
+    for i in range(n_want):
+        try:
+            pair = [torch.empty((C_total, HKV, D), dtype=torch.bfloat16, pin_memory=True) for _ in range(2)]
+        except RuntimeError as e:
+            refused_at_gb = round((2 * len(host_k) + 1) * buf_gb, 1)
+            log(f"host K/V: pinned allocation refused at about {refused_at_gb} GB ({str(e).splitlines()[0][:80]})")
+            pair = None
+            if len(host_k) > 1:           # head room: give the last pair back
+                host_k.pop(); host_v.pop()
+            break
+        host_k.append(pair[0]); host_v.append(pair[1])
+    if not host_k:
+        sys.exit("bench.py: could not pin one layer of host K / V")
+    n_host = len(host_k)
     for i in range(n_host):
-        for dst, seed in ((host_k, 1000 + i), (host_v, 2000 + i)):
-            h = torch.empty((C_total, HKV, D), dtype=torch.bfloat16, pin_memory=True)
+        for h, seed in ((host_k[i], 1000 + i), (host_v[i], 2000 + i)):
             g = torch.Generator(device=dev).manual_seed(seed)
             step = 1 << 18
-            for s in range(0, C_total, step):
-                e = min(C_total, s + step)
-                h[s:e].copy_(torch.randn((e - s, HKV, D), generator=g, device=dev).to(torch.bfloat16))
-            dst.append(h)
+            for s0 in range(0, C_total, step):
+                e0 = min(C_total, s0 + step)
+                h[s0:e0].copy_(torch.randn((e0 - s0, HKV, D), generator=g, device=dev).to(torch.bfloat16))
         if n_host > 2:
             log(f"host K/V: layer buffer {i + 1} of {n_host} filled")
-    log(f"host K/V: {n_host} layer buffer(s), {2 * n_host * C_total * HKV * D * 2 / 1e9:.1f} GB pinned")
+    pinned_gb = round(2 * n_host * buf_gb, 1)
+    log(f"host K/V: {n_host} layer buffer(s), {pinned_gb} GB pinned")
 
     qs, wants, krs = [], [], []
     gq = torch.Generator(device=dev).manual_seed(7)
@@ -557,8 +596,10 @@ def main():
         gbs = bytes_layer / (kern_ms * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None}
-    roof["traffic"] = measured_traffic("score_gemm_kernel", f"tokens={args.tokens},B={B},S={S}")
-    roof.update({"kernel": "score_gemm_kernel", "kernel_ms": round(kern_ms, 4), "launches_timed": n_rec.value,
+    scan_kernel = "score_scan4_kernel" if B * ((S + 31) // 32 * 32) > 128 else "score_gemm_kernel"
+    roof["traffic"] = measured_traffic(scan_kernel, f"tokens={args.tokens},B={B},S={S}")
+    roof["traffic_source"] = traffic_source(scan_kernel, f"tokens={args.tokens},B={B},S={S}")
+    roof.update({"kernel": scan_kernel, "kernel_ms": round(kern_ms, 4), "launches_timed": n_rec.value,
                  "flops_per_launch": flops, "algorithmic_bytes_per_launch": bytes_layer,
                  "hbm_gbs_at_this_batch": round(bytes_layer / (kern_ms * 1e-3) / 1e9, 1)})
 
@@ -598,7 +639,10 @@ def main():
             sweep.append({"B": b1, "S": s1, "call_ms": round(call_ms, 4), "GB/s": round(by / call_ms / 1e6, 1),
                           "frac_hbm": round(by / call_ms / 1e6 / HBM_PEAK_GBS, 4), "scan_kernel_ms": round(ms1, 4),
                           "scan_kernel_frac_hbm": round(by / ms1 / 1e6 / HBM_PEAK_GBS, 4), "algorithmic_bytes": by,
-                          "traffic": measured_traffic("score_gemm_kernel", f"tokens={args.tokens},B={b1},S={s1}")})
+                          "scan_TFLOP/s": round(2.0 * b1 * ((s1 + 31) // 32 * 32) * HKV * D * C_total / ms1 / 1e9, 1),
+                          "scan_kernel": "score_scan4_kernel" if b1 * ((s1 + 31) // 32 * 32) > 128 else "score_gemm_kernel",
+                          "traffic": measured_traffic("score_scan4_kernel" if b1 * ((s1 + 31) // 32 * 32) > 128 else "score_gemm_kernel",
+                                                      f"tokens={args.tokens},B={b1},S={s1}")})
         _lib.check(lib.msa_profile_enable(0), "msa_profile_enable")
     if args.sweep_only:
         print(json.dumps({"hbm_regime_sweep": sweep}), flush=True)
@@ -639,7 +683,10 @@ def main():
         "config": {"workload": "configs[3]: 100M-token bank, K_r HBM-resident, K/V pinned host, B=16 x S=128, top-16",
                    "bank_tokens": args.tokens, "chunks": C_total, "docs": n_docs, "routed_layers": L, "batch": B,
                    "query_tokens": S, "top_k": TOPK, "kr_hbm_gb": round(C_total * HKV * D * 2 * L / 1e9, 1),
-                   "host_kv_layer_buffers": n_host, "gather": args.gather,
+                   "host_kv_layer_buffers": n_host, "host_kv_pinned_gb": pinned_gb, "pinned_refused_at_gb": refused_at_gb,
+                   "host_kv_note": "fewer layer buffers than routed layers: the box refuses pinned host memory past "
+                                   "about 56 GB; the routed layers share the buffers round-robin" if n_host < L else None,
+                   "gather": args.gather,
                    "gather_host_ms_per_layer": {k: round(v / (args.steps * L) * 1e3, 3) for k, v in host_s.items()}, "selected_chunks_per_layer": int(np.mean(sel_chunks)),
                    "mode": "cosine/mean-heads/max-tokens/max-chunks"},
         "roofline": roof, "cpu_baseline": cpu, "hbm_regime_sweep": sweep, "other_kernels": extras, "parity": "needles exact on all layers",

@@ -160,22 +160,10 @@ struct Mma<float> {
   }
 };
 
-// The MFMA-bound form (bf16, 256 x 256, one workgroup per compute unit) stages its operand tiles with buffer loads that write
-// LDS directly: no staging registers, no ds_write, and room for a third stage of the operand that comes from HBM.
-// LDS then holds two stages of the query tile (2 x 32 KB) and three of the K_r tile (3 x 32 KB), 160 KB in all, in
-// un-padded 128-byte rows whose 16-byte units are XOR-swizzled by (row >> 1) & 7 (conflict-free operand reads; a
-// direct load cannot pad, its 64 lanes fill 1 KB of LDS in lane order, so the swizzle is applied to the global
-// address each lane fetches).  K_r tile kt + 2 and query tile kt + 1 are requested at the start of step kt; the wait in
-// front of the step's barrier leaves the newest K_r tile in flight.  7.5 % faster than the register-staged form in a
-// stand-alone copy of the loop (1312-1320 against 1218-1229 TFLOP/s).
-constexpr int kDtlStageBytes = 256 * 128;
-constexpr int kDtlLdsBytes = 5 * kDtlStageBytes;
-template <typename T, int BM, int BN, int kSets, bool kStream>
-constexpr bool score_tile_is_direct() {
-  return sizeof(T) == 2 && BM == 256 && BN == 256 && kSets == 1 && !kStream;
-}
-
-// The HBM-bound form for up to 128 query rows (bf16, 128 x 256, streaming over N tiles) uses the same loads with three
+// The HBM-bound form for up to 128 query rows (bf16, 128 x 256, streaming over N tiles) stages its operand tiles with
+// buffer loads that write LDS directly (no staging registers, no ds_write; un-padded 128-byte rows whose 16-byte units
+// are XOR-swizzled by (row >> 1) & 7: a direct load cannot pad, its 64 lanes fill 1 KB of LDS in lane order, so the
+// swizzle is applied to the global address each lane fetches), three
 // stages of each operand (3 x 16 KB + 3 x 32 KB = 144 KB): both operands are requested two K steps ahead, which keeps
 // 96 KB per compute unit in flight (returns are in order, so the query tile has to run as far ahead as the K_r tile for
 // the K_r tile's lead to count).
@@ -194,17 +182,17 @@ constexpr bool score_tile_is_direct_stream() {
 // kStream: one workgroup per compute-unit slot walks N tiles blockIdx.x, blockIdx.x + gridDim.x, ... (one M tile
 // only) with the load / store / multiply pipeline running across tile boundaries: the first K tiles of the next N
 // tile are already in flight while the last ones of the current tile are multiplied and its epilogue runs, so the
-// HBM stream never drains between tiles.  That is what the HBM-bound shapes need; the MFMA-bound ones keep one
-// workgroup per tile, which leaves compute units free for kernels of other streams.
+// HBM stream never drains between tiles.  That is what the HBM-bound shapes need; the fp32 form keeps one
+// workgroup per tile.
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool kDocMax, bool kStream>
-__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vgpr(251))) void score_gemm_kernel(
+__global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     const T* __restrict__ qs,            // [M_rows, K]  pre-summed queries, M_rows = B * S_pad
     const T* __restrict__ kr,            // [C, K]
     const uint32_t* __restrict__ row_bits,  // [ceil(M_alloc / 32)] scored-row bitmask
     uint32_t* __restrict__ out_key,      // [B, n_docs] or [B, C], zeroed
     const int32_t* __restrict__ chunk_doc,  // [C] document of every chunk (kDocMax)
     int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t tiles_m, int32_t tiles_n,
-    int32_t m_group, int32_t n_docs, GatherJob job, uint32_t* __restrict__ sched, int32_t pool_n) {
+    int32_t m_group, int32_t n_docs) {
   constexpr int kThreads = WAVES_M * WAVES_N * 64;
   constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;
   constexpr int TM = WM / 32, TN = WN / 32;
@@ -213,7 +201,6 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vg
 
   extern __shared__ __align__(16) char lds[];
   constexpr int kBufBytes = (BM + BN) * kRowStride;   // [A tile | B tile] per buffer, two buffers
-  constexpr bool kDtl = score_tile_is_direct<T, BM, BN, kSets, kStream>();
   constexpr bool kDtlStream = score_tile_is_direct_stream<T, BM, BN, kSets, kStream>();
 
   // XCD-aware tile order: workgroups are dealt round-robin to the 8 XCDs, so each XCD gets one
@@ -233,59 +220,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vg
     tm = (within / per_group) * m_group + rem % m_group;
     return tn < tiles_n && tm < tiles_m;
   };
-  // The direct-to-LDS form is persistent: the workgroups of an XCD share the XCD's tiles, position p of its dense
-  // order naming (group of M tiles by group) an N tile of the XCD's range with the group's M tiles side by side;
-  // workgroup w of the XCD takes positions w, w + (workgroups of the XCD), ...  With a gather job attached the last
-  // workgroup of the launch does not score: it fetches the K / V rows of an earlier selection from the pinned host bank
-  // while the others scan (a copy on a compute unit of its own disturbs no scoring workgroup, and no scoring
-  // workgroup's share of tiles depends on where a separate copy kernel's wavefronts would have landed).  The XCDs'
-  // N ranges are sized in proportion to their scoring workgroups.
-  const int xcd = blockIdx.x % 8, wg_in_xcd = blockIdx.x / 8;
-  const int wgs_all = (int)gridDim.x, scoring_wgs = wgs_all - (job.active ? 1 : 0);
-  const bool is_copy_wg = kDtl && job.active && (int)blockIdx.x == wgs_all - 1;
-  auto wgs_before = [&](int x) {      // scoring workgroups on XCDs 0 .. x - 1 (workgroup b sits on XCD b % 8)
-    int n = 0;
-    for (int y = 0; y < x; ++y) n += (scoring_wgs - y + 7) / 8;
-    return n;
-  };
-  const int wgs_in_xcd = (scoring_wgs - xcd + 7) / 8;
-  // the last pool_n N tiles belong to no XCD: they are the pool every workgroup draws from when its share is done
-  const int tiles_n_own = tiles_n - pool_n;
-  const int n_begin = (int)((int64_t)tiles_n_own * wgs_before(xcd) / max(scoring_wgs, 1));
-  const int n_stop = (int)((int64_t)tiles_n_own * (wgs_before(xcd) + wgs_in_xcd) / max(scoring_wgs, 1));
-  const int n_in_xcd = n_stop - n_begin;
-  const int dense_total = n_in_xcd * tiles_m, pool_total = pool_n * tiles_m;
-  // position p of the dense order over n_in N tiles from nb on (group of M tiles by group, a group's M tiles adjacent)
-  auto decode_range = [&](int p, int nb, int n_in, int& tm, int& tn) {
-    const int full_groups = tiles_m / m_group, full = full_groups * n_in * m_group;
-    int g, rem, mg;
-    if (p < full) { g = p / (n_in * m_group); rem = p - g * n_in * m_group; mg = m_group; }
-    else { g = full_groups; rem = p - full; mg = tiles_m - full_groups * m_group; }
-    tn = nb + rem / mg;
-    tm = g * m_group + rem % mg;
-  };
-  auto decode_dense = [&](int p, int& tm, int& tn) { decode_range(p, n_begin, n_in_xcd, tm, tn); };
-  if constexpr (kDtl) {
-    if (is_copy_wg) {
-      // plan (sorted, de-duplicated selection -> copy entries), host rows, then the documents an earlier sample
-      // already fetched; the workgroup barriers order the three steps' memory
-      msa_gather::plan_body(job.doc_sel, job.doc_chunk_off, job.n_docs, job.B, job.k,
-                            (int32_t)min(job.capacity_rows, (int64_t)0x7fffffff), job.dedup,
-                            job.cu_sel, job.plan, reinterpret_cast<int32_t*>(lds), (int)threadIdx.x, kThreads);
-      __syncthreads();
-      const int groups = kThreads / msa_gather::kCopyRowLanes;
-      const int group = (int)threadIdx.x / msa_gather::kCopyRowLanes, lane_in_row = (int)threadIdx.x % msa_gather::kCopyRowLanes;
-      msa_gather::copy_body<false, 8>(job.k_src, job.v_src, job.plan, job.B * job.k, job.row_vecs, job.capacity_rows,
-                                   job.k_dst, job.v_dst, 0, 1, group, groups, lane_in_row);
-      __syncthreads();
-      if (job.dedup)
-        msa_gather::copy_body<true, 8>(nullptr, nullptr, job.plan, job.B * job.k, job.row_vecs, job.capacity_rows,
-                                    job.k_dst, job.v_dst, 0, 1, group, groups, lane_in_row);
-      return;
-    }
-    if (wg_in_xcd >= dense_total) return;
-    decode_dense(wg_in_xcd, tile_m, tile_n);
-  } else if constexpr (!kStream) {
+  if constexpr (!kStream) {
     if (!decode_tile(blockIdx.x, tile_m, tile_n)) return;
   }
   if (tile_n >= tiles_n || tile_m >= tiles_m) return;
@@ -430,39 +365,10 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vg
     }
   };
 
-  // ---- direct-to-LDS form (see score_tile_is_direct) ----
-  // A wavefront's load instruction i covers rows (wave * 4 + i) * 8 .. + 8 of the operand tile: lane l lands in LDS at
-  // byte 16 * l of that 1 KB block, i.e. row l / 8, unit slot l % 8, and fetches the unit that belongs there.
+  // ---- direct-to-LDS form (see score_tile_is_direct_stream) ----
+  // A wavefront's load instruction covers 8 rows of the operand tile: lane l lands in LDS at byte 16 * l of that 1 KB
+  // block, i.e. row l / 8, unit slot l % 8, and fetches the unit that belongs there.
   const int dtl_row = (lane >> 3), dtl_slot = lane & 7;
-  auto dtl_voff = [&](int i) {
-    const int row = (wave * 4 + i) * 8 + dtl_row;
-    return row * (int)row_bytes_g + ((dtl_slot ^ ((row >> 1) & 7)) * 16);
-  };
-  __amdgpu_buffer_rsrc_t rsrc_la = rsrc_a;      // direct-to-LDS form: the query tile the loads have reached (K_r: rsrc_ld)
-  auto dtl_load_a = [&](int stage, int kt) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      MSA_LOAD_TO_LDS(rsrc_la, lds + stage * kDtlStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes, 0);
-  };
-  auto dtl_load_b = [&](int stage, int kt) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      MSA_LOAD_TO_LDS(rsrc_ld, lds + (2 + stage) * kDtlStageBytes + (wave * 4 + i) * 1024, dtl_voff(i), kt * kRowBytes,
-                      kStreamHint);
-  };
-  auto dtl_frags = [&](int sa, int sb, int sub, int slot) {
-    const int unit = sub * 2 + half;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-      const int row = wm * WM + i * 32 + l32;
-      fa[slot][i] = *reinterpret_cast<const Frag*>(lds + sa * kDtlStageBytes + row * 128 + ((unit ^ ((row >> 1) & 7)) * 16));
-    }
-#pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int row = wn * WN + j * 32 + l32;
-      fb[slot][j] = *reinterpret_cast<const Frag*>(lds + (2 + sb) * kDtlStageBytes + row * 128 + ((unit ^ ((row >> 1) & 7)) * 16));
-    }
-  };
 
   // Epilogue of the N tile starting at chunk `tile_n0`.  acc[i][j][e] is row 8*(e/4) + 4*half + e%4, column l32 of
   // its 32x32 block.  Consecutive row blocks of one query are folded into `run` (each half of the wavefront over its
@@ -580,176 +486,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) __attribute__((amdgpu_num_vg
     emit(run_q, tile_n0, run, any);
   };
 
-  if constexpr (kDtl) {
-    static_assert(kThreads == 512 && kSub == 4, "the direct-to-LDS form is laid out for 8 wavefronts of bf16");
-    // vmcnt(4) / vmcnt(0) with the other counters left alone: the four newest loads are the K_r tile two steps ahead
-    constexpr int kWaitAllButNewestB = 0x0F74, kWaitAll = 0x0F70;
-    // The workgroup barrier of this form is written out: __syncthreads() carries a release fence, for which the
-    // compiler drains every outstanding load that writes LDS (vmcnt(0)), the K_r tile two steps ahead included, which
-    // is exactly the wait the third stage exists to avoid.  The explicit vmcnt wait in front of it covers the tiles
-    // the next step reads; the LDS reads of this step are drained by lgkmcnt(0).
-    auto dtl_barrier = [&]() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
-    // Persistent: the workgroup's tiles form one sequence of K steps.  The query loads run one step ahead of the MFMAs
-    // and the K_r loads two, across tile boundaries, so a tile's first operands are in LDS before the previous tile's
-    // epilogue starts and the compute unit does not idle while a tile ramps up.  Each of the three positions (K_r
-    // loads, query loads, MFMAs) steps through the same tile list; a position that reaches a tile end takes over the
-    // tile of the position ahead of it (the K_r loads decode the list).
-    int tm_b = tile_m, tn_b = tile_n, p_b = wg_in_xcd, kt_b = 0;   // K_r loads
-    int tm_a = tile_m, tn_a = tile_n, kt_a = 0;                    // query loads
-    bool valid_a = true, valid_b = true;
-    // Once the workgroup's own share is done it draws tiles from the pool.  During the first steps of the tile in front
-    // of a pool tile one lane draws the position (an atomic that returns), publishes it (an exchange that returns, so
-    // its arrival says the word is in L2) and every wavefront reads it back: one hop per K step, issued in front of the
-    // step's tile loads, so the waits that already close the step (all but the newest K_r loads) cover it and no
-    // wavefront waits for the hand-out itself.  The position is in use from step 3; the K_r loads leave the tile three
-    // steps before its end, hence at least 6 K tiles per tile (the host offers no pool otherwise).
-    // The three hops keep their operands in v251 - v254, above the registers the compiler may allocate in this kernel
-    // (amdgpu_num_vgpr on its declaration): a value on its way back from memory must not sit in a register the
-    // compiler may copy or reuse before the step's wait has passed, and the compiler, which does not see these
-    // instructions' results, adds no waits of its own for them.  Each memory instruction sits behind five wait states:
-    // its address registers may have been written by a lane read just in front of the statement (a restored spill),
-    // and the hazard between the two is not resolved inside an asm statement.
-    int own_left = (dense_total - wg_in_xcd + wgs_in_xcd - 1) / wgs_in_xcd - 1;   // own tiles behind the K_r loads' one
-    uint32_t* const pool_counter = sched;
-    uint32_t* const my_claim = sched + kSchedCounterWords + blockIdx.x;
-    const bool drawer = __builtin_amdgcn_readfirstlane(tid >> 6) == 0;
-    int p_next = 0;
-    const uint32_t zero_off = 0;
-#if defined(__HIP_DEVICE_COMPILE__)
-    asm volatile("v_mov_b32 v253, 1" ::: "v251", "v252", "v253", "v254");
-#endif
-    auto set_rsrc_b = [&]() {
-      rsrc_ld = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(gb) + (int64_t)tn_b * BN * row_bytes_g, 0,
-                                                  (int)(min(BN, C - tn_b * BN) * row_bytes_g), 0x00020000);
-    };
-    auto set_rsrc_a = [&]() {
-      rsrc_la = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(ga) + (int64_t)tm_a * BM * row_bytes_g, 0,
-                                                  (int)(min(BM, M_rows - tm_a * BM) * row_bytes_g), 0x00020000);
-    };
-    auto advance_b = [&]() {
-      if (++kt_b == k_tiles) {
-        kt_b = 0;
-        if (own_left > 0) {
-          --own_left;
-          p_b += wgs_in_xcd;
-          decode_dense(p_b, tm_b, tn_b);
-          set_rsrc_b();
-        } else {
-          valid_b = p_next < pool_total;            // (no pool: 0 < 0 ends the walk)
-          if (valid_b) {
-            decode_range(p_next, tiles_n_own, pool_n, tm_b, tn_b);
-            set_rsrc_b();
-          }
-        }
-      }
-    };
-    auto advance_a = [&]() {      // the K_r position is ahead by one step, so at a tile end it already names the next tile
-      if (++kt_a == k_tiles) {
-        kt_a = 0;
-        tm_a = tm_b; tn_a = tn_b;
-        valid_a = valid_b;                   // (at least two K tiles per tile: the K_r position is still in that tile)
-        if (valid_a) set_rsrc_a();
-      }
-    };
-    dtl_load_a(0, 0);
-    advance_a();
-    dtl_load_b(0, 0);
-    advance_b();
-    if (valid_b) {
-      dtl_load_b(1, kt_b);
-      advance_b();
-      __builtin_amdgcn_s_waitcnt(kWaitAllButNewestB);
-    } else {
-      __builtin_amdgcn_s_waitcnt(kWaitAll);
-    }
-    dtl_barrier();
-    dtl_frags(0, 0, 0, 0);
-    fetch_rows();
-    fetch_docs(n0);
-    // (the prefetches of a tile are issued before the tile loads of its first step: the waits, which count from the
-    // newest load, cover them)
-    int sa = 0, sb = 0, kt = 0;
-    for (;;) {
-      const int sb1 = sb == 2 ? 0 : sb + 1, sb2 = sb1 == 2 ? 0 : sb1 + 1;
-      const bool more = valid_a, more2 = valid_b;    // a next step exists / its successor exists
-#if defined(__HIP_DEVICE_COMPILE__)
-      if (pool_n > 0 && own_left == 0 && more2 && kt < 4) {      // the tile behind this one comes from the pool
-        if (kt == 0) {
-          if (drawer && lane == 0)       // v252 = counter++ (back before this step's closing wait returns)
-            asm volatile("s_nop 4\n\tglobal_atomic_add v252, %0, v253, %1 sc0" ::"v"(zero_off), "s"(pool_counter) : "v252", "v254", "memory");
-        } else if (kt == 1) {
-          if (drawer && lane == 0)       // word = v252; its old value comes back in v254, which tells the word is in L2
-            asm volatile("s_nop 4\n\tglobal_atomic_swap v254, %0, v252, %1 sc0" ::"v"(zero_off), "s"(my_claim) : "v254", "memory");
-        } else if (kt == 2) {            // every wavefront reads the word back (past the L1: device scope)
-          asm volatile("s_nop 4\n\tglobal_load_dword v251, %0, %1 sc1" ::"v"(zero_off), "s"(my_claim) : "v251", "memory");
-        } else {                         // complete since step 2's closing wait
-          asm volatile("v_readfirstlane_b32 %0, v251" : "=s"(p_next));
-        }
-      }
-#endif
-      if (more) {
-        dtl_load_a(sa ^ 1, kt_a);      // stage of the step before this one: its last reads were behind the previous barrier
-        advance_a();
-      }
-      if (more2) {
-        dtl_load_b(sb2, kt_b);
-        advance_b();
-      }
-      // One sub-step: the operand reads of the next one, then this one's MFMAs.  A tile's first sub-step multiplies
-      // into zero (the constant operand of the instruction) instead of into accumulators cleared beforehand: 128
-      // register moves per wavefront and tile that nothing could overlap, since the first MFMAs wait for them.
-      auto substep = [&](auto sub_tag, auto fresh_tag) {
-        constexpr int sub = decltype(sub_tag)::value;
-        constexpr bool fresh = decltype(fresh_tag)::value;
-        if constexpr (sub + 1 < kSub) {
-          dtl_frags(sa, sb, sub + 1, (sub + 1) & 1);
-        } else {
-          if (more) {
-            if (more2) __builtin_amdgcn_s_waitcnt(kWaitAllButNewestB);
-            else __builtin_amdgcn_s_waitcnt(kWaitAll);
-            dtl_barrier();
-            dtl_frags(sa ^ 1, sb1, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-          }
-        }
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-          for (int j = 0; j < TN; ++j) {
-            if constexpr (fresh) acc[i][j] = Mma<T>::mma(fa[sub & 1][i], fb[sub & 1][j], floatx16_t{});
-            else acc[i][j] = Mma<T>::mma(fa[sub & 1][i], fb[sub & 1][j], acc[i][j]);
-          }
-        if constexpr (sub + 1 < kSub) {
-          // issue order of the sub-step: each of the six operand reads of the next sub-step behind one MFMA of this
-          // one, the last two MFMAs behind them (2.5 % faster than the order the scheduler picks by itself)
-#pragma unroll
-          for (int g = 0; g < 6; ++g) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one MFMA
-            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
-          }
-          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
-        }
-      };
-      if (kt == 0) substep(std::integral_constant<int, 0>{}, std::true_type{});
-      else substep(std::integral_constant<int, 0>{}, std::false_type{});
-      substep(std::integral_constant<int, 1>{}, std::false_type{});
-      substep(std::integral_constant<int, 2>{}, std::false_type{});
-      substep(std::integral_constant<int, 3>{}, std::false_type{});
-      sa ^= 1;
-      sb = sb1;
-      if (++kt == k_tiles) {
-        epilogue(n0);
-        if (!more) break;
-        kt = 0;
-        tile_m = tm_a;      // the query loads entered the next tile during this tile's last step
-        tile_n = tn_a;
-        m0 = tile_m * BM;
-        n0 = tile_n * BN;
-        fetch_rows();
-        fetch_docs(n0);
-      }
-    }
-  } else if constexpr (kDtlStream) {
+  if constexpr (kDtlStream) {  } else if constexpr (kDtlStream) {
     static_assert(kThreads == 512 && kSub == 4 && TM == 2 && TN == 2, "laid out for 8 wavefronts of 64 x 64");
     constexpr int kAStage = BM * 128, kBStage = BN * 128, kStages = 3;
     constexpr int kALoads = BM / 64, kBLoads = BN / 64;      // 1 KB blocks (8 rows) per wavefront and stage
@@ -1292,11 +1029,9 @@ int compute_units() {
 
 template <typename T, int BM, int BN, int WAVES_M, int WAVES_N, int kSets, bool kDocMax, bool kStream>
 int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key, const int32_t* chunk_doc,
-                int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t n_docs, hipStream_t st,
-                const GatherJob* job, bool* job_taken, uint32_t* sched) {
-  const size_t lds = score_tile_is_direct<T, BM, BN, kSets, kStream>()          ? (size_t)kDtlLdsBytes
-                     : score_tile_is_direct_stream<T, BM, BN, kSets, kStream>() ? (size_t)kDtlStreamLdsBytes
-                                                                                 : (size_t)2 * (BM + BN) * kRowStride;
+                int32_t M_rows, int32_t C, int32_t K, int32_t blocks_per_query, int32_t n_docs, hipStream_t st) {
+  const size_t lds = score_tile_is_direct_stream<T, BM, BN, kSets, kStream>() ? (size_t)kDtlStreamLdsBytes
+                                                                               : (size_t)2 * (BM + BN) * kRowStride;
   const int tiles_m = (M_rows + BM - 1) / BM;
   const int tiles_n = (C + BN - 1) / BN;
   // M tiles are walked in groups of 8 per K_r tile: a group's query rows (4 MiB in bf16) are what an XCD's L2
@@ -1312,28 +1047,6 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
     }
     grid = std::min(tiles_n, compute_units() * std::max<int>(1, (int)(kLdsPerCu / lds)));
   }
-  GatherJob no_job{};
-  int pool_n = 0;
-  const GatherJob* the_job = &no_job;
-  if (score_tile_is_direct<T, BM, BN, kSets, kStream>()) {
-    // persistent: one workgroup per compute unit walks its XCD's tiles; with a gather job the last one copies instead.
-    // The loop needs at least two K tiles per tile.
-    if (K * (int)sizeof(T) < 2 * kRowBytes) {
-      msa_set_error("score_gemm: K=%d too small for the direct-to-LDS form", K);
-      return MSA_EINVAL;
-    }
-    grid = std::min(kSchedMaxWorkgroups, std::max(16, compute_units() / 8 * 8));
-    // The XCDs do not run at one speed (their ends lay up to 6 % apart with fixed ranges, in an order that changes from
-    // launch to launch): the last eighth of the N tiles is a pool the workgroups draw from one tile at a time once
-    // their own share is done (a sixth to a twenty-fourth measured alike at 196 tiles per workgroup, the larger pools
-    // slightly better at 39).  Worth it when a workgroup has tiles enough for the pool to even the ends out, and
-    // possible when a tile is deep enough for a draw to come back in time.
-    if ((int64_t)tiles_m * tiles_n >= (int64_t)16 * grid && K * (int)sizeof(T) >= 6 * kRowBytes) pool_n = tiles_n / 8;
-    if (job != nullptr && job->active) {
-      the_job = job;
-      if (job_taken) *job_taken = true;
-    }
-  }
   auto kern = score_gemm_kernel<T, BM, BN, WAVES_M, WAVES_N, kSets, kDocMax, kStream>;
   static std::atomic<int> lds_limit_raised{0};
   MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(kern), (int)lds));
@@ -1345,7 +1058,7 @@ int launch_gemm(const void* qs, const void* kr, const uint32_t* row_bits, uint32
   if (slot >= 0) MSA_HIP(hipEventRecord(g_timer.start[slot], st));
   kern<<<grid, WAVES_M * WAVES_N * 64, lds, st>>>(static_cast<const T*>(qs), static_cast<const T*>(kr), row_bits, out_key,
                                                   chunk_doc, M_rows, C, K, blocks_per_query, tiles_m, tiles_n, m_group,
-                                                  n_docs, *the_job, sched, pool_n);
+                                                  n_docs);
   MSA_LAUNCH_CHECK();
   if (slot >= 0) MSA_HIP(hipEventRecord(g_timer.stop[slot], st));
   return MSA_OK;
@@ -1408,17 +1121,18 @@ int launch_scan4(const void* qs, const void* kr, const uint32_t* row_bits, uint3
 // ahead (1.5 % faster than the register-staged 128 x 384 it replaced, which beat register-staged 128 x 256 by 3 % and
 // 128 x 128 by 8 %; more register sets of loads in flight or 16 wavefronts measured 0-6 % slower: the bytes in flight
 // are not what limits this shape, the query tile's own traffic and the MFMA work are - with a query tile of zeros the
-// same launch streams at the rate of the 64-row form).  More rows are MFMA-bound: 256 x 256 tile.
+// same launch streams at the rate of the 64-row form).  More rows are MFMA-bound: the 256 x 256 tile of
+// score_scan4_kernel, which is also the form that can carry a gather job.
 template <bool kDocMax>
 int launch_gemm_for(int32_t dtype, const void* qs, const void* kr, const uint32_t* row_bits, uint32_t* out_key,
                     const int32_t* chunk_doc, int32_t M_rows, int32_t C, int32_t K, int32_t bpq, int32_t n_docs,
                     hipStream_t st, const GatherJob* job, bool* job_taken, uint32_t* sched) {
   if (dtype != MSA_BF16)
-    return launch_gemm<float, 128, 128, 2, 2, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
+    return launch_gemm<float, 128, 128, 2, 2, 1, kDocMax, false>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
   if (M_rows <= 64)
-    return launch_gemm<bf16_t, 64, 128, 2, 2, 2, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
+    return launch_gemm<bf16_t, 64, 128, 2, 2, 2, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
   if (M_rows <= 128)
-    return launch_gemm<bf16_t, 128, 256, 2, 4, 1, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
+    return launch_gemm<bf16_t, 128, 256, 2, 4, 1, kDocMax, true>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st);
   return launch_scan4<kDocMax>(qs, kr, row_bits, out_key, chunk_doc, M_rows, C, K, bpq, n_docs, st, job, job_taken, sched);
 }
 

@@ -97,3 +97,40 @@ def test_tile_pool_switch_is_exported():
     lib = _lib.load()
     assert lib.msa_route_set_tile_pool(0) == 0
     assert lib.msa_route_set_tile_pool(1) == 0
+
+
+def test_build_guard_flags_compiler_code_in_the_asm_statements_registers():
+    """The build checks the device assembly of the hand-scheduled scan: code the compiler generated for it (outside
+    the inline-asm regions) must stay below v128, leave the accumulation registers alone and use no scratch."""
+    from msa_amd import build as B
+    ok = """
+_ZN12_GLOBAL__N_118score_scan4_kernelILb1EEEvPKt:
+	v_add_u32_e32 v5, v4, v3
+	;;#ASMSTART
+	v_mfma_f32_32x32x16_bf16 a[0:15], v[128:131], v[144:147], a[0:15]
+	;;#ASMEND
+	s_endpgm
+"""
+    assert B.check_kernel_contracts(ok, "score_scan4_kernel", max_compiler_vgpr=127, no_agpr=True) == []
+    bad = ok.replace("v_add_u32_e32 v5, v4, v3", "v_accvgpr_write_b32 a3, v7\n\tv_mov_b32_e32 v130, v2\n\tscratch_store_dword off, v1, s32")
+    problems = B.check_kernel_contracts(bad, "score_scan4_kernel", max_compiler_vgpr=127, no_agpr=True)
+    assert len(problems) == 3, problems
+    assert B.check_kernel_contracts(ok, "no_such_kernel") != []
+
+
+def test_build_guard_fails_on_a_forced_spill():
+    """With the compiler's share of the scan kernel's registers cut to 24 the kernel spills, and the check that
+    build() runs on the device assembly reports it (this compiles route_score.hip once: about 15 s)."""
+    from msa_amd import build as B
+    src = open(os.path.join(B.CSRC, "route_score.hip")).read()
+    assert "constexpr int kScan4CompilerVgprs = 128;" in src
+    tmp = os.path.join(B.CSRC, "_guard_probe.hip")            # beside the sources: it includes its neighbours
+    try:
+        open(tmp, "w").write(src.replace("constexpr int kScan4CompilerVgprs = 128;", "constexpr int kScan4CompilerVgprs = 24;"))
+        asm = B._device_asm(tmp)
+    finally:
+        if os.path.exists(tmp):
+            os.remove(tmp)
+    problems = B.check_kernel_contracts(asm, "score_scan4_kernel", max_compiler_vgpr=127, no_agpr=True)
+    assert problems, "a spilling build passed the check"
+    assert any("spill" in p or "scratch" in p or "private_segment" in p or "accumulation" in p for p in problems), problems[:5]

@@ -40,6 +40,13 @@ extern "C" {
 #define MSA_MODE_COSINE 0      /* q L2-normalised per head here, K_r expected normalised, scale 1 */
 #define MSA_MODE_SCALED_DOT 1  /* raw dot product times `scale` (head_dim^-0.5 in the reference) */
 
+/* reductions of msa_route_topk_reduce (the reference's query_reduce_method / chunk_reduce_method strings) */
+#define MSA_QUERY_MAX 0    /* max over the scored tokens (src/msa_service.py:749-750): what msa_route_topk does */
+#define MSA_QUERY_MEAN 1   /* sum over the scored tokens / their number, at least 1 (:751-767) */
+#define MSA_QUERY_LAST 2   /* the token at position (number of scored tokens - 1) (:768-780) */
+#define MSA_CHUNK_MAX 0    /* max over a document's chunks (:787-792): what msa_route_topk does */
+#define MSA_CHUNK_MEAN 1   /* mean over a document's chunks (:794-811) */
+
 const char* msa_last_error(void);
 int msa_abi_version(void);
 
@@ -125,6 +132,18 @@ int msa_route_topk(const msa_bank* bank, int32_t layer, const void* q, const uin
 int msa_route_topk_static(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8,
                           int32_t B, int32_t S, int32_t Hq, int32_t mode, float scale, int32_t topk,
                           float* scores_out, int32_t* doc_out, int64_t* doc_global_out, void* stream);
+
+/* msa_route_topk with the reference's other reductions over a query's tokens and over a document's chunks
+ * (Memory.prefill_stage2, src/msa_service.py:749-811; the head reduction stays the mean).  query_reduce MEAN / LAST
+ * collapse every query to one row before the scan (both are linear in the query row or pick one row), so the scan
+ * reads the bank once for one row block per query.  A query without scored tokens gets -inf scores as in
+ * msa_route_topk (LAST: also when the token at that position is not scored).  chunk_reduce MEAN scores every chunk
+ * (the per-chunk plane of msa_chunk_scores), averages each document's chunks and selects from those means; it needs
+ * the workspace of msa_route_workspace_bytes, the others that of msa_route_topk_workspace_bytes. */
+int msa_route_topk_reduce(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
+                          int32_t S, int32_t Hq, int32_t mode, float scale, int32_t query_reduce, int32_t chunk_reduce,
+                          int32_t topk, float* scores_out, int32_t* doc_out, int64_t* doc_global_out, void* workspace,
+                          size_t workspace_bytes, void* stream);
 
 /* Measurement hook (no counterpart in the reference): while enabled, every launch of the scoring
  * kernel inside msa_chunk_scores / msa_route_topk is bracketed by a HIP event pair on its own

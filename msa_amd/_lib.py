@@ -31,6 +31,8 @@ SIGNATURES = {
     "msa_chunk_scores": (C.c_int, [_vp, _i32, _vp, _vp, _i32, _i32, _i32, _i32, _f32, _vp, _vp, _sz, _vp]),
     "msa_route_topk": (C.c_int, [_vp, _i32, _vp, _vp, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _vp, _vp, _vp, _sz,
                                  _vp]),
+    "msa_route_topk_reduce": (C.c_int, [_vp, _i32, _vp, _vp, _i32, _i32, _i32, _i32, _f32, _i32, _i32, _i32, _vp, _vp, _vp,
+                                        _vp, _sz, _vp]),
     "msa_route_topk_static": (C.c_int, [_vp, _i32, _vp, _vp, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _vp, _vp, _vp]),
     "msa_profile_enable": (C.c_int, [_i32]),
     "msa_profile_collect": (C.c_int, [_vp, _i32, _vp]),

@@ -30,6 +30,7 @@ struct RouteWorkspace {
   size_t off_key;       // uint32 [B, n_docs] (routing) or [B, C] (chunk scores): order-preserving keys of the unscaled scores
   size_t off_cand;      // uint64 [B, topk_blocks, kTopkMax] sorted candidates
   size_t off_sched;     // tile pool words of the persistent scan (counter cleared by the prologue kernel)
+  size_t off_collapsed; // fp32 [B, Hkv * D] + int32 [B]: a query collapsed to one row (mean / last over its tokens), tokens that counted
   size_t bytes;
 };
 
@@ -40,6 +41,8 @@ static inline int32_t topk_blocks_for(int64_t n_docs) {
 RouteWorkspace route_workspace_layout(int32_t B, int32_t S, int32_t Hkv, int32_t D, int64_t plane_cols, int64_t n_docs,
                                       int32_t dtype);
 
+// query_reduce: MSA_QUERY_*; extra_plane_cols: words per query reserved behind the key plane (the per-document keys
+// of the chunk-mean reduction).
 // Runs prologue + scoring GEMM on `st`; on success the keys (per document with doc_max, else per chunk) sit at
 // layout_out->off_key and score = key_to_f32(key) * (*mul_out); key 0 = nothing scored.
 // `job`: an optional gather to run inside the scan's launch; *job_taken tells whether the launch form could carry it
@@ -47,4 +50,5 @@ RouteWorkspace route_workspace_layout(int32_t B, int32_t S, int32_t Hkv, int32_t
 int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
                          int32_t S, int32_t Hq, int32_t mode, float scale, bool doc_max, void* workspace,
                          size_t workspace_bytes, hipStream_t st, RouteWorkspace* layout_out, float* mul_out,
-                         const char* who, const GatherJob* job = nullptr, bool* job_taken = nullptr);
+                         const char* who, const GatherJob* job = nullptr, bool* job_taken = nullptr,
+                         int32_t query_reduce = MSA_QUERY_MAX, int64_t extra_plane_cols = 0);

@@ -129,6 +129,113 @@ __global__ void presum_queries_kernel(const TIn* __restrict__ q, const uint8_t* 
 }
 
 // ------------------------------------------------------------------------------------------
+// The other reductions over a query's tokens (src/msa_service.py:751-780): "mean" (sum over the scored tokens / their
+// number) and "last" (the token at position count - 1, count = scored tokens).  Both are linear in the query row, or
+// pick one, so they collapse the query to ONE pre-summed row before the scan: mean_t (q_t . k) = (mean_t q_t) . k.
+// The scan and its max over rows then run unchanged on one row block per query whose 32 rows all hold that row.
+//
+// collapse_queries_kernel: one workgroup per (query, KV group); its 16 slots of 16 lanes take tokens slot, slot + 16,
+// ...; a slot sums, over its tokens that count, the group's (normalised, in cosine mode) heads; the slots meet in LDS in
+// a fixed order.  Writes the fp32 row and, from group 0, the number of tokens that counted.
+// ------------------------------------------------------------------------------------------
+constexpr int kQueryMax = MSA_QUERY_MAX, kQueryMean = MSA_QUERY_MEAN, kQueryLast = MSA_QUERY_LAST;
+
+template <typename TIn>
+__global__ __launch_bounds__(256) void collapse_queries_kernel(const TIn* __restrict__ q, const uint8_t* __restrict__ qmask,
+                                                               int32_t S, int32_t Hq, int32_t Hkv, int32_t normalize,
+                                                               int32_t query_reduce, float* __restrict__ rows,
+                                                               int32_t* __restrict__ counts) {
+  __shared__ float part[16][kHeadDim];
+  __shared__ int n_scored;
+  const int b = blockIdx.x, g = blockIdx.y;
+  const int G = Hq / Hkv;
+  const int slot = threadIdx.x >> 4, j = threadIdx.x & 15;
+  // scored tokens of the query (every wavefront counts them: the result is needed by all)
+  int count = 0;
+  if (qmask == nullptr) {
+    count = S;
+  } else {
+    const int lane = threadIdx.x & 63;
+    for (int base = 0; base < S; base += 64) {
+      const int t = base + lane;
+      count += __builtin_popcountll(__ballot(t < S && qmask[(int64_t)b * S + t] != 0));
+    }
+  }
+  const int last = max(count - 1, 0);
+  auto counts_in = [&](int t) {
+    const bool scored = qmask == nullptr || qmask[(int64_t)b * S + t] != 0;
+    return query_reduce == kQueryLast ? (t == last && scored) : scored;
+  };
+  float acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+  int used = 0;
+  for (int t = slot; t < S; t += 16) {
+    if (!counts_in(t)) continue;                       // (uniform over the slot's 16 lanes)
+    ++used;
+    const TIn* p0 = q + (((int64_t)b * S + t) * Hq + g * G) * kHeadDim + 8 * j;
+    for (int h = 0; h < G; ++h) {
+      float x[8];
+      const TIn* p = p0 + (int64_t)h * kHeadDim;
+      if constexpr (sizeof(TIn) == 2) {
+        const uint4 w = *reinterpret_cast<const uint4*>(p);
+        x[0] = bf16lo(w.x); x[1] = bf16hi(w.x); x[2] = bf16lo(w.y); x[3] = bf16hi(w.y);
+        x[4] = bf16lo(w.z); x[5] = bf16hi(w.z); x[6] = bf16lo(w.w); x[7] = bf16hi(w.w);
+      } else {
+        const float4 lo = *reinterpret_cast<const float4*>(p);
+        const float4 hi = *reinterpret_cast<const float4*>(p + 4);
+        x[0] = lo.x; x[1] = lo.y; x[2] = lo.z; x[3] = lo.w; x[4] = hi.x; x[5] = hi.y; x[6] = hi.z; x[7] = hi.w;
+      }
+      float inv = 1.f;
+      if (normalize) {
+        float ssq = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) ssq += x[i] * x[i];
+        inv = 1.0f / fmaxf(sqrtf(row16_sum(ssq)), 1e-12f);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += x[i] * inv;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) part[slot][8 * j + i] = acc[i];
+  if (threadIdx.x == 0) n_scored = 0;
+  __syncthreads();
+  if (j == 0 && used) atomicAdd(&n_scored, used);
+  __syncthreads();
+  if (threadIdx.x < kHeadDim) {
+    float sum = 0.f;
+    for (int s2 = 0; s2 < 16; ++s2) sum += part[s2][threadIdx.x];
+    const int n = n_scored;
+    rows[((int64_t)b * Hkv + g) * kHeadDim + threadIdx.x] = n > 0 ? sum / (float)n : 0.f;
+    if (g == 0 && threadIdx.x == 0) counts[b] = n;
+  }
+}
+
+// One row block (32 rows) per query, every row the collapsed row; mask words, padding words, the key plane and the
+// tile pool's counter as presum_queries_kernel leaves them.  One workgroup per row.
+template <typename TOut>
+__global__ void broadcast_rows_kernel(const float* __restrict__ rows, const int32_t* __restrict__ counts, int32_t Hkv,
+                                      TOut* __restrict__ qs, uint32_t* __restrict__ row_bits, int32_t mask_words,
+                                      uint32_t* __restrict__ key_plane, int64_t clear_words, uint32_t* __restrict__ sched) {
+  const int row = blockIdx.x, b = row >> 5;
+  const int K = Hkv * kHeadDim;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_words; i += (int64_t)gridDim.x * blockDim.x)
+    key_plane[i] = 0u;
+  const bool any = counts[b] > 0;
+  if ((row & 31) == 0 && threadIdx.x == 0) row_bits[row >> 5] = any ? 0xffffffffu : 0u;
+  if (blockIdx.x == 0) {
+    for (int w = (int)(gridDim.x >> 5) + (int)threadIdx.x; w < mask_words; w += blockDim.x) row_bits[w] = 0u;
+    if (threadIdx.x == 0) sched[0] = 0u;
+  }
+  for (int c = threadIdx.x; c < K; c += blockDim.x) {
+    const float x = any ? rows[(int64_t)b * K + c] : 0.f;
+    if constexpr (sizeof(TOut) == 2) qs[(int64_t)row * K + c] = f32_to_bf16(x);
+    else qs[(int64_t)row * K + c] = x;
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // MFMA operand traits.  LDS rows hold 128 bytes of K (64 bf16 or 32 fp32) plus 16 bytes of pad,
 // which makes the 16-byte / 4-byte operand reads of a 32-row block bank-conflict free.
 // ------------------------------------------------------------------------------------------
@@ -486,7 +593,7 @@ __global__ __launch_bounds__(WAVES_M* WAVES_N * 64) void score_gemm_kernel(
     emit(run_q, tile_n0, run, any);
   };
 
-  if constexpr (kDtlStream) {  } else if constexpr (kDtlStream) {
+  if constexpr (kDtlStream) {
     static_assert(kThreads == 512 && kSub == 4 && TM == 2 && TN == 2, "laid out for 8 wavefronts of 64 x 64");
     constexpr int kAStage = BM * 128, kBStage = BN * 128, kStages = 3;
     constexpr int kALoads = BM / 64, kBLoads = BN / 64;      // 1 KB blocks (8 rows) per wavefront and stage
@@ -1156,6 +1263,7 @@ RouteWorkspace route_workspace_layout(int32_t B, int32_t S, int32_t Hkv, int32_t
   w.topk_blocks = topk_blocks_for(n_docs);
   w.off_cand = off;     off = align_up(off + (size_t)B * w.topk_blocks * kTopkMax * sizeof(uint64_t), 256);
   w.off_sched = off;    off = align_up(off + kSchedBytes, 256);
+  w.off_collapsed = off; off = align_up(off + (size_t)B * Hkv * D * sizeof(float) + (size_t)B * sizeof(int32_t), 256);
   w.bytes = off;
   return w;
 }
@@ -1257,7 +1365,7 @@ extern "C" size_t msa_route_workspace_bytes(int32_t B, int32_t S, int32_t Hq, in
   (void)Hq; (void)topk;
   if (B <= 0 || S <= 0 || Hkv <= 0 || D <= 0 || C <= 0 || n_docs <= 0) return 0;
   // sized for fp32 queries so one workspace serves both dtypes, and for the per-chunk plane of msa_chunk_scores
-  return route_workspace_layout(B, S, Hkv, D, std::max(C, n_docs), n_docs, MSA_F32).bytes;
+  return route_workspace_layout(B, S, Hkv, D, C + n_docs, n_docs, MSA_F32).bytes;
 }
 
 extern "C" size_t msa_route_topk_workspace_bytes(int32_t B, int32_t S, int32_t Hq, int32_t Hkv, int32_t D,
@@ -1270,8 +1378,11 @@ extern "C" size_t msa_route_topk_workspace_bytes(int32_t B, int32_t S, int32_t H
 int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
                          int32_t S, int32_t Hq, int32_t mode, float scale, bool doc_max, void* workspace,
                          size_t workspace_bytes, hipStream_t st, RouteWorkspace* layout_out, float* mul_out,
-                         const char* who, const GatherJob* job, bool* job_taken) {
+                         const char* who, const GatherJob* job, bool* job_taken, int32_t query_reduce,
+                         int64_t extra_plane_cols) {
   if (job_taken) *job_taken = false;
+  MSA_REQUIRE(query_reduce == kQueryMax || query_reduce == kQueryMean || query_reduce == kQueryLast,
+              "%s: bad query reduction %d", who, query_reduce);
   MSA_REQUIRE(bank != nullptr, "%s: null bank", who);
   MSA_REQUIRE(layer >= 0 && layer < bank->n_layers, "%s: layer %d out of range", who, layer);
   if (bank->kr_dev[layer] == nullptr) {
@@ -1289,7 +1400,10 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
   MSA_REQUIRE((int64_t)B * ((S + 31) / 32 * 32) < (int64_t)1 << 24, "%s: too many query rows", who);
 
   const int64_t plane_cols = doc_max ? bank->n_docs : bank->C;
-  const RouteWorkspace w = route_workspace_layout(B, S, bank->Hkv, bank->D, plane_cols, bank->n_docs, bank->dtype);
+  // a collapsed query (mean / last over its tokens) is one row: one row block per query
+  const int32_t S_scan = query_reduce == kQueryMax ? S : 1;
+  const RouteWorkspace w = route_workspace_layout(B, S_scan, bank->Hkv, bank->D, plane_cols + extra_plane_cols, bank->n_docs,
+                                                  bank->dtype);
   if (w.bytes > workspace_bytes) {
     msa_set_error("%s: workspace of %zu bytes, need %zu", who, workspace_bytes, w.bytes);
     return MSA_ESIZE;
@@ -1303,14 +1417,32 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
   const int normalize = mode == MSA_MODE_COSINE ? 1 : 0;
   const int pthreads = bank->Hkv * 16;
   const int64_t clear_words = (int64_t)B * plane_cols;
-  if (bank->dtype == MSA_BF16)
+  if (query_reduce != kQueryMax) {
+    float* rows = reinterpret_cast<float*>(ws + w.off_collapsed);
+    int32_t* counts = reinterpret_cast<int32_t*>(rows + (size_t)B * bank->Hkv * bank->D);
+    const dim3 cgrid((unsigned)B, (unsigned)bank->Hkv);
+    if (bank->dtype == MSA_BF16) {
+      collapse_queries_kernel<bf16_t><<<cgrid, 256, 0, st>>>(static_cast<const bf16_t*>(q), qmask_u8, S, Hq, bank->Hkv,
+                                                             normalize, query_reduce, rows, counts);
+      MSA_LAUNCH_CHECK();
+      broadcast_rows_kernel<bf16_t><<<w.M_rows, 256, 0, st>>>(rows, counts, bank->Hkv, static_cast<bf16_t*>(qs), row_bits,
+                                                              w.mask_words, key, clear_words, sched);
+    } else {
+      collapse_queries_kernel<float><<<cgrid, 256, 0, st>>>(static_cast<const float*>(q), qmask_u8, S, Hq, bank->Hkv,
+                                                            normalize, query_reduce, rows, counts);
+      MSA_LAUNCH_CHECK();
+      broadcast_rows_kernel<float><<<w.M_rows, 256, 0, st>>>(rows, counts, bank->Hkv, static_cast<float*>(qs), row_bits,
+                                                             w.mask_words, key, clear_words, sched);
+    }
+  } else if (bank->dtype == MSA_BF16) {
     presum_queries_kernel<bf16_t, bf16_t><<<w.M_rows, pthreads, 0, st>>>(
         static_cast<const bf16_t*>(q), qmask_u8, B, S, w.S_pad, Hq, bank->Hkv, normalize, static_cast<bf16_t*>(qs),
         row_bits, w.mask_words, key, clear_words, sched);
-  else
+  } else {
     presum_queries_kernel<float, float><<<w.M_rows, pthreads, 0, st>>>(
         static_cast<const float*>(q), qmask_u8, B, S, w.S_pad, Hq, bank->Hkv, normalize, static_cast<float*>(qs),
         row_bits, w.mask_words, key, clear_words, sched);
+  }
   MSA_LAUNCH_CHECK();
 
   const int32_t K = bank->Hkv * bank->D;

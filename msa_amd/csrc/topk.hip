@@ -196,7 +196,60 @@ int route_topk_impl(const msa_bank* bank, int32_t layer, const void* q, const ui
   return MSA_OK;
 }
 
+// keys of the per-chunk scores [B, C] -> keys of each document's mean over its chunks [B, n_docs]; a query whose
+// chunk keys are 0 (no scored token) keeps 0.  One thread per (query, document).
+__global__ void doc_mean_kernel(const uint32_t* __restrict__ chunk_key, const int32_t* __restrict__ doc_chunk_off,
+                                int64_t C, int32_t n_docs, uint32_t* __restrict__ doc_key) {
+  const int d = blockIdx.x * blockDim.x + threadIdx.x, b = blockIdx.y;
+  if (d >= n_docs) return;
+  const int c0 = doc_chunk_off[d], c1 = doc_chunk_off[d + 1];
+  float sum = 0.f;
+  bool none = c1 <= c0;
+  for (int c = c0; c < c1; ++c) {
+    const uint32_t k = chunk_key[(int64_t)b * C + c];
+    if (k == 0) none = true;
+    else sum += key_to_f32(k);
+  }
+  doc_key[(int64_t)b * n_docs + d] = none ? 0u : f32_to_key(sum / (float)(c1 - c0));
+}
+
 }  // namespace
+
+extern "C" int msa_route_topk_reduce(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
+                                     int32_t S, int32_t Hq, int32_t mode, float scale, int32_t query_reduce,
+                                     int32_t chunk_reduce, int32_t topk, float* scores_out, int32_t* doc_out,
+                                     int64_t* doc_global_out, void* workspace, size_t workspace_bytes, void* stream) {
+  const char* who = "msa_route_topk_reduce";
+  MSA_REQUIRE(chunk_reduce == MSA_CHUNK_MAX || chunk_reduce == MSA_CHUNK_MEAN, "%s: bad chunk reduction %d", who, chunk_reduce);
+  MSA_REQUIRE(scores_out && doc_out, "%s: null output", who);
+  MSA_REQUIRE(topk > 0 && topk <= kTopkMax, "%s: topk=%d out of range (1..%d)", who, topk, kTopkMax);
+  MSA_REQUIRE(bank != nullptr, "%s: null bank", who);
+  RouteWorkspace w;
+  float mul;
+  hipStream_t st = as_stream(stream);
+  const bool doc_max = chunk_reduce == MSA_CHUNK_MAX;
+  // (chunk mean: the scan leaves one key per (query, chunk); the per-document keys go behind that plane)
+  int rc = route_scores_to_keys(bank, layer, q, qmask_u8, B, S, Hq, mode, scale, doc_max, workspace, workspace_bytes, st, &w,
+                                &mul, who, nullptr, nullptr, query_reduce, doc_max ? 0 : bank->n_docs);
+  if (rc != MSA_OK) return rc;
+  char* ws = static_cast<char*>(workspace);
+  const uint32_t* key = reinterpret_cast<const uint32_t*>(ws + w.off_key);
+  if (!doc_max) {
+    uint32_t* doc_key = reinterpret_cast<uint32_t*>(ws + w.off_key) + (size_t)B * bank->C;
+    const dim3 mgrid((unsigned)((bank->n_docs + 255) / 256), (unsigned)B);
+    doc_mean_kernel<<<mgrid, 256, 0, st>>>(key, bank->doc_chunk_off_dev, bank->C, (int32_t)bank->n_docs, doc_key);
+    MSA_LAUNCH_CHECK();
+    key = doc_key;
+  }
+  uint64_t* cand = reinterpret_cast<uint64_t*>(ws + w.off_cand);
+  dim3 grid((unsigned)w.topk_blocks, (unsigned)B);
+  doc_topk_kernel<<<grid, kWaves * 64, 0, st>>>(key, (int32_t)bank->n_docs, topk, cand);
+  MSA_LAUNCH_CHECK();
+  merge_topk_kernel<<<B, kMergeWaves * 64, 0, st>>>(cand, w.topk_blocks, bank->doc_global_id_dev, mul, topk, scores_out, doc_out,
+                                      doc_global_out);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
 
 extern "C" int msa_route_topk(const msa_bank* bank, int32_t layer, const void* q, const uint8_t* qmask_u8, int32_t B,
                               int32_t S, int32_t Hq, int32_t mode, float scale, int32_t topk, float* scores_out,

@@ -102,12 +102,13 @@ class Memory:
         self.head_reduce_method, self.query_reduce_method = mc.head_reduce_method, mc.query_reduce_method
         self.chunk_reduce_method, self.aux_loss_method = mc.chunk_reduce_method, mc.aux_loss_method
         self.decouple_router = mc.decouple_router
-        # the kernels implement the shipped reductions only (src/msa_service.py:742-813 has others)
-        for name, got, want in (("head_reduce_method", self.head_reduce_method, "mean"),
-                                ("query_reduce_method", self.query_reduce_method, "max")):
-            if got != want:
-                raise NotImplementedError(f"Unsupported {name.split('_')[0]} reduce method: {got}")
-        if self.chunk_reduce_method != "max":
+        # the reductions of src/msa_service.py:742-813: heads "mean" (the kernels sum a group's heads before the
+        # scan, which a max over heads does not allow), tokens "max" / "mean" / "last", chunks "max" / "mean"
+        if self.head_reduce_method != "mean":
+            raise NotImplementedError(f"Unsupported head reduce method: {self.head_reduce_method}")
+        if self.query_reduce_method not in ops.QUERY_REDUCE:
+            raise NotImplementedError(f"Unsupported query reduce method: {self.query_reduce_method}")
+        if self.chunk_reduce_method not in ops.CHUNK_REDUCE:
             raise ValueError(f"Invalid chunk reduction method: {self.chunk_reduce_method}")
         # -1 marks "already cosine, do not scale" exactly as the reference does (:318-321)
         self.scaling = -1.0 if (self.aux_loss_method == "INFONCE" and self.decouple_router) else cfg.head_dim ** -0.5
@@ -290,7 +291,8 @@ class Memory:
     # ---------------------------------------------------------------- scorer (:703-828)
     def _route(self, layer_idx: int, q_bshd: torch.Tensor, mask_bs: Optional[torch.Tensor], mode: str, scale: float):
         top_k = self.model_config.doc_top_k
-        scores, doc, gid = ops.route_topk(self.bank, self._layer_slot[layer_idx], q_bshd, mask_bs, mode, scale, top_k)
+        scores, doc, gid = ops.route_topk(self.bank, self._layer_slot[layer_idx], q_bshd, mask_bs, mode, scale, top_k,
+                                          query_reduce=self.query_reduce_method, chunk_reduce=self.chunk_reduce_method)
         return scores, doc, gid
 
     def prefill_stage2(self, layer_idx: int, query_states: torch.Tensor, query_mask: torch.Tensor):
@@ -339,6 +341,9 @@ class MSAService(Memory, MemoryClientBase):
         else:
             mode, scale = "scaled_dot", (1.0 if self.scaling < 0 else self.scaling)
         scores, doc, gid = self._route(layer_idx, q_bshd, query_mask, mode, scale)
+        if fused_normalize and self.scaling > 0:
+            # normalised queries are still multiplied by head_dim^-0.5 unless the router is decoupled (:318-321, 1095-1096)
+            scores = scores * self.scaling
         doc = torch.where(scores > -1e9, doc, torch.full_like(doc, -1))      # drop invalid picks (:1190-1191)
         B, k = doc.shape
         cap = B * k * self.bank.max_doc_chunks
@@ -365,6 +370,8 @@ class MSAService(Memory, MemoryClientBase):
         else:
             mode, scale = "scaled_dot", (1.0 if self.scaling < 0 else self.scaling)
         scores, doc, gid = self._route(layer_idx, q, query_mask, mode, scale)
+        if fused_normalize and self.scaling > 0:
+            scores = scores * self.scaling                   # (:318-321, 1095-1096: only a decoupled router skips the scale)
         valid = scores > -1e9
         doc = torch.where(valid, doc, torch.full_like(doc, -1))
         if self._ids_host is None or self._ids_host.shape != doc.shape:

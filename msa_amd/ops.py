@@ -184,17 +184,33 @@ def chunk_scores(bank: Bank, layer: int, q: torch.Tensor, qmask: Optional[torch.
     return out
 
 
+QUERY_REDUCE = {"max": 0, "mean": 1, "last": 2}     # the reference's query_reduce_method (src/msa_service.py:749-780)
+CHUNK_REDUCE = {"max": 0, "mean": 1}                # chunk_reduce_method (:787-811)
+
+
 def route_topk(bank: Bank, layer: int, q: torch.Tensor, qmask: Optional[torch.Tensor] = None, mode: str = "cosine",
-               scale: float = 1.0, topk: int = 16):
-    """``(scores [B, k] fp32, doc [B, k] int32 0-based, doc_global [B, k] int64)``."""
+               scale: float = 1.0, topk: int = 16, query_reduce: str = "max", chunk_reduce: str = "max"):
+    """``(scores [B, k] fp32, doc [B, k] int32 0-based, doc_global [B, k] int64)``.  ``query_reduce`` / ``chunk_reduce``
+    other than "max" take the reference's other reductions (``msa_route_topk_reduce``)."""
     B, S, Hq, qm = _route_args(bank, q, qmask, mode)
-    ws = bank.workspace(B, S, Hq, topk, q.device)
+    if query_reduce not in QUERY_REDUCE:
+        raise NotImplementedError(f"Unsupported query reduce method: {query_reduce}")
+    if chunk_reduce not in CHUNK_REDUCE:
+        raise ValueError(f"Invalid chunk reduction method: {chunk_reduce}")
     scores = torch.empty((B, topk), dtype=torch.float32, device=q.device)
     doc = torch.empty((B, topk), dtype=torch.int32, device=q.device)
     gid = torch.empty((B, topk), dtype=torch.int64, device=q.device)
-    check(_lib.load().msa_route_topk(bank.handle, layer, ptr(q), ptr(qm), B, S, Hq, MODES[mode], scale, topk,
-                                     ptr(scores), ptr(doc), ptr(gid), ptr(ws), ws.numel(), _stream()),
-          "msa_route_topk")
+    if query_reduce == "max" and chunk_reduce == "max":
+        ws = bank.workspace(B, S, Hq, topk, q.device)
+        check(_lib.load().msa_route_topk(bank.handle, layer, ptr(q), ptr(qm), B, S, Hq, MODES[mode], scale, topk,
+                                         ptr(scores), ptr(doc), ptr(gid), ptr(ws), ws.numel(), _stream()),
+              "msa_route_topk")
+    else:
+        ws = bank.workspace(B, S, Hq, topk, q.device, chunk_plane=chunk_reduce != "max")
+        check(_lib.load().msa_route_topk_reduce(bank.handle, layer, ptr(q), ptr(qm), B, S, Hq, MODES[mode], scale,
+                                                QUERY_REDUCE[query_reduce], CHUNK_REDUCE[chunk_reduce], topk, ptr(scores),
+                                                ptr(doc), ptr(gid), ptr(ws), ws.numel(), _stream()),
+              "msa_route_topk_reduce")
     return scores, doc, gid
 
 

@@ -122,11 +122,16 @@ def chunk_scores(
     mode: str = "cosine",   # "cosine": q normalised here, kr assumed normalised, scale 1
     scale: float | None = None,
     chunk_block: int = 4096,
+    query_reduce: str = "max",
 ) -> torch.Tensor:
     """``s[b,c] = max_{t valid} (1/Hq) sum_h q'[b,t,h] . kr[c, h // G] * scale``.
 
     Restates matmul (:730) -> mask (:733) -> mean over the Hq heads (:745) ->
     max over tokens (:750).  A query with no valid token scores -inf.
+    ``query_reduce`` "mean": sum over the valid tokens / max(their number, 1)
+    (:751-767); "last": the token at position (number of valid tokens - 1), -inf
+    if that position is not a valid token (:768-780, where a masked position
+    carries the dtype's lowest value).
     """
     B, S, Hq, D = q.shape
     C, Hkv, _ = kr.shape
@@ -146,18 +151,39 @@ def chunk_scores(
         kb = kr[c0 : c0 + chunk_block]                      # [c, Hkv, D]
         # per-head dots then mean over all Hq heads
         s = torch.einsum("bsgjd,cgd->bsc", qg, kb) * (sc / Hq)
-        s = s.masked_fill(~qmask[:, :, None], NEG_INF)
-        out[:, c0 : c0 + chunk_block] = s.max(dim=1).values
+        if query_reduce == "max":
+            s = s.masked_fill(~qmask[:, :, None], NEG_INF)
+            red = s.max(dim=1).values
+        elif query_reduce == "mean":
+            n = qmask.sum(dim=1).clamp(min=1).to(F64)
+            red = torch.where(qmask[:, :, None], s, torch.zeros_like(s)).sum(dim=1) / n[:, None]
+            red = torch.where((qmask.sum(dim=1) > 0)[:, None], red, torch.full_like(red, NEG_INF))
+        elif query_reduce == "last":
+            n = qmask.sum(dim=1)
+            last = (n - 1).clamp(min=0)
+            red = s[torch.arange(B), last]
+            ok = qmask[torch.arange(B), last] & (n > 0)
+            red = torch.where(ok[:, None], red, torch.full_like(red, NEG_INF))
+        else:
+            raise NotImplementedError(f"Unsupported query reduce method: {query_reduce}")
+        out[:, c0 : c0 + chunk_block] = red
     return out
 
 
-def doc_scores(cs: torch.Tensor, doc_chunk_off: np.ndarray) -> torch.Tensor:
-    """Max over each document's chunks (scatter_reduce amax, :789-792, :817-820)."""
+def doc_scores(cs: torch.Tensor, doc_chunk_off: np.ndarray, chunk_reduce: str = "max") -> torch.Tensor:
+    """Max over each document's chunks (scatter_reduce amax, :789-792, :817-820); ``chunk_reduce``
+    "mean": their mean (sum / count, :794-811)."""
     B = cs.shape[0]
     n = len(doc_chunk_off) - 1
     out = torch.empty((B, n), dtype=cs.dtype)
     for d in range(n):
-        out[:, d] = cs[:, int(doc_chunk_off[d]) : int(doc_chunk_off[d + 1])].max(dim=1).values
+        part = cs[:, int(doc_chunk_off[d]) : int(doc_chunk_off[d + 1])]
+        if chunk_reduce == "max":
+            out[:, d] = part.max(dim=1).values
+        elif chunk_reduce == "mean":
+            out[:, d] = part.sum(dim=1) / part.shape[1]
+        else:
+            raise ValueError(f"Invalid chunk reduction method: {chunk_reduce}")
     return out
 
 

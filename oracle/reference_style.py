@@ -113,7 +113,8 @@ def group_queries(query_states: torch.Tensor, query_mask: torch.Tensor, num_kv_g
 
 
 def stage2_scores_topk(q5: torch.Tensor, m5: torch.Tensor, rk: torch.Tensor, pool_ids: torch.Tensor,
-                       doc_num_chunks: List[int], top_k: int, slice_chunk_size: int = 16 * 1024):
+                       doc_num_chunks: List[int], top_k: int, slice_chunk_size: int = 16 * 1024,
+                       query_reduce: str = "max", chunk_reduce: str = "max"):
     """The scorer loop: per slice matmul (:730) -> masked_fill (:733) ->
     mean over heads (:745) -> max over tokens (:750) -> amax chunk->slice doc
     (:787-792) -> amax slice doc->bank doc (:816-820); then topk (:826).
@@ -136,9 +137,28 @@ def stage2_scores_topk(q5: torch.Tensor, m5: torch.Tensor, rk: torch.Tensor, poo
         kt = rk[:, :, start:end].transpose(-1, -2).unsqueeze(2)              # [1, Hkv, 1, D, Cs]
         s = torch.matmul(q5, kt)                                             # [B, Hkv, G, S, Cs]
         s.masked_fill_(blocked, lowest)
-        s = s.flatten(1, 2).mean(dim=1).max(dim=1).values                    # [B, Cs]
+        s = s.flatten(1, 2).mean(dim=1)                                      # [B, S, Cs]
+        if query_reduce == "max":
+            s = s.max(dim=1).values                                          # [B, Cs]
+        elif query_reduce == "mean":                                         # :751-767
+            seen = m5.squeeze(2).squeeze(1)                                  # [B, S, 1]
+            s = torch.where(seen, s, torch.zeros_like(s)).sum(dim=1) / seen.sum(dim=1).clamp(min=1.0)
+        elif query_reduce == "last":                                         # :768-780
+            n_seen = m5.reshape(B, -1).sum(dim=1).long()
+            at = (n_seen - 1).clamp(min=0).view(B, 1, 1).expand(-1, 1, s.shape[2])
+            s = s.gather(1, at).squeeze(1)
+        else:
+            raise NotImplementedError(f"Unsupported query reduce method: {query_reduce}")
+        index = local0.view(1, -1).expand(B, -1)
         per_doc = torch.full((B, bank_ids.numel()), -float("inf"), dtype=dtype)
-        per_doc.scatter_reduce_(1, local0.view(1, -1).expand(B, -1), s, reduce="amax", include_self=True)
+        if chunk_reduce == "max":
+            per_doc.scatter_reduce_(1, index, s, reduce="amax", include_self=True)
+        elif chunk_reduce == "mean":                                         # :794-811
+            sums = torch.zeros_like(per_doc).scatter_reduce(1, index, s, reduce="sum", include_self=False)
+            counts = torch.zeros_like(per_doc).scatter_reduce(1, index, torch.ones_like(s), reduce="sum", include_self=False)
+            per_doc = torch.where(counts > 0, sums / counts.clamp(min=1.0), per_doc)
+        else:
+            raise ValueError(f"Invalid chunk reduction method: {chunk_reduce}")
         table.scatter_reduce_(1, bank_ids.view(1, -1).expand(B, -1), per_doc, reduce="amax", include_self=True)
     return torch.topk(table, k=min(top_k, table.shape[1]), dim=1)
 

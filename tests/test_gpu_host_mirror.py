@@ -220,9 +220,16 @@ def test_unsupported_reductions_raise(env):
     bad = cfgm.MSAConfig(msa_config=dict(cfgm.default_msa_config(), head_reduce_method="max"))
     with pytest.raises(NotImplementedError, match="Unsupported head reduce method"):
         env["svc"].Memory(0, cfgm.GenerateConfig(devices=[0]), cfgm.ModelConfig(), cfgm.MemoryConfig(), bad)
-    bad = cfgm.MSAConfig(msa_config=dict(cfgm.default_msa_config(), chunk_reduce_method="mean"))
+    bad = cfgm.MSAConfig(msa_config=dict(cfgm.default_msa_config(), chunk_reduce_method="median"))
     with pytest.raises(ValueError, match="Invalid chunk reduction method"):
         env["svc"].Memory(0, cfgm.GenerateConfig(devices=[0]), cfgm.ModelConfig(), cfgm.MemoryConfig(), bad)
+    bad = cfgm.MSAConfig(msa_config=dict(cfgm.default_msa_config(), query_reduce_method="first"))
+    with pytest.raises(NotImplementedError, match="Unsupported query reduce method"):
+        env["svc"].Memory(0, cfgm.GenerateConfig(devices=[0]), cfgm.ModelConfig(), cfgm.MemoryConfig(), bad)
+    # the reference's other token / chunk reductions are accepted (src/msa_service.py:751-811)
+    ok = cfgm.MSAConfig(msa_config=dict(cfgm.default_msa_config(), query_reduce_method="mean", chunk_reduce_method="mean"))
+    mem = env["svc"].Memory(0, cfgm.GenerateConfig(devices=[0]), cfgm.ModelConfig(), cfgm.MemoryConfig(), ok)
+    assert (mem.query_reduce_method, mem.chunk_reduce_method) == ("mean", "mean")
     layer = _layer(env).cuda()
     with pytest.raises(Exception, match="error!"):
         layer(torch.zeros(1, 1, HID).cuda(), torch.zeros(1, 1).long().cuda())

@@ -143,6 +143,40 @@ def test_chunk_scores(ops, dtype, mode, B, S):
     assert cf.rel_err(got2.cpu(), want2) < TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("mode", ["cosine", "scaled_dot"])
+@pytest.mark.parametrize("query_reduce,chunk_reduce", [("mean", "max"), ("last", "max"), ("max", "mean"), ("mean", "mean"),
+                                                        ("last", "mean")])
+def test_route_topk_other_reductions(ops, dtype, mode, query_reduce, chunk_reduce):
+    """query_reduce_method mean / last and chunk_reduce_method mean (src/msa_service.py:751-811) against the oracle:
+    scores of the returned documents within tolerance, the selection by the acceptance rule, a query without scored
+    tokens all -inf."""
+    say(f"route_topk_reduce dtype={dtype} mode={mode} query={query_reduce} chunk={chunk_reduce}")
+    B, S, Hq, Hkv, D, k = 6, 50, 32, 8, 128, 8
+    doc_chunks = _ragged(8, 700, 1, 7)
+    bank, kr, dco, gids, _, _ = _make_bank(ops, doc_chunks, Hkv, D, dtype, 61, normalize=(mode == "cosine"))
+    q = _randn((B, S, Hq, D), 62, dtype)
+    mask = torch.ones(B, S, dtype=torch.bool)
+    mask[1, S // 2:] = False                                  # a prefix of scored tokens
+    mask[2, 3] = False; mask[2, 10] = False                   # holes (position count - 1 is scored)
+    mask[3] = False                                           # nothing scored
+    mask[4, 1:] = False                                       # one token
+    scores, doc, gid = ops.route_topk(bank, 1, q.cuda(), mask.cuda(), mode, D ** -0.5, k, query_reduce=query_reduce,
+                                      chunk_reduce=chunk_reduce)
+    torch.cuda.synchronize()
+    scores, doc = scores.cpu(), doc.cpu().long()
+    ds = cf.doc_scores(cf.chunk_scores(q, mask, kr, mode, query_reduce=query_reduce), dco, chunk_reduce)
+    live = [b for b in range(B) if b != 3]
+    assert torch.isinf(scores[3]).all() and (scores[3] < 0).all()
+    # mean scores sit close together: the acceptance gap is widened by the dtype's score error
+    scale = float(ds[live].abs().max())
+    gap = max(1e-3, 2 * TOL[dtype] * scale)
+    assert not cf.topk_acceptable(ds[live], doc[live], k, gap=gap)
+    picked = torch.gather(ds[live], 1, doc[live])
+    assert cf.rel_err(scores[live], picked) < TOL[dtype]
+    assert (scores[live][:, :-1] >= scores[live][:, 1:]).all()
+
+
 def test_chunk_scores_fully_masked_query(ops):
     say("chunk_scores fully masked")
     bank, kr, *_ = _make_bank(ops, [3, 4, 5], 8, 128, torch.bfloat16, 31)

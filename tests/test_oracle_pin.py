@@ -214,6 +214,60 @@ def test_scores_topk_reference_style_agrees(mode):
     assert (got_i >= 1).all()                                                   # dummy slot 0 never wins
 
 
+@pytest.mark.parametrize("query_reduce,chunk_reduce", [("mean", "max"), ("last", "max"), ("max", "mean"), ("mean", "mean"),
+                                                        ("last", "mean")])
+def test_other_reductions_brute_force_and_reference_style_agree(query_reduce, chunk_reduce):
+    """The reference's other reductions over tokens and chunks (src/msa_service.py:751-811), pinned by plain loops over
+    every (query, token, head, chunk) and by the reference-style op sequence (several slices)."""
+    B, S, Hq, Hkv, D, k = 3, 7, 8, 2, 16, 4
+    G = Hq // Hkv
+    doc_chunks = _ragged(11, 40, 1, 6)
+    _, dco, _, _, cd = cf.chunk_table([n * 4 for n in doc_chunks], 4)
+    kr = _bank(2, doc_chunks, Hkv, D, normalize=False).double()
+    q = torch.randn(B, S, Hq, D).double()
+    mask = torch.ones(B, S, dtype=torch.bool)
+    mask[1, 4:] = False                       # a prefix of 4 scored tokens
+    mask[2, 0] = False; mask[2, 3] = False    # holes: 5 scored tokens, position 4 is scored
+    sc = D ** -0.5
+    C = kr.shape[0]
+    # brute force
+    want_c = torch.empty(B, C, dtype=torch.float64)
+    for b in range(B):
+        seen = [t for t in range(S) if mask[b, t]]
+        for c in range(C):
+            per_tok = []
+            for t in range(S):
+                tot = 0.0
+                for h in range(Hq):
+                    tot += float(q[b, t, h] @ kr[c, h // G]) * sc
+                per_tok.append(tot / Hq)
+            if query_reduce == "mean":
+                want_c[b, c] = sum(per_tok[t] for t in seen) / max(len(seen), 1)
+            else:
+                want_c[b, c] = per_tok[len(seen) - 1] if mask[b, len(seen) - 1] else -math.inf
+                if query_reduce == "max":
+                    want_c[b, c] = max(per_tok[t] for t in seen)
+    got_c = cf.chunk_scores(q, mask, kr, "scaled_dot", query_reduce=query_reduce)
+    assert torch.allclose(got_c, want_c, atol=1e-12)
+    want_d = torch.empty(B, len(doc_chunks), dtype=torch.float64)
+    for d in range(len(doc_chunks)):
+        cols = [float("nan")] * 0
+        for b in range(B):
+            vals = [float(want_c[b, c]) for c in range(int(dco[d]), int(dco[d + 1]))]
+            want_d[b, d] = max(vals) if chunk_reduce == "max" else sum(vals) / len(vals)
+    got_d = cf.doc_scores(got_c, dco, chunk_reduce)
+    assert torch.allclose(got_d, want_d, atol=1e-12)
+    # the reference-style sequence (fp64 here), slices of 32 chunks
+    qh = q.permute(0, 2, 1, 3).contiguous()
+    q5, m5 = rs.group_queries(qh, mask, G, sc)
+    rk = kr.transpose(0, 1).unsqueeze(0)
+    got_s, got_i = rs.stage2_scores_topk(q5, m5, rk, torch.as_tensor(cd + 1), doc_chunks, k, slice_chunk_size=32,
+                                         query_reduce=query_reduce, chunk_reduce=chunk_reduce)
+    want_s, want_i = cf.topk_docs(want_d, k)
+    assert torch.allclose(got_s, want_s, atol=1e-9)
+    assert torch.equal(got_i - 1, want_i)
+
+
 def test_make_slices_doc_aligned_and_tail_merge():
     chunks = [600] * 5 + [100]
     sl = rs.make_slices(chunks, 1024)

@@ -304,7 +304,10 @@ int msa_qk_norm_rope(const void* q, const void* k, const void* v, int64_t q_row_
  * Hkv v heads | Hr_back router heads (so one [rk | q | k | v | rq] matrix serves stage 1 with Hr_front = Hkv, stage 2
  * with a pointer 1024 rows in and Hr_back = Hq, and the decode step's q | k | v slice).  K a multiple of 64.
  * Outputs are dense: q_out [T, Hq, 128], k_out / v_out [T, Hkv, 128], r_out [T, Hr_front + Hr_back, 128]
- * (router heads are stored as projected: no norm, no rotary). */
+ * (router heads are stored as projected: no norm, no rotary).  All of x, w, the outputs and the norm weights are
+ * bf16 (q_norm_w / k_norm_w: 128 values each, 16-byte aligned like x, w and the outputs); the rotary tables are fp32
+ * [rope_rows, 64].  The element types cannot be checked through this interface: a caller with fp32 norm weights
+ * converts them first (or uses msa_qk_norm_rope, which takes a dtype). */
 int msa_qkv_proj(const void* x, int64_t T, int32_t K, const void* w, int32_t Hq, int32_t Hkv, int32_t Hr_front,
                  int32_t Hr_back, const int64_t* positions, const void* q_norm_w, const void* k_norm_w, float eps,
                  const float* rope_cos, const float* rope_sin, int32_t rope_rows, void* q_out, void* k_out,

@@ -145,3 +145,71 @@ def load_docs(path: str):
         return None
     with open(f) as fh:
         return [json.loads(line) for line in fh if line.strip()]
+
+
+# --------------------------------------------------------------------------------------------------------------
+# Banks the reference wrote (Memory.serialize, src/msa_service.py:351-404): a directory of ``layer_<i>_k.pt``,
+# ``layer_<i>_v.pt``, ``layer_<i>_rk.pt`` (one pooled tensor each, ``[1, Hkv, C, D]``), ``prefix_cache.pt``
+# (``{layer: (k, v)}``, ``[1, Hkv, n, D]``), ``meta.pt`` and ``stub.json``.  The tensor files are plain tensors and
+# load with ``weights_only=True``; ``meta.pt`` pickles the reference's Document objects and is never opened here: the
+# caller supplies the documents (ids and chunk counts, bank order), as the reference's own meta would.
+# --------------------------------------------------------------------------------------------------------------
+def _load_plain(path: str):
+    return torch.load(path, map_location="cpu", weights_only=True)
+
+
+def reference_bank_layers(path: str) -> List[int]:
+    """Router layers a reference bank directory holds K_r for."""
+    out = []
+    for name in os.listdir(path):
+        if name.startswith("layer_") and name.endswith("_rk.pt"):
+            out.append(int(name[len("layer_"):-len("_rk.pt")]))
+    return sorted(out)
+
+
+def read_reference_layer(path: str, layer: int) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """``(rk, k, v)`` of one layer of a reference bank, chunk-major ``[C, Hkv, D]`` (the reference keeps
+    ``[1, Hkv, C, D]``).  Whatever device the reference restored each of them to (its deserialize puts K on the
+    GPU and leaves K_r on the host, :447-461, the reverse of where its scorer and gather read them), here all three
+    come back as host tensors and the caller places them: K_r in HBM, K / V in pinned host memory."""
+    out = []
+    for tag in ("rk", "k", "v"):
+        f = os.path.join(path, f"layer_{layer}_{tag}.pt")
+        if not os.path.exists(f):
+            raise FileNotFoundError(f"{f}: the reference bank has no {tag} for layer {layer}")
+        t = _load_plain(f)
+        if not isinstance(t, torch.Tensor) or t.dim() != 4 or t.shape[0] != 1:
+            raise ValueError(f"{f}: expected one tensor [1, Hkv, C, D], got {type(t).__name__} "
+                             f"{tuple(t.shape) if isinstance(t, torch.Tensor) else ''}")
+        out.append(t[0].transpose(0, 1).contiguous())
+    if not (out[0].shape == out[1].shape == out[2].shape):
+        raise ValueError(f"layer {layer}: rk / k / v shapes differ: {[tuple(x.shape) for x in out]}")
+    return out[0], out[1], out[2]
+
+
+def read_reference_prefix(path: str) -> Dict[int, Tuple[torch.Tensor, torch.Tensor]]:
+    """Template-prefix K / V of every layer, ``{layer: (k, v)}`` with ``[1, Hkv, n, D]`` tensors (empty if absent)."""
+    f = os.path.join(path, "prefix_cache.pt")
+    if not os.path.exists(f):
+        return {}
+    raw = _load_plain(f)
+    return {int(layer): (kv[0], kv[1]) for layer, kv in raw.items()}
+
+
+def convert_reference_bank(src: str, dst: str, docs, header: dict) -> None:
+    """Converts a bank directory the reference wrote into this format (``save_bank``), one layer at a time.
+    ``docs``: the documents in bank order (objects with ``doc_id``, ``num_chunks`` and optionally ``doc``);
+    ``header``: the scoring / pooling hyper-parameters to record (see ``Memory.serialize``)."""
+    counts = [int(d.num_chunks) for d in docs]
+    off = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+    layers = reference_bank_layers(src)
+    if not layers:
+        raise ValueError(f"{src}: no layer_<i>_rk.pt files")
+    rk, k, v = {}, {}, {}
+    for layer in layers:
+        rk[layer], k[layer], v[layer] = read_reference_layer(src, layer)
+        if rk[layer].shape[0] != int(off[-1]):
+            raise ValueError(f"layer {layer}: {rk[layer].shape[0]} chunks, the documents add up to {int(off[-1])}")
+    os.makedirs(dst, exist_ok=True)
+    save_docs(dst, docs)
+    save_bank(dst, header, off.tolist(), [int(d.doc_id) for d in docs], rk, k, v, read_reference_prefix(src))

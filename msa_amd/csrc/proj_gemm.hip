@@ -293,6 +293,11 @@ extern "C" int msa_qkv_proj(const void* x, int64_t T, int32_t K, const void* w, 
   MSA_REQUIRE((Hr_front + Hr_back == 0) || r_out != nullptr, "msa_qkv_proj: router heads without an output");
   MSA_REQUIRE(rope_rows > 0 && eps > 0.f, "msa_qkv_proj: rope_rows / eps");
   MSA_REQUIRE((((uintptr_t)x | (uintptr_t)w) & 15) == 0, "msa_qkv_proj: x / w must be 16-byte aligned");
+  MSA_REQUIRE((((uintptr_t)q_norm_w | (uintptr_t)k_norm_w) & 15) == 0,
+              "msa_qkv_proj: q_norm_w / k_norm_w (128 bf16 each) must be 16-byte aligned");
+  MSA_REQUIRE((((uintptr_t)rope_cos | (uintptr_t)rope_sin) & 3) == 0 &&
+                  (((uintptr_t)q_out | (uintptr_t)k_out | (uintptr_t)v_out | (uintptr_t)r_out) & 15) == 0,
+              "msa_qkv_proj: rope tables (fp32 [rope_rows, 64]) 4-byte and outputs 16-byte aligned");
   const int64_t heads = (int64_t)Hq + 2 * Hkv + Hr_front + Hr_back;
   MSA_REQUIRE(heads * kHeadDim < ((int64_t)1 << 20), "msa_qkv_proj: too many heads");
   MSA_REQUIRE((int64_t)BM * K * 2 < ((int64_t)1 << 31), "msa_qkv_proj: K too large");

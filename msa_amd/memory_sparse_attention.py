@@ -125,7 +125,9 @@ class MemorySparseAttention(nn.Module):
         x = hidden_states.reshape(B * S, -1)
         pos = position_ids.reshape(-1).contiguous()
         has_router = self.is_router_layer and self.decouple_router
-        if hidden_states.dtype == torch.bfloat16 and D == 128 and x.shape[1] % 64 == 0:
+        if (hidden_states.dtype == torch.bfloat16 and D == 128 and x.shape[1] % 64 == 0
+                and self.q_norm.weight.dtype == torch.bfloat16 and self.k_norm.weight.dtype == torch.bfloat16
+                and self.q_proj.weight.dtype == torch.bfloat16):
             w_all = self._all_weight(hidden_states.device)
             lo = Hkv * D if has_router else 0                   # rows of router_k_proj in front of q | k | v
             if has_router and router == "k":
@@ -153,11 +155,15 @@ class MemorySparseAttention(nn.Module):
         """[router_k_proj | q_proj | k_proj | v_proj | router_q_proj] rows in one matrix (q | k | v alone on layers
         without a decoupled router): stage 1 multiplies by the first four, stage 2 by the last four, a decode step by
         the middle three, all as contiguous row ranges of this one copy."""
-        if self._qkv_weight is None or self._qkv_weight.device != device:
-            parts = [self.q_proj.weight, self.k_proj.weight, self.v_proj.weight]
-            if self.is_router_layer and self.decouple_router:
-                parts = [self.router_k_proj[0].weight] + parts + [self.router_q_proj[0].weight]
-            self._qkv_weight = torch.cat(parts, dim=0).contiguous()
+        parts = [self.q_proj.weight, self.k_proj.weight, self.v_proj.weight]
+        if self.is_router_layer and self.decouple_router:
+            parts = [self.router_k_proj[0].weight] + parts + [self.router_q_proj[0].weight]
+        # the copy follows its sources: loading a state dict, .to(dtype / device) or an in-place update of any of
+        # them changes the storage pointer, the dtype or the version counter, and the copy is rebuilt
+        key = tuple((w.data_ptr(), w._version, w.dtype, w.device) for w in parts) + (device,)
+        if self._qkv_weight is None or self._qkv_weight_key != key:
+            self._qkv_weight = torch.cat([w.detach().to(device) for w in parts], dim=0).contiguous()
+            self._qkv_weight_key = key
         return self._qkv_weight
 
     def _fused_weight(self, device):

@@ -282,6 +282,24 @@ class Memory:
             files.copy_into(layer, "v", v[layer])
         self.load_pooled(docs, rk, k, v, files.prefix())
 
+    def load_reference_bank(self, path: str, docs: List[Document]) -> None:
+        """Adopts a bank directory written by the reference's ``Memory.serialize`` (src/msa_service.py:351-404):
+        ``layer_<i>_{k,v,rk}.pt`` and ``prefix_cache.pt`` are read as plain tensors (``weights_only=True``) and
+        transposed to chunk-major; ``meta.pt`` pickles Document objects and is not opened, so the documents (ids
+        and chunk counts, bank order) come from the caller.  K_r goes to the device, K / V into pinned host
+        memory, whatever device the reference's own restore would have chosen (:447-461)."""
+        from . import bank_io
+        have = bank_io.reference_bank_layers(path)
+        missing = [l for l in self.router_layer_ids if l not in have]
+        if missing:
+            raise ValueError(f"{path}: no pooled tensors for router layers {missing}")
+        rk, k, v = {}, {}, {}
+        for layer in self.router_layer_ids:
+            r, kk, vv = bank_io.read_reference_layer(path, layer)
+            rk[layer] = r.to(self.device)
+            k[layer], v[layer] = kk.pin_memory(), vv.pin_memory()
+        self.load_pooled(docs, rk, k, v, bank_io.read_reference_prefix(path))
+
     def get_max_local_pool_doc_id(self) -> int:
         return int(self.block_desc.pool_ids_cpu[-1])
 

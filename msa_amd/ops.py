@@ -402,6 +402,17 @@ def qkv_proj(x: torch.Tensor, w: torch.Tensor, Hq: int, Hkv: int, positions: tor
         raise ValueError(f"qkv_proj: x [T, K] and w [{heads * D}, K] in bf16")
     if positions.dtype != torch.int64 or positions.numel() != T:
         raise ValueError("qkv_proj: positions int64 [T]")
+    for name, nw in (("q_norm_w", q_norm_w), ("k_norm_w", k_norm_w)):
+        if nw.dtype != torch.bfloat16 or nw.numel() != D or not nw.is_contiguous():
+            raise ValueError(f"qkv_proj: {name} must be {D} contiguous bf16 weights, got {nw.dtype} x {nw.numel()}")
+    for name, tab in (("cos", rope[0]), ("sin", rope[1])):
+        if tab.dtype != torch.float32 or tab.dim() != 2 or tab.shape[1] != D // 2 or not tab.is_contiguous():
+            raise ValueError(f"qkv_proj: the {name} table must be contiguous fp32 [rows, {D // 2}], got {tab.dtype} "
+                             f"{tuple(tab.shape)}")
+    if rope[0].shape != rope[1].shape:
+        raise ValueError("qkv_proj: cos / sin tables differ in shape")
+    if not (x.is_contiguous() and w.is_contiguous()) or x.data_ptr() % 16 or w.data_ptr() % 16:
+        raise ValueError("qkv_proj: x and w must be contiguous and 16-byte aligned")
     dev = x.device
     q = torch.empty((T, Hq, D), dtype=x.dtype, device=dev)
     k = torch.empty((T, Hkv, D), dtype=x.dtype, device=dev)

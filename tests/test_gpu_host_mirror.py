@@ -213,6 +213,20 @@ def test_layer_stage1_stage2_decode_against_oracle(env):
     pk_b, pv_b = fresh.get_template_prefix_kvcaches(1)
     assert torch.equal(pk_a, pk_b) and torch.equal(pv_a, pv_b)
 
+    # ---- the same bank in the reference's own file layout ([1, Hkv, C, D] tensors, one file each) converts
+    with tempfile.TemporaryDirectory() as tmp:
+        for tag, src in (("rk", service._rk), ("k", service._k), ("v", service._v)):
+            torch.save(src[1].cpu().transpose(0, 1).unsqueeze(0).contiguous(), f"{tmp}/layer_1_{tag}.pt")
+        torch.save({l: (a.cpu(), b.cpu()) for l, (a, b) in service.template_prefix_kvcache.items()},
+                   f"{tmp}/prefix_cache.pt")
+        conv = svc_mod.MSAService(0, env["config"].GenerateConfig(devices=[0]),
+                                  env["config"].ModelConfig(doc_top_k=TOPK, pooling_kernel_size=P, router_layer_idx="1"),
+                                  env["config"].MemoryConfig(pooling_kernel_size=P), env["cfg"])
+        conv.load_reference_bank(tmp, docs)
+    K4, V4, s4, n4, g4 = conv.doc_query(rq, mask.bool().cuda(), 1)
+    assert torch.equal(K4, K) and torch.equal(V4, V) and torch.equal(s4, s2) and torch.equal(g4, g2) and torch.equal(n4, n_sel)
+    assert conv._k[1].is_pinned() and conv._rk[1].is_cuda
+
 
 def test_unsupported_reductions_raise(env):
     say("unsupported reduce methods")

@@ -453,6 +453,30 @@ def test_config1_routing_layer_fp32(ops):
 
 
 # ------------------------------------------------------------------ fused projection GEMM
+def test_qkv_proj_refuses_operands_the_kernel_would_misread(ops):
+    """fp32 norm weights, a rotary table of the wrong width or type, and a misaligned weight view are refused on the
+    host instead of being read as something else."""
+    say("qkv_proj argument checks")
+    D, T, K = 128, 64, 128
+    x = torch.zeros((T, K), dtype=torch.bfloat16, device="cuda")
+    w = torch.zeros((4 * D, K), dtype=torch.bfloat16, device="cuda")
+    pos = torch.zeros(T, dtype=torch.int64, device="cuda")
+    nw = torch.ones(D, dtype=torch.bfloat16, device="cuda")
+    rope = ops.rope_tables(16, D, 1e6)
+    ops.qkv_proj(x, w, 2, 1, pos, nw, nw, 1e-6, rope)
+    with pytest.raises(ValueError, match="q_norm_w"):
+        ops.qkv_proj(x, w, 2, 1, pos, nw.float(), nw, 1e-6, rope)
+    with pytest.raises(ValueError, match="k_norm_w"):
+        ops.qkv_proj(x, w, 2, 1, pos, nw, nw[:64], 1e-6, rope)
+    with pytest.raises(ValueError, match="table"):
+        ops.qkv_proj(x, w, 2, 1, pos, nw, nw, 1e-6, (rope[0].double(), rope[1].double()))
+    with pytest.raises(ValueError, match="table"):
+        ops.qkv_proj(x, w, 2, 1, pos, nw, nw, 1e-6, (rope[0][:, :32].contiguous(), rope[1][:, :32].contiguous()))
+    wide = torch.zeros((4 * D * K + 4,), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError, match="aligned"):
+        ops.qkv_proj(x, wide[4:].view(4 * D, K), 2, 1, pos, nw, nw, 1e-6, rope)
+
+
 @pytest.mark.parametrize("T,K,Hq,Hkv,front,back", [(300, 320, 4, 2, 2, 0), (70, 64, 8, 1, 0, 8), (513, 2560, 32, 8, 8, 0),
                                                     (1000, 2560, 32, 8, 0, 32), (257, 192, 3, 1, 0, 0)])
 def test_qkv_proj_gemm_with_norm_rope_epilogue(ops, T, K, Hq, Hkv, front, back):
@@ -657,3 +681,16 @@ def test_route_topk_gather_equals_the_two_calls(B, S, dtype):
     assert torch.equal(cu_, want_g[2])
     n = int(cu_[-1])
     assert n > 0 and torch.equal(k_[:n], want_g[0][:n]) and torch.equal(v_[:n], want_g[1][:n])
+    # outputs too small for the selection: both forms stop at the capacity (cu_sel clamps there, later rows are
+    # dropped, nothing past the capacity is written), also where a shared document's second use lies past it
+    sel[4, 1] = sel[0, 1]
+    full = ops.gather_kv_device(bank, 0, sel, cap)
+    short = int(full[2][-1]) // 2
+    bufs = [tuple(torch.full((cap, Hkv, D), 7.0, dtype=dtype, device="cuda") for _ in range(2)) for _ in range(2)]
+    want_g = ops.gather_kv_device(bank, 0, sel, short, out=bufs[0])
+    _, (k_, v_, cu_) = ops.route_topk_gather(bank, 1, q, mask.cuda(), "cosine", 1.0, 8, 0, sel, short, out=bufs[1])
+    torch.cuda.synchronize()
+    assert int(cu_[-1]) == short and torch.equal(cu_, want_g[2]) and torch.equal(cu_, full[2].clamp(max=short))
+    for got, alone, whole in ((k_, want_g[0], full[0]), (v_, want_g[1], full[1])):
+        assert torch.equal(got[:short], whole[:short]) and torch.equal(alone[:short], whole[:short])
+        assert (got[short:] == 7.0).all() and (alone[short:] == 7.0).all()

@@ -155,3 +155,64 @@ def test_prefill_worker_block_inputs_and_split():
     assert inp.doc_ids[0, :3].tolist() == [-2, -2, -2] and inp.doc_ids[0, 3:12].tolist() == [1] * 9
     assert inp.position_ids[0, 3:12].tolist() == list(range(9)) and inp.position_ids[0, 12] == 0
     assert inp.chunk_sizes == [2, 2, 1]
+
+
+def test_reference_bank_files_convert_to_the_native_format(tmp_path):
+    """A bank directory in the reference's file layout (tests/golden/make_reference_style_bank.py) is read without
+    its meta.pt, transposed to chunk-major, and converts to the native format bit for bit."""
+    from types import SimpleNamespace
+    from msa_amd import bank_io
+    from tests.golden import make_reference_style_bank as mk
+    src, dst = str(tmp_path / "ref"), str(tmp_path / "native")
+    mk.write(src)
+    layers, prefix = mk.expected()
+    assert bank_io.reference_bank_layers(src) == mk.LAYERS
+    rk, k, v = bank_io.read_reference_layer(src, 19)
+    C = sum(mk.DOC_CHUNKS)
+    assert rk.shape == (C, mk.HKV, mk.D) and rk.is_contiguous()
+    assert torch.equal(rk, layers[19]["rk"][0].transpose(0, 1))
+    assert torch.equal(k[5, 1], layers[19]["k"][0, 1, 5]) and torch.equal(v[2, 0], layers[19]["v"][0, 0, 2])
+    docs = [SimpleNamespace(doc_id=i, num_chunks=n, doc=f"text {i}") for i, n in zip(mk.DOC_IDS, mk.DOC_CHUNKS)]
+    bank_io.convert_reference_bank(src, dst, docs, {"pooling_kernel_size": 64, "aux_loss_method": "INFONCE"})
+    files = bank_io.BankFiles(dst)
+    assert files.header["router_layers"] == mk.LAYERS and files.shape == (C, mk.HKV, mk.D)
+    assert files.doc_chunk_off.tolist() == [0, 3, 4, 8, 10] and files.doc_global_id.tolist() == mk.DOC_IDS
+    for l in mk.LAYERS:
+        for tag in ("rk", "k", "v"):
+            got = torch.empty(files.shape, dtype=torch.bfloat16)
+            files.copy_into(l, tag, got)
+            assert torch.equal(got, layers[l][tag][0].transpose(0, 1))
+    back = files.prefix()
+    assert sorted(back) == sorted(prefix)
+    assert all(torch.equal(back[l][0], prefix[l][0]) and torch.equal(back[l][1], prefix[l][1]) for l in prefix)
+    assert [r["doc"] for r in bank_io.load_docs(dst)] == [d.doc for d in docs]
+    # documents that do not add up to the stored chunks are refused
+    with pytest.raises(ValueError, match="add up"):
+        bank_io.convert_reference_bank(src, str(tmp_path / "bad"), docs[:-1], {})
+
+
+def test_concatenated_projection_weights_follow_their_sources():
+    """The [router_k | q | k | v | router_q] copy the fused projection multiplies by is rebuilt when a source weight
+    is updated in place, replaced by a loaded state dict, or converted to another dtype; otherwise it is reused."""
+    from msa_amd import memory_sparse_attention as msa
+    cfg = mconfig.MSAConfig(hidden_size=64, num_hidden_layers=2, num_attention_heads=2, num_key_value_heads=1, head_dim=128,
+                            intermediate_size=64, vocab_size=50,
+                            msa_config=dict(mconfig.default_msa_config(), router_layer_idx="1"))
+    layer = msa.MemorySparseAttention(cfg, 1)
+    dev = torch.device("cpu")
+
+    def want():
+        return torch.cat([layer.router_k_proj[0].weight, layer.q_proj.weight, layer.k_proj.weight, layer.v_proj.weight,
+                          layer.router_q_proj[0].weight])
+    first = layer._all_weight(dev)
+    assert torch.equal(first, want()) and layer._all_weight(dev) is first
+    with torch.no_grad():
+        layer.k_proj.weight.mul_(2.0)                                     # in-place update (an optimizer step)
+    assert torch.equal(layer._all_weight(dev), want()) and layer._all_weight(dev) is not first
+    state = {k: torch.randn_like(v) for k, v in layer.state_dict().items()}
+    layer.load_state_dict(state)                                          # copy_ into the same storage
+    assert torch.equal(layer._all_weight(dev), want())
+    layer.bfloat16()                                                      # new dtype
+    got = layer._all_weight(dev)
+    assert got.dtype == torch.bfloat16 and torch.equal(got, want())
+    assert torch.equal(layer._fused_weight(dev), torch.cat([layer.q_proj.weight, layer.k_proj.weight, layer.v_proj.weight]))

@@ -281,6 +281,11 @@ int msa_flash_attn(const void* q, const int32_t* cu_q, const void* k, const void
                    const int64_t* kv_off, const int32_t* kv_len, int32_t B, int32_t total_q,
                    int32_t Hq, int32_t Hkv, int32_t D, float scale, int32_t causal, void* out,
                    void* stream);
+/* msa_flash_attn has two forms of its kernel: 32 (token, head) columns per wavefront, two workgroups per compute unit,
+ * and a wide one (64 columns per wavefront, one wavefront per SIMD, the tile step written at the instruction level)
+ * that it picks when the call has at least 4096 columns.  form 0: by size (the default), 1: always the first,
+ * 2: always the wide one.  A test and measurement aid (no counterpart in the reference); process-wide. */
+int msa_flash_set_form(int32_t form);
 
 /* ---------------------------------------------------------------------------------------------
  * Fused helpers around the attention call.  msa_qk_norm_rope replaces q_norm / k_norm + apply_rotary_pos_emb

@@ -42,12 +42,13 @@ def _compile(src: str) -> str:
 #  * score_scan4_kernel (route_score.hip): its asm statements own v128-v255 and all accumulation registers across
 #    statements.  The code the compiler generates for that kernel must therefore stay below v128, touch no
 #    accumulation register (the compiler would only do so to spill), and use no scratch memory.
+#  * flash_wide_kernel (flash_attn.hip): likewise, its statements own v56-v255 and all accumulation registers.
 #  * flash_attn_kernel (flash_attn.hip): its direct-to-LDS loads are asm statements the compiler does not order
 #    against LDS reads; a spill would add vector-memory waits in the middle of that ring.  No scratch, no spills.
 # ---------------------------------------------------------------------------------------------------------------
 CONTRACTS = {
     "route_score.hip": [("score_scan4_kernel", {"max_compiler_vgpr": 127, "no_agpr": True})],
-    "flash_attn.hip": [("flash_attn_kernel", {})],
+    "flash_attn.hip": [("flash_attn_kernel", {}), ("flash_wide_kernel", {"max_compiler_vgpr": 55, "no_agpr": True})],
 }
 
 
@@ -125,9 +126,9 @@ def build(jobs: int = 8) -> str:
     """Compiles every source (always, even if the library exists), checks the inline-asm contracts on the device
     assembly and links the shared library."""
     srcs = sources()
-    gen = os.path.join(CSRC, "gen_scan_asm.py")
-    if subprocess.run([sys.executable, gen, "--check"]).returncode != 0:
-        raise RuntimeError("csrc/scan_asm.inc is not what csrc/gen_scan_asm.py generates: run the generator")
+    for gen, inc in (("gen_scan_asm.py", "scan_asm.inc"), ("gen_flash_asm.py", "flash_asm.inc")):
+        if subprocess.run([sys.executable, os.path.join(CSRC, gen), "--check"]).returncode != 0:
+            raise RuntimeError(f"csrc/{inc} is not what csrc/{gen} generates: run the generator")
     with ThreadPoolExecutor(max_workers=min(jobs, len(srcs) + len(CONTRACTS))) as ex:
         checks = [ex.submit(_check_contracts, s) for s in srcs if os.path.basename(s) in CONTRACTS]
         objs = list(ex.map(_compile, srcs))

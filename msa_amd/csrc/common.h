@@ -41,6 +41,18 @@ static inline hipError_t raise_dynamic_lds_limit(std::atomic<int>& done, const v
   return e;
 }
 
+// Compute units of the current device (asked once; the library drives one device per process).
+static inline int device_compute_units() {
+  static const int n = [] {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+      cus = 256;
+    return cus;
+  }();
+  return n;
+}
+
 typedef uint16_t bf16_t;  // raw bf16 bits
 
 __device__ __forceinline__ float bf16_to_f32(bf16_t x) { return __uint_as_float(((uint32_t)x) << 16); }

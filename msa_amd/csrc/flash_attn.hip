@@ -450,6 +450,305 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The wide form: one wavefront per SIMD, 64 (token, head) columns per wavefront, 256 per workgroup; the tile step is
+// written at the instruction level (flash_asm.inc, generated by gen_flash_asm.py, which describes the schedule, the
+// LDS rings and the registers the statements own: v56 - v255, every accumulation register, s84 - s95).  The code the
+// compiler allocates stays below v56 (amdgpu_num_vgpr) and only names values for the statements: tile resources,
+// the masked-or-not choice per tile, the rescale of O when a reference maximum moved.
+#include "flash_asm.inc"
+
+constexpr int kWideLdsBytes = 6 * kTileBytes;   // rings of three K and three V tiles
+constexpr int kWideCompilerVgprs = 56;
+
+#define FLASHW_ASM(TEXT) asm volatile(TEXT ::: FLASHW_CLOBBERS)
+#define FLASHW_SETQ(CB, KS, W) \
+  asm volatile(FLASHW_SET_Q##CB##_##KS ::"v"((W).x), "v"((W).y), "v"((W).z), "v"((W).w) : FLASHW_CLOBBERS)
+#define FLASHW_GETO(CB, D, X)                                                                                          \
+  asm volatile(FLASHW_GET_O##CB##_##D                                                                                  \
+               : "=v"((X)[0]), "=v"((X)[1]), "=v"((X)[2]), "=v"((X)[3]), "=v"((X)[4]), "=v"((X)[5]), "=v"((X)[6]),     \
+                 "=v"((X)[7]), "=v"((X)[8]), "=v"((X)[9]), "=v"((X)[10]), "=v"((X)[11]), "=v"((X)[12]), "=v"((X)[13]), \
+                 "=v"((X)[14]), "=v"((X)[15]))
+
+// The launch is persistent: one workgroup per compute unit walks the token blocks of its KV head (workgroup w serves
+// head w % Hkv, so with eight heads a head keeps to one XCD and its K / V to that XCD's L2, and is the (w / Hkv)-th of
+// the n workgroups of the head).  A head's blocks are listed sample by sample, under the causal mask a sample's late
+// (long) blocks first, and dealt out in rounds of n that alternate direction: workgroup c takes position c of an even
+// round and n - 1 - c of an odd one, so the workgroup that drew the longest block of a round draws the shortest of the
+// next (a sample of 2 n causal blocks splits evenly), and the n workgroups stay on the same sample's K / V.
+template <int G>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kWideCompilerVgprs))) void flash_wide_kernel(
+    const bf16_t* __restrict__ q, const int32_t* __restrict__ cu_q, const bf16_t* __restrict__ k,
+    const bf16_t* __restrict__ v, const int64_t* __restrict__ kv_off, const int32_t* __restrict__ kv_len, int32_t B,
+    int32_t Hq, int32_t Hkv, float scale_log2e, int32_t causal, bf16_t* __restrict__ out, int32_t total_blocks) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  constexpr int kTokPerWave = 64 / G;
+  constexpr int kTokPerBlock = 4 * kTokPerWave;
+  extern __shared__ __align__(16) char lds[];
+
+  const int g = blockIdx.x % Hkv, c_wg = blockIdx.x / Hkv, n_wg = gridDim.x / Hkv;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, half = lane >> 5;
+  const int row_elems = Hkv * kHeadDim;
+  const int row_bytes = row_elems * 2;
+
+  // per-lane LDS read positions (slot 0) and global offsets of the wavefront's four 1 KB blocks of a tile: the same
+  // row / piece assignment and swizzles as the 32-column form
+  {
+    int k_at[8], v_at[4];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) k_at[ks] = l32 * kRowBytes + (((2 * ks + half) ^ (l32 & 15)) * 16);
+    const int r = (lane & 15) >> 2;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+      v_at[d] = 3 * kTileBytes + (4 * half + r) * kRowBytes + ((d ^ r) * 64) + (lane & 16) * 2 + (lane & 3) * 8;
+    asm volatile(FLASHW_SET_KAT ::"v"(k_at[0]), "v"(k_at[1]), "v"(k_at[2]), "v"(k_at[3]), "v"(k_at[4]), "v"(k_at[5]),
+                 "v"(k_at[6]), "v"(k_at[7])
+                 : FLASHW_CLOBBERS);
+    asm volatile(FLASHW_SET_VAT ::"v"(v_at[0]), "v"(v_at[1]), "v"(v_at[2]), "v"(v_at[3]) : FLASHW_CLOBBERS);
+    int koff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 4 * (4 * wave + i) + (lane >> 4);
+      koff[i] = row * row_bytes + ((lane & 15) ^ (row & 15)) * 16;
+    }
+    asm volatile(FLASHW_SET_KOFF ::"v"(koff[0]), "v"(koff[1]), "v"(koff[2]), "v"(koff[3]) : FLASHW_CLOBBERS);
+  }
+  const int tile_row0 = 16 * wave + (lane >> 4);               // the lane's row in the wavefront's first block; + 4 i
+  const int v_piece = ((lane & 15) ^ ((tile_row0 & 3) << 2)) * 16;   // (the same for the four blocks: rows 4 apart)
+  const uint32_t ldsw = lds_address(lds) + 4 * wave * 1024;     // this wavefront's first block of ring slot 0
+
+  for (int round = 0; round * n_wg < total_blocks; ++round) {
+    int blk = round * n_wg + ((round & 1) ? n_wg - 1 - c_wg : c_wg);
+    int b = 0;
+    bool found = false;
+    for (; b < B; ++b) {
+      const int sq_b = cu_q ? cu_q[b + 1] - cu_q[b] : 1;
+      const int nb = (sq_b + kTokPerBlock - 1) / kTokPerBlock;
+      if (blk < nb) {
+        if (causal) blk = nb - 1 - blk;
+        found = true;
+        break;
+      }
+      blk -= nb;
+    }
+    if (!found) continue;
+    const int q_first = cu_q ? cu_q[b] : b;
+    const int sq = cu_q ? cu_q[b + 1] - q_first : 1;
+    const int t0 = blk * kTokPerBlock;
+    const int L = kv_len[b];
+    const int64_t base = kv_off[b];
+
+    int tok[2], head[2], limit[2];
+    bool col_ok[2];
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+      const int col = 32 * cb + l32;
+      tok[cb] = t0 + wave * kTokPerWave + col / G;
+      head[cb] = g * G + col % G;
+      col_ok[cb] = tok[cb] < sq;
+      limit[cb] = col_ok[cb] ? (causal ? max(0, L - sq + tok[cb] + 1) : L) : 0;
+    }
+    const int last_tok = min(sq, t0 + kTokPerBlock) - 1;
+    const int kmax = causal ? max(0, min(L, L - sq + last_tok + 1)) : L;
+    const int n_tiles = (kmax + kKeysPerTile - 1) / kKeysPerTile;
+    asm volatile(FLASHW_SET_LIMIT ::"v"(limit[0] - 4 * half), "v"(limit[1] - 4 * half) : FLASHW_CLOBBERS);
+    int wave_min_limit = min(limit[0], limit[1]);
+#pragma unroll
+    for (int x = 32; x > 0; x >>= 1) wave_min_limit = min(wave_min_limit, __shfl_xor(wave_min_limit, x));
+    wave_min_limit = __builtin_amdgcn_readfirstlane(wave_min_limit);
+
+    struct TilePos { uintptr_t at; int left; };
+    auto first_pos = [&](const bf16_t* src) {
+      return TilePos{reinterpret_cast<uintptr_t>(src) + (base * row_elems + g * kHeadDim) * 2, kmax};
+    };
+    TilePos k_pos = first_pos(k), v_pos = first_pos(v);
+    auto tile_rsrc = [&](TilePos& p, int& rows) -> u32x4_t {
+      rows = min(kKeysPerTile, p.left);
+      const u32x4_t r = {(uint32_t)p.at, (uint32_t)(p.at >> 32) & 0xffffu,
+                         (uint32_t)max(0, (rows - 1) * row_bytes + kRowBytes), 0x00020000u};
+      p.at += (uintptr_t)kKeysPerTile * row_bytes;
+      p.left -= kKeysPerTile;
+      return r;
+    };
+    // the next V tile's resource; a last tile of fewer than 64 keys has its missing rows fetched from its last key
+    // (they meet probabilities of zero and must be finite), which is the last change the block's V offsets see
+    auto set_voff = [&](int rows) {
+      int vo[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) vo[i] = min(tile_row0 + 4 * i, rows - 1) * row_bytes + v_piece;
+      asm volatile(FLASHW_SET_VOFF ::"v"(vo[0]), "v"(vo[1]), "v"(vo[2]), "v"(vo[3]) : FLASHW_CLOBBERS);
+    };
+    auto next_v = [&]() -> u32x4_t {
+      int rows;
+      const u32x4_t r = tile_rsrc(v_pos, rows);
+      if (rows > 0 && rows < kKeysPerTile) set_voff(rows);
+      return r;
+    };
+    auto next_k = [&]() -> u32x4_t {
+      int rows;
+      return tile_rsrc(k_pos, rows);
+    };
+    set_voff(kKeysPerTile);
+
+    if (n_tiles > 0) {
+      // K(0), K(1), V(0), K(2), V(1): the order the steps' waits count on
+      u32x4_t r = next_k();
+      asm volatile(FLASHW_LOAD4_K ::[dst] "s"(ldsw), [r] "s"(r) : FLASHW_CLOBBERS);
+      r = next_k();
+      asm volatile(FLASHW_LOAD4_K ::[dst] "s"(ldsw + kTileBytes), [r] "s"(r) : FLASHW_CLOBBERS);
+      r = next_v();
+      asm volatile(FLASHW_LOAD4_V ::[dst] "s"(ldsw + 3 * kTileBytes), [r] "s"(r) : FLASHW_CLOBBERS);
+      r = next_k();
+      asm volatile(FLASHW_LOAD4_K ::[dst] "s"(ldsw + 2 * kTileBytes), [r] "s"(r) : FLASHW_CLOBBERS);
+      r = next_v();
+      asm volatile(FLASHW_LOAD4_V ::[dst] "s"(ldsw + 4 * kTileBytes), [r] "s"(r) : FLASHW_CLOBBERS);
+    }
+    // Q^T operand fragments into the accumulation registers they stay in, behind the tile loads so that their
+    // latency runs under the tiles': eight 16-byte loads in flight per column block
+#define FLASHW_LOADQ(CB)                                                                                             \
+  {                                                                                                                  \
+    const bf16_t* qrow = q + ((int64_t)(q_first + (col_ok[CB] ? tok[CB] : 0)) * Hq + head[CB]) * kHeadDim + 8 * half; \
+    uint4 w[8];                                                                                                      \
+    _Pragma("unroll") for (int ks = 0; ks < 8; ++ks)                                                                 \
+        w[ks] = col_ok[CB] ? *reinterpret_cast<const uint4*>(qrow + 16 * ks) : make_uint4(0, 0, 0, 0);               \
+    FLASHW_SETQ(CB, 0, w[0]); FLASHW_SETQ(CB, 1, w[1]); FLASHW_SETQ(CB, 2, w[2]); FLASHW_SETQ(CB, 3, w[3]);          \
+    FLASHW_SETQ(CB, 4, w[4]); FLASHW_SETQ(CB, 5, w[5]); FLASHW_SETQ(CB, 6, w[6]); FLASHW_SETQ(CB, 7, w[7]);          \
+  }
+    FLASHW_LOADQ(0)
+    FLASHW_LOADQ(1)
+#undef FLASHW_LOADQ
+    FLASHW_ASM(FLASHW_INIT);
+
+    if (n_tiles > 0) {
+      asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
+      FLASHW_ASM(FLASHW_QK_FIRST);
+
+      // The statements repeat with period six (LDS slots and score buffers are immediates), so the loop over the
+      // tiles is unrolled by six; tile 0 (nothing to multiply by V yet) stands in front.
+      int t = 0, flag;
+#define FLASHW_HALF_A(TEXT) asm volatile(TEXT : [flag] "=&s"(flag) : [c] "s"(scale_log2e) : FLASHW_CLOBBERS)
+#define FLASHW_STEP(A_TEXT, A_TEXT_M, B_TEXT, B_TEXT_LAST)                                                          \
+  {                                                                                                                 \
+    if ((t + 1) * kKeysPerTile > wave_min_limit) {                                                                  \
+      asm volatile(A_TEXT_M : [flag] "=&s"(flag) : [c] "s"(scale_log2e), [t64] "s"(t * kKeysPerTile) : FLASHW_CLOBBERS); \
+    } else {                                                                                                        \
+      FLASHW_HALF_A(A_TEXT);                                                                                        \
+    }                                                                                                               \
+    if (flag) FLASHW_ASM(FLASHW_RESCALE);                                                                           \
+    if (++t < n_tiles) {                                                                                            \
+      const u32x4_t rk = next_k();                                                                                  \
+      const u32x4_t rv = next_v();                                                                                  \
+      asm volatile(B_TEXT ::[c] "s"(scale_log2e), [rk] "s"(rk), [rv] "s"(rv), [ldsw] "s"(ldsw) : FLASHW_CLOBBERS);  \
+    } else {                                                                                                        \
+      asm volatile(B_TEXT_LAST ::[c] "s"(scale_log2e) : FLASHW_CLOBBERS);                                           \
+      break;                                                                                                        \
+    }                                                                                                               \
+  }
+      do {
+        FLASHW_STEP(FLASHW_A_FIRST, FLASHW_A_FIRST_M, FLASHW_B0, FLASHW_B0_LAST)
+        for (;;) {
+          FLASHW_STEP(FLASHW_A1, FLASHW_A1_M, FLASHW_B1, FLASHW_B1_LAST)
+          FLASHW_STEP(FLASHW_A2, FLASHW_A2_M, FLASHW_B2, FLASHW_B2_LAST)
+          FLASHW_STEP(FLASHW_A3, FLASHW_A3_M, FLASHW_B3, FLASHW_B3_LAST)
+          FLASHW_STEP(FLASHW_A4, FLASHW_A4_M, FLASHW_B4, FLASHW_B4_LAST)
+          FLASHW_STEP(FLASHW_A5, FLASHW_A5_M, FLASHW_B5, FLASHW_B5_LAST)
+          FLASHW_STEP(FLASHW_A0, FLASHW_A0_M, FLASHW_B0, FLASHW_B0_LAST)
+        }
+      } while (false);
+#undef FLASHW_STEP
+#undef FLASHW_HALF_A
+      const int i = t % 6;                      // of the tile behind the last: its half A alone is left (O += V^T . P^T)
+      switch (i) {
+        case 0: FLASHW_ASM(FLASHW_PV0); break;
+        case 1: FLASHW_ASM(FLASHW_PV1); break;
+        case 2: FLASHW_ASM(FLASHW_PV2); break;
+        case 3: FLASHW_ASM(FLASHW_PV3); break;
+        case 4: FLASHW_ASM(FLASHW_PV4); break;
+        case 5: FLASHW_ASM(FLASHW_PV5); break;
+      }
+      FLASHW_ASM(FLASHW_DRAIN);
+      // nothing may still be writing LDS, and every wavefront must be done reading it, when the next block's tiles
+      // are requested (or the workgroup ends)
+      asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    }
+
+    float m0, m1, lsum[2];
+    asm volatile(FLASHW_GET_ML : "=v"(m0), "=v"(m1), "=v"(lsum[0]), "=v"(lsum[1]));
+    (void)m0; (void)m1;
+    // the columns' rows again, from the lane id (nothing per lane is kept in registers across the tile loop)
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int half_e = lane_e >> 5;
+    int64_t orow_e[2];
+    bool ok_e[2];
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+      const int col = 32 * cb + (lane_e & 31);
+      const int tk = t0 + wave * kTokPerWave + col / G;
+      ok_e[cb] = tk < sq;
+      orow_e[cb] = ((int64_t)(q_first + tk) * Hq + g * G + col % G) * kHeadDim + 4 * half_e;
+    }
+#define FLASHW_STORE(CB, D)                                                                              \
+  {                                                                                                      \
+    float x[16];                                                                                         \
+    FLASHW_GETO(CB, D, x);                                                                               \
+    if (ok_e[CB]) {                                                                                      \
+      bf16_t* orow = out + orow_e[CB];                                                                   \
+      _Pragma("unroll") for (int e4 = 0; e4 < 4; ++e4) {                                                 \
+        uint2 w;                                                                                         \
+        w.x = pack_bf16x2(x[4 * e4] * inv[CB], x[4 * e4 + 1] * inv[CB]);                                 \
+        w.y = pack_bf16x2(x[4 * e4 + 2] * inv[CB], x[4 * e4 + 3] * inv[CB]);                             \
+        *reinterpret_cast<uint2*>(orow + 32 * D + 8 * e4) = w;                                           \
+      }                                                                                                  \
+    }                                                                                                    \
+  }
+    float inv[2];
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+      const float l = half_wave_sum(lsum[cb]);
+      inv[cb] = l > 0.f ? 1.0f / l : 0.f;        // a row that sees no key yields zeros
+    }
+    FLASHW_STORE(0, 0) FLASHW_STORE(0, 1) FLASHW_STORE(0, 2) FLASHW_STORE(0, 3)
+    FLASHW_STORE(1, 0) FLASHW_STORE(1, 1) FLASHW_STORE(1, 2) FLASHW_STORE(1, 3)
+#undef FLASHW_STORE
+  }
+#endif
+}
+
+template <int G>
+int flash_wide_launch_g(const void* q, const int32_t* cu_q, const void* k, const void* v, const int64_t* kv_off,
+                        const int32_t* kv_len, int32_t B, int32_t total_q, int32_t Hq, int32_t Hkv, float scale,
+                        int32_t causal, void* out, hipStream_t st) {
+  constexpr int kTokPerBlock = 4 * 64 / G;
+  const int64_t blocks = ((int64_t)total_q + kTokPerBlock - 1) / kTokPerBlock + B;   // upper bound over ragged samples
+  MSA_REQUIRE(blocks < (int64_t)1 << 30, "flash attention: too many query rows");
+  // one workgroup per compute unit, the same number for every KV head
+  const int per_head = (int)std::min<int64_t>(blocks, std::max(1, device_compute_units() / Hkv));
+  auto kern = flash_wide_kernel<G>;
+  static std::atomic<int> lds_limit_raised{0};
+  MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(kern), kWideLdsBytes));
+  kern<<<dim3((unsigned)(per_head * Hkv)), 256, kWideLdsBytes, st>>>(
+      static_cast<const bf16_t*>(q), cu_q, static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v), kv_off, kv_len,
+      B, Hq, Hkv, scale * 1.4426950408889634f, causal, static_cast<bf16_t*>(out), (int32_t)blocks);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
+
+template <typename... Args>
+int flash_wide_launch(int G, Args... args) {
+  switch (G) {
+    case 1: return flash_wide_launch_g<1>(args...);
+    case 2: return flash_wide_launch_g<2>(args...);
+    case 4: return flash_wide_launch_g<4>(args...);
+    case 8: return flash_wide_launch_g<8>(args...);
+  }
+  msa_set_error("flash attention: GQA group size %d unsupported (1, 2, 4, 8)", G);
+  return MSA_EINVAL;
+}
+
+std::atomic<int> g_flash_form{0};   // 0: by size, 1: the 32-column form, 2: the wide form
+
 template <int G, bool kSplit>
 int flash_launch_g(const void* q, const int32_t* cu_q, const void* k, const void* v, const int64_t* kv_off,
                    const int32_t* kv_len, int32_t B, int32_t total_q, int32_t Hq, int32_t Hkv, float scale,
@@ -496,8 +795,18 @@ extern "C" int msa_flash_attn(const void* q, const int32_t* cu_q, const void* k,
               "msa_flash_attn: q, k, v and out must be 16-byte aligned");
   const int G = Hq / Hkv;
   MSA_REQUIRE(G == 1 || G == 2 || G == 4 || G == 8, "msa_flash_attn: GQA group size %d unsupported (1, 2, 4, 8)", G);
+  // the wide form wants enough columns to fill its 256-column workgroups
+  const int form = g_flash_form.load(std::memory_order_relaxed);
+  if (form == 2 || (form == 0 && (int64_t)total_q * G >= 4096))
+    return flash_wide_launch(G, q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale, causal, out, as_stream(stream));
   return flash_launch<false>(G, q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, scale,
                              causal, out, SplitPlan{1, 0}, (float*)nullptr, (float*)nullptr, as_stream(stream));
+}
+
+extern "C" int msa_flash_set_form(int32_t form) {
+  MSA_REQUIRE(form >= 0 && form <= 2, "msa_flash_set_form: 0 (by size), 1 (32-column form) or 2 (wide form)");
+  g_flash_form.store(form, std::memory_order_relaxed);
+  return MSA_OK;
 }
 
 int flash_attn_split_launch(const void* q, const int32_t* cu_q, const void* k, const void* v, const int64_t* kv_off,

@@ -304,17 +304,28 @@ def test_rmsnorm_and_silu_mul_widths(ops, dtype, H):
     assert cf.rel_err(ops.silu_mul(gu.cuda()).cpu(), want) < tol
 
 
+@pytest.fixture(params=[1, 2], ids=["columns32", "wide"])
+def flash_form(request):
+    """Runs a test once per form of the flash kernel (see msa_flash_set_form), and puts the choice by size back."""
+    from msa_amd import _lib
+    lib = _lib.load()
+    _lib.check(lib.msa_flash_set_form(request.param), "msa_flash_set_form")
+    yield request.param
+    _lib.check(lib.msa_flash_set_form(0), "msa_flash_set_form")
+
+
 @pytest.mark.parametrize("Hq,Hkv", [(32, 8), (8, 8), (16, 8), (16, 2), (6, 3)])
 @pytest.mark.parametrize("causal", [True, False])
-def test_flash_kernel_through_the_c_abi(ops, Hq, Hkv, causal):
-    """msa_flash_attn called directly (the host wrapper only picks it for large batches): every tile count parity of
-    its two-tile pipeline (1, 2, 3, 4, 7, 16 tiles of 64 keys), a sample without keys, a causal sample with more
-    query rows than keys (the leading rows see nothing and come out as zeros), single-row and ragged query blocks."""
-    say(f"flash kernel direct Hq={Hq} Hkv={Hkv} causal={causal}")
+def test_flash_kernel_through_the_c_abi(ops, Hq, Hkv, causal, flash_form):
+    """msa_flash_attn called directly (the host wrapper only picks it for large batches), both forms of its kernel:
+    every position of the tile pipelines (1, 2, 3, 4, 7, 16 tiles of 64 keys; the wide form's statements repeat every
+    six tiles), a sample without keys, a causal sample with more query rows than keys (the leading rows see nothing
+    and come out as zeros), single-row and ragged query blocks."""
+    say(f"flash kernel direct Hq={Hq} Hkv={Hkv} causal={causal} form={flash_form}")
     from msa_amd import _lib
     D = 128
-    sq = [130, 1, 33, 64, 200, 5, 7, 40]
-    L = [400, 70, 33, 1000, 200, 192, 0, 10]
+    sq = [130, 1, 33, 64, 200, 5, 7, 40, 300]
+    L = [400, 70, 33, 1000, 200, 192, 0, 10, 777]
     cu_q = np.concatenate([[0], np.cumsum(sq)])
     cu_kv = np.concatenate([[0], np.cumsum(L)])
     q = _randn((int(cu_q[-1]), Hq, D), 300, torch.bfloat16)
@@ -343,12 +354,12 @@ def test_flash_kernel_through_the_c_abi(ops, Hq, Hkv, causal):
 
 
 @pytest.mark.parametrize("causal", [True, False])
-def test_flash_kernel_ignores_stale_lds(ops, causal):
+def test_flash_kernel_ignores_stale_lds(ops, causal, flash_form):
     """The flash kernel's K / V tiles arrive in LDS by direct loads; rows past a sample's last key are not loaded.
     With every compute unit's LDS filled with NaN patterns beforehand (LDS is not cleared between kernels), ragged
     samples whose last tile is partly or almost wholly empty must still give the oracle's result: scores of rows that
     were not loaded are masked by a select, and V rows that were not loaded are never multiplied (0 x NaN)."""
-    say(f"flash kernel after an LDS fill of NaNs causal={causal}")
+    say(f"flash kernel after an LDS fill of NaNs causal={causal} form={flash_form}")
     import ctypes as C
     from msa_amd import _lib
     lib = _lib.load()

@@ -458,12 +458,10 @@ __global__ __launch_bounds__(kWaves * 64, 2) void flash_attn_kernel(
 // the masked-or-not choice per tile, the rescale of O when a reference maximum moved.
 #include "flash_asm.inc"
 
-constexpr int kWideLdsBytes = 6 * kTileBytes;   // rings of three K and three V tiles
+constexpr int kWideLdsBytes = 10 * kTileBytes;  // rings of three K and three V tiles, 16 KB of query rows per wavefront
 constexpr int kWideCompilerVgprs = 56;
 
 #define FLASHW_ASM(TEXT) asm volatile(TEXT ::: FLASHW_CLOBBERS)
-#define FLASHW_SETQ(CB, KS, W) \
-  asm volatile(FLASHW_SET_Q##CB##_##KS ::"v"((W).x), "v"((W).y), "v"((W).z), "v"((W).w) : FLASHW_CLOBBERS)
 #define FLASHW_GETO(CB, D, X)                                                                                          \
   asm volatile(FLASHW_GET_O##CB##_##D                                                                                  \
                : "=v"((X)[0]), "=v"((X)[1]), "=v"((X)[2]), "=v"((X)[3]), "=v"((X)[4]), "=v"((X)[5]), "=v"((X)[6]),     \
@@ -476,6 +474,9 @@ constexpr int kWideCompilerVgprs = 56;
 // (long) blocks first, and dealt out in rounds of n that alternate direction: workgroup c takes position c of an even
 // round and n - 1 - c of an odd one, so the workgroup that drew the longest block of a round draws the shortest of the
 // next (a sample of 2 n causal blocks splits evenly), and the n workgroups stay on the same sample's K / V.
+// Blocks are pipelined: once a block's last product is issued its LDS rings are free, so the next block's first tiles
+// and its query rows (into 16 KB of LDS per wavefront behind the rings) are requested before the finished block's
+// output is scaled and stored, and the block after that is looked up while those loads are awaited.
 template <int G>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kWideCompilerVgprs))) void flash_wide_kernel(
     const bf16_t* __restrict__ q, const int32_t* __restrict__ cu_q, const bf16_t* __restrict__ k,
@@ -488,13 +489,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kWideCompilerVg
 
   const int g = blockIdx.x % Hkv, c_wg = blockIdx.x / Hkv, n_wg = gridDim.x / Hkv;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int l32 = lane & 31, half = lane >> 5;
   const int row_elems = Hkv * kHeadDim;
   const int row_bytes = row_elems * 2;
 
   // per-lane LDS read positions (slot 0) and global offsets of the wavefront's four 1 KB blocks of a tile: the same
   // row / piece assignment and swizzles as the 32-column form
   {
+    const int l32 = lane & 31, half = lane >> 5;
     int k_at[8], v_at[4];
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) k_at[ks] = l32 * kRowBytes + (((2 * ks + half) ^ (l32 & 15)) * 16);
@@ -514,85 +515,108 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kWideCompilerVg
     }
     asm volatile(FLASHW_SET_KOFF ::"v"(koff[0]), "v"(koff[1]), "v"(koff[2]), "v"(koff[3]) : FLASHW_CLOBBERS);
   }
-  const int tile_row0 = 16 * wave + (lane >> 4);               // the lane's row in the wavefront's first block; + 4 i
-  const int v_piece = ((lane & 15) ^ ((tile_row0 & 3) << 2)) * 16;   // (the same for the four blocks: rows 4 apart)
-  const uint32_t ldsw = lds_address(lds) + 4 * wave * 1024;     // this wavefront's first block of ring slot 0
+  const uint32_t ldsw = lds_address(lds) + 4 * wave * 1024;                    // this wavefront's first block of ring slot 0
+  const uint32_t ldsq = lds_address(lds) + 6 * kTileBytes + wave * kTileBytes;  // its query rows
 
-  for (int round = 0; round * n_wg < total_blocks; ++round) {
-    int blk = round * n_wg + ((round & 1) ? n_wg - 1 - c_wg : c_wg);
-    int b = 0;
-    bool found = false;
-    for (; b < B; ++b) {
-      const int sq_b = cu_q ? cu_q[b + 1] - cu_q[b] : 1;
-      const int nb = (sq_b + kTokPerBlock - 1) / kTokPerBlock;
-      if (blk < nb) {
-        if (causal) blk = nb - 1 - blk;
-        found = true;
-        break;
+  // a block of the walk: everything that names it is wave-uniform
+  struct Block {
+    int q_first, sq, t0, kmax, n_tiles, L;
+    int64_t base;
+  };
+  // (a workgroup's positions in the list only grow, so the search for a position's sample resumes where the last
+  // one ended: `cur_b` is a sample, `before` the number of blocks of the samples in front of it)
+  int cur_b = 0, before = 0;
+  auto find_block = [&](int& round, Block& blkout) -> bool {
+    for (; round * n_wg < total_blocks; ++round) {
+      const int pos = round * n_wg + ((round & 1) ? n_wg - 1 - c_wg : c_wg);
+      for (; cur_b < B; ++cur_b) {
+        const int first = cu_q ? cu_q[cur_b] : cur_b;
+        const int sq_b = cu_q ? cu_q[cur_b + 1] - first : 1;
+        const int nb = (sq_b + kTokPerBlock - 1) / kTokPerBlock;
+        if (pos - before < nb) {
+          int blk = pos - before;
+          if (causal) blk = nb - 1 - blk;
+          blkout.q_first = first;
+          blkout.sq = sq_b;
+          blkout.t0 = blk * kTokPerBlock;
+          blkout.L = kv_len[cur_b];
+          blkout.base = kv_off[cur_b];
+          const int last_tok = min(sq_b, blkout.t0 + kTokPerBlock) - 1;
+          blkout.kmax = causal ? max(0, min(blkout.L, blkout.L - sq_b + last_tok + 1)) : blkout.L;
+          blkout.n_tiles = (blkout.kmax + kKeysPerTile - 1) / kKeysPerTile;
+          ++round;
+          return true;
+        }
+        before += nb;
       }
-      blk -= nb;
     }
-    if (!found) continue;
-    const int q_first = cu_q ? cu_q[b] : b;
-    const int sq = cu_q ? cu_q[b + 1] - q_first : 1;
-    const int t0 = blk * kTokPerBlock;
-    const int L = kv_len[b];
-    const int64_t base = kv_off[b];
+    return false;
+  };
 
-    int tok[2], head[2], limit[2];
-    bool col_ok[2];
+  // running positions of the K and V tile streams of the block whose tiles are being loaded
+  struct TilePos { uintptr_t at; int left; };
+  TilePos k_pos{0, 0}, v_pos{0, 0};
+  auto tile_rsrc = [&](TilePos& p, int& rows) -> u32x4_t {
+    rows = min(kKeysPerTile, p.left);
+    const u32x4_t r = {(uint32_t)p.at, (uint32_t)(p.at >> 32) & 0xffffu,
+                       (uint32_t)max(0, (rows - 1) * row_bytes + kRowBytes), 0x00020000u};
+    p.at += (uintptr_t)kKeysPerTile * row_bytes;
+    p.left -= kKeysPerTile;
+    return r;
+  };
+  // the V offsets of a tile of `rows` keys: a last tile of fewer than 64 keys has its missing rows fetched from its
+  // last key (they meet probabilities of zero and must be finite), which is the last change a block's offsets see
+  auto set_voff = [&](int rows) {
+    int lane_v = lane;
+    asm volatile("" : "+v"(lane_v));
+    const int row0 = 16 * wave + (lane_v >> 4);                          // the lane's row in the first block; + 4 i
+    const int piece = ((lane_v & 15) ^ ((row0 & 3) << 2)) * 16;          // (the same for the four blocks)
+    int vo[4];
 #pragma unroll
-    for (int cb = 0; cb < 2; ++cb) {
-      const int col = 32 * cb + l32;
-      tok[cb] = t0 + wave * kTokPerWave + col / G;
-      head[cb] = g * G + col % G;
-      col_ok[cb] = tok[cb] < sq;
-      limit[cb] = col_ok[cb] ? (causal ? max(0, L - sq + tok[cb] + 1) : L) : 0;
+    for (int i = 0; i < 4; ++i) vo[i] = min(row0 + 4 * i, rows - 1) * row_bytes + piece;
+    asm volatile(FLASHW_SET_VOFF ::"v"(vo[0]), "v"(vo[1]), "v"(vo[2]), "v"(vo[3]) : FLASHW_CLOBBERS);
+  };
+  auto next_v = [&]() -> u32x4_t {
+    int rows;
+    const u32x4_t r = tile_rsrc(v_pos, rows);
+    if (rows > 0 && rows < kKeysPerTile) set_voff(rows);
+    return r;
+  };
+  auto next_k = [&]() -> u32x4_t {
+    int rows;
+    return tile_rsrc(k_pos, rows);
+  };
+  // requests a block's query rows and its first tiles (K(0), K(1), V(0), K(2), V(1): the order the steps' waits count
+  // on); every wavefront must be done with the LDS rings
+  auto request_block = [&](const Block& nb) {
+    {
+      // the wavefront's 64 columns are 16 blocks of four rows; a buffer resource over the sample's query rows
+      const uintptr_t qa = reinterpret_cast<uintptr_t>(q) + (uintptr_t)nb.q_first * Hq * kRowBytes;
+      const u32x4_t rq = {(uint32_t)qa, (uint32_t)(qa >> 32) & 0xffffu, (uint32_t)min((int64_t)nb.sq * Hq * kRowBytes, (int64_t)0xffffff00),
+                          0x00020000u};
+      int lane_q = lane;
+      asm volatile("" : "+v"(lane_q));
+#pragma unroll
+      for (int j4 = 0; j4 < 4; ++j4) {
+        int qo[4];
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const int col = 4 * (4 * j4 + jj) + (lane_q >> 4);            // of the wavefront's 64
+          const int tok = nb.t0 + wave * kTokPerWave + col / G;
+          const int piece = (lane_q & 15) ^ (col & 15);
+          // a column past the sample's rows reads from beyond the extent (nothing is fetched; the column is masked)
+          qo[jj] = tok < nb.sq ? (tok * Hq + g * G + col % G) * kRowBytes + piece * 16 : -16;
+        }
+        asm volatile(FLASHW_LOADQ4 ::[dst] "s"(ldsq + j4 * 4096), [r] "s"(rq), [o0] "v"(qo[0]), [o1] "v"(qo[1]),
+                     [o2] "v"(qo[2]), [o3] "v"(qo[3])
+                     : FLASHW_CLOBBERS);
+      }
     }
-    const int last_tok = min(sq, t0 + kTokPerBlock) - 1;
-    const int kmax = causal ? max(0, min(L, L - sq + last_tok + 1)) : L;
-    const int n_tiles = (kmax + kKeysPerTile - 1) / kKeysPerTile;
-    asm volatile(FLASHW_SET_LIMIT ::"v"(limit[0] - 4 * half), "v"(limit[1] - 4 * half) : FLASHW_CLOBBERS);
-    int wave_min_limit = min(limit[0], limit[1]);
-#pragma unroll
-    for (int x = 32; x > 0; x >>= 1) wave_min_limit = min(wave_min_limit, __shfl_xor(wave_min_limit, x));
-    wave_min_limit = __builtin_amdgcn_readfirstlane(wave_min_limit);
-
-    struct TilePos { uintptr_t at; int left; };
-    auto first_pos = [&](const bf16_t* src) {
-      return TilePos{reinterpret_cast<uintptr_t>(src) + (base * row_elems + g * kHeadDim) * 2, kmax};
-    };
-    TilePos k_pos = first_pos(k), v_pos = first_pos(v);
-    auto tile_rsrc = [&](TilePos& p, int& rows) -> u32x4_t {
-      rows = min(kKeysPerTile, p.left);
-      const u32x4_t r = {(uint32_t)p.at, (uint32_t)(p.at >> 32) & 0xffffu,
-                         (uint32_t)max(0, (rows - 1) * row_bytes + kRowBytes), 0x00020000u};
-      p.at += (uintptr_t)kKeysPerTile * row_bytes;
-      p.left -= kKeysPerTile;
-      return r;
-    };
-    // the next V tile's resource; a last tile of fewer than 64 keys has its missing rows fetched from its last key
-    // (they meet probabilities of zero and must be finite), which is the last change the block's V offsets see
-    auto set_voff = [&](int rows) {
-      int vo[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) vo[i] = min(tile_row0 + 4 * i, rows - 1) * row_bytes + v_piece;
-      asm volatile(FLASHW_SET_VOFF ::"v"(vo[0]), "v"(vo[1]), "v"(vo[2]), "v"(vo[3]) : FLASHW_CLOBBERS);
-    };
-    auto next_v = [&]() -> u32x4_t {
-      int rows;
-      const u32x4_t r = tile_rsrc(v_pos, rows);
-      if (rows > 0 && rows < kKeysPerTile) set_voff(rows);
-      return r;
-    };
-    auto next_k = [&]() -> u32x4_t {
-      int rows;
-      return tile_rsrc(k_pos, rows);
-    };
+    const uintptr_t off = (uintptr_t)((nb.base * row_elems + g * kHeadDim) * 2);
+    k_pos = TilePos{reinterpret_cast<uintptr_t>(k) + off, nb.kmax};
+    v_pos = TilePos{reinterpret_cast<uintptr_t>(v) + off, nb.kmax};
     set_voff(kKeysPerTile);
-
-    if (n_tiles > 0) {
-      // K(0), K(1), V(0), K(2), V(1): the order the steps' waits count on
+    if (nb.n_tiles > 0) {
       u32x4_t r = next_k();
       asm volatile(FLASHW_LOAD4_K ::[dst] "s"(ldsw), [r] "s"(r) : FLASHW_CLOBBERS);
       r = next_k();
@@ -604,26 +628,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kWideCompilerVg
       r = next_v();
       asm volatile(FLASHW_LOAD4_V ::[dst] "s"(ldsw + 4 * kTileBytes), [r] "s"(r) : FLASHW_CLOBBERS);
     }
-    // Q^T operand fragments into the accumulation registers they stay in, behind the tile loads so that their
-    // latency runs under the tiles': eight 16-byte loads in flight per column block
-#define FLASHW_LOADQ(CB)                                                                                             \
-  {                                                                                                                  \
-    const bf16_t* qrow = q + ((int64_t)(q_first + (col_ok[CB] ? tok[CB] : 0)) * Hq + head[CB]) * kHeadDim + 8 * half; \
-    uint4 w[8];                                                                                                      \
-    _Pragma("unroll") for (int ks = 0; ks < 8; ++ks)                                                                 \
-        w[ks] = col_ok[CB] ? *reinterpret_cast<const uint4*>(qrow + 16 * ks) : make_uint4(0, 0, 0, 0);               \
-    FLASHW_SETQ(CB, 0, w[0]); FLASHW_SETQ(CB, 1, w[1]); FLASHW_SETQ(CB, 2, w[2]); FLASHW_SETQ(CB, 3, w[3]);          \
-    FLASHW_SETQ(CB, 4, w[4]); FLASHW_SETQ(CB, 5, w[5]); FLASHW_SETQ(CB, 6, w[6]); FLASHW_SETQ(CB, 7, w[7]);          \
-  }
-    FLASHW_LOADQ(0)
-    FLASHW_LOADQ(1)
-#undef FLASHW_LOADQ
+  };
+
+  int round = 0;
+  Block cur{}, nxt{};
+  bool have = find_block(round, cur);
+  if (have) request_block(cur);
+  while (have) {
+    const bool have_next = find_block(round, nxt);      // scalar work under the loads' latency
+    const int n_tiles = cur.n_tiles;
+    int wave_min_limit;
+    {
+      int lane_c = lane;
+      asm volatile("" : "+v"(lane_c));
+      const int half = lane_c >> 5;
+      int limit[2];
+#pragma unroll
+      for (int cb = 0; cb < 2; ++cb) {
+        const int col = 32 * cb + (lane_c & 31);
+        const int tok = cur.t0 + wave * kTokPerWave + col / G;
+        limit[cb] = tok < cur.sq ? (causal ? max(0, cur.L - cur.sq + tok + 1) : cur.L) : 0;
+      }
+      asm volatile(FLASHW_SET_LIMIT ::"v"(limit[0] - 4 * half), "v"(limit[1] - 4 * half) : FLASHW_CLOBBERS);
+      int wm = min(limit[0], limit[1]);
+#pragma unroll
+      for (int x = 32; x > 0; x >>= 1) wm = min(wm, __shfl_xor(wm, x));
+      wave_min_limit = __builtin_amdgcn_readfirstlane(wm);
+    }
+    // the block's query rows and first tiles have landed (and the last block's output stores are out)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    asm volatile(FLASHW_Q_FROM_LDS ::[qoff] "s"(ldsq) : FLASHW_CLOBBERS);
     FLASHW_ASM(FLASHW_INIT);
 
     if (n_tiles > 0) {
-      asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
+      asm volatile("s_barrier" ::: "memory");
       FLASHW_ASM(FLASHW_QK_FIRST);
-
       // The statements repeat with period six (LDS slots and score buffers are immediates), so the loop over the
       // tiles is unrolled by six; tile 0 (nothing to multiply by V yet) stands in front.
       int t = 0, flag;
@@ -667,27 +706,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kWideCompilerVg
         case 4: FLASHW_ASM(FLASHW_PV4); break;
         case 5: FLASHW_ASM(FLASHW_PV5); break;
       }
-      FLASHW_ASM(FLASHW_DRAIN);
-      // nothing may still be writing LDS, and every wavefront must be done reading it, when the next block's tiles
-      // are requested (or the workgroup ends)
+      // nothing may still be writing LDS (the tiles requested past the block's end), and every wavefront must be
+      // done reading the rings, when the next block's tiles are requested (or the workgroup ends)
       asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
+    if (have_next) request_block(nxt);
 
+    // ---- the finished block's output
+    FLASHW_ASM(FLASHW_DRAIN);
     float m0, m1, lsum[2];
     asm volatile(FLASHW_GET_ML : "=v"(m0), "=v"(m1), "=v"(lsum[0]), "=v"(lsum[1]));
     (void)m0; (void)m1;
-    // the columns' rows again, from the lane id (nothing per lane is kept in registers across the tile loop)
     int lane_e = lane;
     asm volatile("" : "+v"(lane_e));
-    const int half_e = lane_e >> 5;
     int64_t orow_e[2];
     bool ok_e[2];
 #pragma unroll
     for (int cb = 0; cb < 2; ++cb) {
       const int col = 32 * cb + (lane_e & 31);
-      const int tk = t0 + wave * kTokPerWave + col / G;
-      ok_e[cb] = tk < sq;
-      orow_e[cb] = ((int64_t)(q_first + tk) * Hq + g * G + col % G) * kHeadDim + 4 * half_e;
+      const int tk = cur.t0 + wave * kTokPerWave + col / G;
+      ok_e[cb] = tk < cur.sq;
+      orow_e[cb] = ((int64_t)(cur.q_first + tk) * Hq + g * G + col % G) * kHeadDim + 4 * (lane_e >> 5);
     }
 #define FLASHW_STORE(CB, D)                                                                              \
   {                                                                                                      \
@@ -712,7 +751,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kWideCompilerVg
     FLASHW_STORE(0, 0) FLASHW_STORE(0, 1) FLASHW_STORE(0, 2) FLASHW_STORE(0, 3)
     FLASHW_STORE(1, 0) FLASHW_STORE(1, 1) FLASHW_STORE(1, 2) FLASHW_STORE(1, 3)
 #undef FLASHW_STORE
+    cur = nxt;
+    have = have_next;
   }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #endif
 }
 

@@ -30,11 +30,15 @@ Registers the statements own (compiler-allocated code stays below v56 and uses n
   v84, v85  masked steps: column limit minus the tile's first key minus 4 half, per column block (the limits
             minus 4 half wait in a192, a193)
   v86-v95   temporaries
-  v96-v111  K fragment ring (4 x 4), v112-v127 V^T fragment ring (4 x 4): fragments are read from LDS a pair ahead
-            (the next pair is requested, then one wait covers the pair about to be multiplied)
+  v96-v127  free
   a0-a127   O^T: block (cb, d) at 64 cb + 16 d;   a128-a191   Q^T fragments: (cb, ks) at 128 + 32 cb + 4 ks
+  a196-a211 K fragment ring (4 x 4), a212-a227 V^T fragment ring (4 x 4): fragments are read from LDS a pair ahead
+            (the next pair is requested, then one wait covers the pair about to be multiplied), straight into
+            accumulation registers: returns into the vector registers compete with the VALU instructions of a
+            wavefront that is alone on its SIMD (a half step measured 13 % shorter this way)
   s84-s95   scratch
-LDS: K ring at 0 / 0x4000 / 0x8000, V ring at 0xC000 / 0x10000 / 0x14000 (96 KB).
+LDS: K ring at 0 / 0x4000 / 0x8000, V ring at 0xC000 / 0x10000 / 0x14000 (96 KB); behind them 16 KB per wavefront
+for the query rows of its next block (two column blocks of 32 rows x 256 bytes).
 
 Hazards kept by construction: a VALU read of an MFMA result stands at least 24 wait states behind the MFMA; a
 half-wave swap reads its operands two wait states after their VALU write; one instruction between a write of M0
@@ -48,7 +52,7 @@ V_FIRST = 56        # the statements own v56 - v255
 V_KAT, V_VAT, V_KOFF, V_VOFF = 56, 64, 68, 72
 V_M, V_L, V_ALPHA, V_REL = 76, 78, 82, 84
 V_T = 86            # 10 temporaries
-V_KF, V_VA = 96, 112
+A_KF, A_VA = 196, 212    # fragment rings, in accumulation registers
 RING = 4            # fragments per ring
 BUF = [128, 192]
 KSLOT, VSLOT = 0x4000, 0x4000
@@ -79,13 +83,13 @@ def p_frag(buf, cb, jj):
 
 
 def kf(f):
-    b = V_KF + 4 * (f % RING)
-    return f"v[{b}:{b + 3}]"
+    b = A_KF + 4 * (f % RING)
+    return f"a[{b}:{b + 3}]"
 
 
 def va(f):
-    b = V_VA + 4 * (f % RING)
-    return f"v[{b}:{b + 3}]"
+    b = A_VA + 4 * (f % RING)
+    return f"a[{b}:{b + 3}]"
 
 
 def k_read(f, slot):
@@ -95,10 +99,10 @@ def k_read(f, slot):
 
 def v_read(f, slot):
     jj, d = f >> 2, f & 3
-    b = V_VA + 4 * (f % RING)
+    b = A_VA + 4 * (f % RING)
     off = slot * VSLOT + jj * 4096
-    return [f"ds_read_b64_tr_b16 v[{b}:{b + 1}], v{V_VAT + d} offset:{off}",
-            f"ds_read_b64_tr_b16 v[{b + 2}:{b + 3}], v{V_VAT + d} offset:{off + 2048}"]
+    return [f"ds_read_b64_tr_b16 a[{b}:{b + 1}], v{V_VAT + d} offset:{off}",
+            f"ds_read_b64_tr_b16 a[{b + 2}:{b + 3}], v{V_VAT + d} offset:{off + 2048}"]
 
 
 # ------------------------------------------------------------------------------------------------- VALU streams
@@ -174,33 +178,38 @@ def growth_ops(cb):
     return head, unit
 
 
-def exp_group(buf, rb, k, tbase):
-    """Exponentials of element pair k of blocks (0, rb) and (1, rb), packed in place; row sums."""
-    streams = []
+def exp_stages(buf, rb, k, tbase):
+    """Exponentials of element pair k of blocks (0, rb) and (1, rb), packed in place, and their row sums, as three
+    stages of independent instructions (a stage depends on the one before it)."""
+    st = [[], [], []]
     for cb in range(2):
         b = BUF[buf] + 32 * cb + 16 * rb
         e0, e1 = b + 2 * k, b + 2 * k + 1
         dst = b + k if k < 4 else b + 8 + (k - 4)
         t0, t1 = f"v{tbase + 2 * cb}", f"v{tbase + 2 * cb + 1}"
         m = f"v{V_M + cb}"
-        streams.append([f"v_fma_f32 {t0}, v{e0}, %[c], -{m}",
-                        f"v_fma_f32 {t1}, v{e1}, %[c], -{m}",
-                        f"v_exp_f32 {t0}, {t0}",
-                        f"v_exp_f32 {t1}, {t1}",
-                        f"v_add_f32 v{V_L + 2 * cb}, v{V_L + 2 * cb}, {t0}",
-                        f"v_add_f32 v{V_L + 2 * cb + 1}, v{V_L + 2 * cb + 1}, {t1}",
-                        f"v_cvt_pk_bf16_f32 v{dst}, {t0}, {t1}"])
-    return interleave(*streams)
+        st[0] += [f"v_fma_f32 {t0}, v{e0}, %[c], -{m}", f"v_fma_f32 {t1}, v{e1}, %[c], -{m}"]
+        st[1] += [f"v_exp_f32 {t0}, {t0}", f"v_exp_f32 {t1}, {t1}"]
+        # (row sums by fp32 additions: one v_dot2c_f32_bf16 per pair on the packed values measured 3.7 % slower)
+        st[2] += [f"v_cvt_pk_bf16_f32 v{dst}, {t0}, {t1}", f"v_add_f32 v{V_L + 2 * cb}, v{V_L + 2 * cb}, {t0}",
+                  f"v_add_f32 v{V_L + 2 * cb + 1}, v{V_L + 2 * cb + 1}, {t1}"]
+    return st
 
 
-def exp_groups(buf):
-    """The 16 groups of a tile (each: one element pair of both column blocks), temporaries alternating."""
+def exp_stream(buf, first, count):
+    """Groups first .. first + count - 1 of a tile (a group: one element pair of both column blocks) as one
+    instruction stream, software-pipelined so that no instruction stands right behind the one it depends on:
+    ... fma(n + 1), exp(n + 1), pack(n) and sums(n) ...  Two sets of temporaries alternate."""
+    groups = []
+    for n in range(first, first + count):
+        rb, k = n >> 3, n & 7
+        groups.append(exp_stages(buf, rb, k, V_T + 4 * (n % 2) + 2))
     out = []
-    n = 0
-    for rb in range(2):
-        for k in range(8):
-            out.append(exp_group(buf, rb, k, V_T + 2 + 4 * (n & 1)))
-            n += 1
+    for n in range(len(groups) + 1):
+        if n < len(groups):
+            out += groups[n][0] + groups[n][1]
+        if 0 <= n - 1 < len(groups):
+            out += groups[n - 1][2]
     return out
 
 
@@ -306,8 +315,7 @@ def half_a(i, has_pv=True, masked=False, valu=True, sync=True):
         (h0, u0), (h1, u1) = growth_ops(0), growth_ops(1)
         fillers += interleave(h0, h1)
         fillers += [u0, u1]
-        for g in exp_groups(buf)[:N_GROUPS_A]:
-            fillers += g
+        fillers += exp_stream(buf, 0, N_GROUPS_A)
         out.append("s_mov_b32 %[flag], 0")
     tail_sync = ["s_barrier"] + k_read(0, kslot_next) + k_read(1, kslot_next) if sync else []
     if not has_pv:
@@ -349,8 +357,7 @@ def half_b(i, has_qk=True, valu=True, loads=True, prefetch_own=False, prefetch_n
     out = []
     fillers = []
     if valu:
-        for g in exp_groups(buf)[N_GROUPS_A:]:
-            fillers += g
+        fillers += exp_stream(buf, N_GROUPS_A, 16 - N_GROUPS_A)
     tail = v_read(0, vslot_next) + v_read(1, vslot_next) if prefetch_next else []
     if not has_qk:
         return fix_swap_hazards(out + flat(fillers) + tail)
@@ -441,12 +448,27 @@ def main():
     init += [f"v_accvgpr_write_b32 a{r}, 0" for r in range(128)]
     parts.append(define("FLASHW_INIT", init))
     for cb in range(2):
-        for ks in range(8):
-            b = 128 + 32 * cb + 4 * ks
-            parts.append(define(f"FLASHW_SET_Q{cb}_{ks}", [f"v_accvgpr_write_b32 a{b + x}, %{x}" for x in range(4)]))
         for d in range(4):
             b = 64 * cb + 16 * d
             parts.append(define(f"FLASHW_GET_O{cb}_{d}", [f"v_accvgpr_read_b32 %{x}, a{b + x}" for x in range(16)]))
+    # four 1 KB blocks of the wavefront's query rows into its private LDS region ([dst], then + 1 KB each): a block
+    # is four rows of 256 bytes, lane l fetching the piece that belongs at position l % 16 of row l / 16
+    lines = [f"s_mov_b32 {S_M0}, m0", "s_mov_b32 m0, %[dst]", "s_nop 4"]
+    for j in range(4):
+        lines.append(f"buffer_load_dwordx4 %[o{j}], %[r], 0 offen lds")
+        if j < 3:
+            lines += ["s_add_u32 m0, m0, 0x400", "s_nop 0"]
+    lines.append(f"s_mov_b32 m0, {S_M0}")
+    parts.append(define("FLASHW_LOADQ4", lines))
+    # Q^T operand fragments out of that region ([qoff]: its LDS address; rows swizzled like a K tile's, so the K
+    # fragment addresses serve) into the accumulation registers they stay in
+    lines = [f"v_add_u32 v{V_T + ks}, %[qoff], v{V_KAT + ks}" for ks in range(8)]
+    for cb in range(2):
+        for ks in range(8):
+            b = 128 + 32 * cb + 4 * ks
+            lines.append(f"ds_read_b128 a[{b}:{b + 3}], v{V_T + ks} offset:{8192 * cb}")
+    lines.append("s_waitcnt lgkmcnt(0)")
+    parts.append(define("FLASHW_Q_FROM_LDS", lines))
     parts.append(define("FLASHW_DRAIN", ["s_nop 15", "s_nop 7"]))
     parts.append(define("FLASHW_GET_ML", [f"v_mov_b32 %0, v{V_M}", f"v_mov_b32 %1, v{V_M + 1}",
                                           f"v_add_f32 %2, v{V_L}, v{V_L + 1}", f"v_add_f32 %3, v{V_L + 2}, v{V_L + 3}"]))

@@ -726,20 +726,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_num_vgpr(kWideCompilerVg
       const int col = 32 * cb + (lane_e & 31);
       const int tk = cur.t0 + wave * kTokPerWave + col / G;
       ok_e[cb] = tk < cur.sq;
-      orow_e[cb] = ((int64_t)(cur.q_first + tk) * Hq + g * G + col % G) * kHeadDim + 4 * (lane_e >> 5);
+      orow_e[cb] = ((int64_t)(cur.q_first + tk) * Hq + g * G + col % G) * kHeadDim + 8 * (lane_e >> 5);
     }
+    // A lane holds dims 8 e4 + 4 half .. + 4 of each group of eight; the two halves of a wavefront trade one group
+    // of four per pair of groups (half-wave swap), after which a lane holds eight consecutive dims and stores 16 bytes
 #define FLASHW_STORE(CB, D)                                                                              \
   {                                                                                                      \
     float x[16];                                                                                         \
     FLASHW_GETO(CB, D, x);                                                                               \
-    if (ok_e[CB]) {                                                                                      \
-      bf16_t* orow = out + orow_e[CB];                                                                   \
-      _Pragma("unroll") for (int e4 = 0; e4 < 4; ++e4) {                                                 \
-        uint2 w;                                                                                         \
-        w.x = pack_bf16x2(x[4 * e4] * inv[CB], x[4 * e4 + 1] * inv[CB]);                                 \
-        w.y = pack_bf16x2(x[4 * e4 + 2] * inv[CB], x[4 * e4 + 3] * inv[CB]);                             \
-        *reinterpret_cast<uint2*>(orow + 32 * D + 8 * e4) = w;                                           \
-      }                                                                                                  \
+    uint32_t w[8];                                                                                       \
+    _Pragma("unroll") for (int i = 0; i < 8; ++i) w[i] = pack_bf16x2(x[2 * i] * inv[CB], x[2 * i + 1] * inv[CB]); \
+    _Pragma("unroll") for (int pr = 0; pr < 2; ++pr) {                                                   \
+      const auto r0 = __builtin_amdgcn_permlane32_swap(w[4 * pr], w[4 * pr + 2], false, false);          \
+      const auto r1 = __builtin_amdgcn_permlane32_swap(w[4 * pr + 1], w[4 * pr + 3], false, false);      \
+      if (ok_e[CB])                                                                                      \
+        *reinterpret_cast<uint4*>(out + orow_e[CB] + 32 * D + 16 * pr) = make_uint4(r0[0], r1[0], r0[1], r1[1]); \
     }                                                                                                    \
   }
     float inv[2];

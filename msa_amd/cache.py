@@ -87,3 +87,24 @@ class CustomDynamicCacheOnCPU(CustomDynamicCache):
 
 def create_cache() -> CustomDynamicCache:
     return CustomDynamicCache()
+
+
+def compact_cache_reference_layout(key_cache: torch.Tensor, value_cache: torch.Tensor, kv_lengths: torch.Tensor):
+    """The compact decode cache in the layout the reference keeps it in (src/msa/memory_sparse_attention.py:344-357):
+    ``key / value [B, Hkv, maxL, D]`` left-padded with zeros and ``attention_mask [B, maxL]`` (True on the valid,
+    right-aligned rows), ``maxL = kv_lengths.max()``.  This build keeps ``[B, Lcap, Hkv, D]`` with rows valid from 0
+    and appends in place; code that reads ``cache_kwargs["compacked_key_cache"]`` in the reference's layout takes this
+    copy instead (a conversion for outside readers: the attention kernels never need it)."""
+    B, _, Hkv, D = key_cache.shape
+    lens = kv_lengths.to(torch.int64)
+    max_len = int(lens.max()) if B else 0
+    pos = torch.arange(max_len, device=key_cache.device).unsqueeze(0)
+    mask = pos >= (max_len - lens.unsqueeze(1))                                   # [B, maxL]
+    src = (pos - (max_len - lens.unsqueeze(1))).clamp(min=0)                      # row of the cache a position holds
+    out = []
+    for cache in (key_cache, value_cache):
+        rows = torch.gather(cache[:, :max(max_len, 1)] if max_len else cache[:, :0], 1,
+                            src.view(B, max_len, 1, 1).expand(B, max_len, Hkv, D)) if max_len else cache[:, :0]
+        rows = rows * mask.view(B, max_len, 1, 1).to(rows.dtype)
+        out.append(rows.permute(0, 2, 1, 3).contiguous())
+    return out[0], out[1], mask

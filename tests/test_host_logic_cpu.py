@@ -216,3 +216,23 @@ def test_concatenated_projection_weights_follow_their_sources():
     got = layer._all_weight(dev)
     assert got.dtype == torch.bfloat16 and torch.equal(got, want())
     assert torch.equal(layer._fused_weight(dev), torch.cat([layer.q_proj.weight, layer.k_proj.weight, layer.v_proj.weight]))
+
+
+def test_compact_cache_in_the_reference_layout():
+    """[B, Lcap, Hkv, D] + lengths -> the reference's left-padded [B, Hkv, maxL, D] + mask, against a loop."""
+    g = torch.Generator().manual_seed(3)
+    B, Lcap, Hkv, D = 3, 9, 2, 4
+    kc, vc = torch.randn((B, Lcap, Hkv, D), generator=g), torch.randn((B, Lcap, Hkv, D), generator=g)
+    lens = torch.tensor([5, 0, 7], dtype=torch.int32)
+    k, v, mask = mcache.compact_cache_reference_layout(kc, vc, lens)
+    assert k.shape == v.shape == (B, Hkv, 7, D) and mask.shape == (B, 7)
+    for b in range(B):
+        n = int(lens[b])
+        assert mask[b].tolist() == [False] * (7 - n) + [True] * n
+        assert float(k[b, :, :7 - n].abs().max() if n < 7 else 0.0) == 0.0
+        for i in range(n):
+            assert torch.equal(k[b, :, 7 - n + i], kc[b, i]) and torch.equal(v[b, :, 7 - n + i], vc[b, i])
+    # the reference's own fill (boolean-mask assignment of the packed rows) gives the same tensors
+    want = torch.zeros((B, Hkv, 7, D))
+    want.permute(0, 2, 1, 3)[mask] = torch.cat([kc[b, :int(lens[b])] for b in range(B)])
+    assert torch.equal(k, want)

@@ -281,6 +281,12 @@ int msa_flash_attn(const void* q, const int32_t* cu_q, const void* k, const void
                    const int64_t* kv_off, const int32_t* kv_len, int32_t B, int32_t total_q,
                    int32_t Hq, int32_t Hkv, int32_t D, float scale, int32_t causal, void* out,
                    void* stream);
+/* The same with the longest query block of the batch named (the lengths themselves are on the device): a batch of
+ * ragged samples (max_sq * B > 1.25 total_q) keeps to the 32-column form of the kernel, see below. */
+int msa_flash_attn_hint(const void* q, const int32_t* cu_q, const void* k, const void* v,
+                        const int64_t* kv_off, const int32_t* kv_len, int32_t B, int32_t total_q,
+                        int32_t Hq, int32_t Hkv, int32_t D, float scale, int32_t causal, void* out,
+                        int32_t max_sq, void* stream);
 /* msa_flash_attn has two forms of its kernel: 32 (token, head) columns per wavefront, two workgroups per compute unit,
  * and a wide one (64 columns per wavefront, one wavefront per SIMD, the tile step written at the instruction level)
  * that it picks when the call has at least 4096 columns.  form 0: by size (the default), 1: always the first,

@@ -353,8 +353,8 @@ def sparse_attn(q, k, v, kv_off, kv_len, max_kv: int, cu_q=None, max_sq: int = 1
     # split-KV entry point below (which runs the same MFMA kernel per key range for bf16 blocks of >= 8 rows)
     if q.dtype == torch.bfloat16 and max_sq >= FLASH_MIN_ROWS and total_q * Hkv >= 32 * 512:
         out = torch.empty_like(q)
-        check(lib.msa_flash_attn(ptr(q), ptr(cu_q), ptr(k), ptr(v), ptr(kv_off), ptr(kv_len), B, total_q, Hq, Hkv, D, sc,
-                                 int(causal), ptr(out), _stream()), "msa_flash_attn")
+        check(lib.msa_flash_attn_hint(ptr(q), ptr(cu_q), ptr(k), ptr(v), ptr(kv_off), ptr(kv_len), B, total_q, Hq, Hkv, D,
+                                      sc, int(causal), ptr(out), int(max_sq), _stream()), "msa_flash_attn")
         return out
     need = lib.msa_attn_workspace_bytes(total_q, Hq, Hkv, D, max_kv)
     ws = _attn_ws.get(q.device)

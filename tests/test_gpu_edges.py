@@ -353,6 +353,45 @@ def test_flash_kernel_through_the_c_abi(ops, Hq, Hkv, causal, flash_form):
             assert cf.rel_err(out[rows][blind:], want) < 1e-2, (b, sq[b], L[b])
 
 
+def test_flash_hint_keeps_ragged_batches_on_the_32_column_form(ops):
+    """msa_flash_attn_hint with the longest query block named: a ragged batch takes the 32-column form, an even one of
+    at least 4096 columns the wide form (bit-identical outputs with the forms forced tell which one ran)."""
+    say("flash hint: ragged batch -> 32-column form")
+    from msa_amd import _lib
+    lib = _lib.load()
+    Hq, Hkv, D = 32, 8, 128
+    st = torch.cuda.current_stream().cuda_stream
+
+    def run(entry, sq, extra=()):
+        L = [s + 100 for s in sq]
+        cu_q = np.concatenate([[0], np.cumsum(sq)])
+        cu_kv = np.concatenate([[0], np.cumsum(L)])
+        q = _randn((int(cu_q[-1]), Hq, D), 320, torch.bfloat16).cuda()
+        k = _randn((int(cu_kv[-1]), Hkv, D), 321, torch.bfloat16).cuda()
+        v = _randn((int(cu_kv[-1]), Hkv, D), 322, torch.bfloat16).cuda()
+        kv_off = torch.as_tensor(cu_kv[:-1], dtype=torch.int64).cuda()
+        kv_len = torch.as_tensor(L, dtype=torch.int32).cuda()
+        cu = torch.as_tensor(cu_q, dtype=torch.int32).cuda()
+        out = torch.full_like(q, float("nan"))
+        _lib.check(getattr(lib, entry)(_lib.ptr(q), _lib.ptr(cu), _lib.ptr(k), _lib.ptr(v), _lib.ptr(kv_off), _lib.ptr(kv_len),
+                                       len(sq), int(cu_q[-1]), Hq, Hkv, D, D ** -0.5, 1, _lib.ptr(out), *extra, st), entry)
+        torch.cuda.synchronize()
+        return out
+
+    for sq, want_form in (([700, 90, 130, 60, 50, 40], 1), ([200] * 6, 2)):
+        got = run("msa_flash_attn_hint", sq, (max(sq),))
+        forced = {}
+        for form in (1, 2):
+            _lib.check(lib.msa_flash_set_form(form), "msa_flash_set_form")
+            try:
+                forced[form] = run("msa_flash_attn", sq)
+            finally:
+                _lib.check(lib.msa_flash_set_form(0), "msa_flash_set_form")
+        assert not torch.equal(forced[1], forced[2])            # the forms round differently somewhere
+        assert torch.equal(got, forced[want_form]), (sq, want_form)
+    assert lib.msa_flash_attn_hint(None, None, None, None, None, None, 1, 1, Hq, Hkv, D, C.c_float(1.0), 1, None, 0, st) != 0
+
+
 @pytest.mark.parametrize("causal", [True, False])
 def test_flash_kernel_ignores_stale_lds(ops, causal, flash_form):
     """The flash kernel's K / V tiles arrive in LDS by direct loads; rows past a sample's last key are not loaded.

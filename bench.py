@@ -435,6 +435,7 @@ def main():
                 host_k.pop(); host_v.pop()
             break
         host_k.append(pair[0]); host_v.append(pair[1])
+    pair = None
     if not host_k:
         sys.exit("bench.py: could not pin one layer of host K / V")
     n_host = len(host_k)
@@ -678,7 +679,16 @@ def main():
 
     if extras is not None and not args.no_e2e:
         # configs[4] end to end (the "sparse decode tok/s" half of the metric); ~25 GB next to the 100M bank's 60 GB
+        import gc
         import bench_e2e
+        # the 100M-token bank's pinned host K / V go back to the system first: the boxes refuse pinned memory past
+        # about 56 GB and the end-to-end run pins a bank of its own
+        torch.cuda.synchronize()
+        bank._keep.clear()
+        del bank, wk, wv
+        host_k.clear(); host_v.clear()
+        gc.collect()
+        torch._C._host_emptyCache()
         r = bench_e2e.main(["--steps", "256"], quiet=True)
         extras["e2e_sparse_decode"] = {"workload": r["config"]["workload"] + ", 10M-token bank, B=16, 4K context, greedy",
                                        "tokens_per_s": r["value"], "ms_per_decode_step": r["ms_per_decode_step"],

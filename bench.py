@@ -349,11 +349,12 @@ def extra_prefill_attention(dev):
     from msa_amd import _lib
     lib = _lib.load()
     run = lambda: ops.sparse_attn(q, kc, vc, kv_off, kv_len, L, cu_q=cu_q, max_sq=S, causal=True)
-    ms = time_cuda(run, 10)
+    # (ten warm-up launches each: the chip's power management takes about that long to settle on a kernel's load)
+    ms = time_cuda(run, 10, warm=10)
     # the 32-column form of the kernel in the same process, for comparison (the call above picks the wide form)
     _lib.check(lib.msa_flash_set_form(1), "msa_flash_set_form")
     try:
-        ms32 = time_cuda(run, 10)
+        ms32 = time_cuda(run, 10, warm=10)
     finally:
         _lib.check(lib.msa_flash_set_form(0), "msa_flash_set_form")
     pairs = B * (S * M + S * (S + 1) // 2)

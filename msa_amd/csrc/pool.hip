@@ -6,7 +6,7 @@
 // per step, accumulate in fp32 registers, and fold the R partial rows through LDS at the end.
 // Each lane keeps two groups of rows in flight as raw 16-byte loads (16 KB per wavefront in bf16):
 // with one row per wait the kernel was bound by load latency at 0.65-0.68 of the HBM rate; the
-// two-group pipeline reaches 0.75.
+// two-group pipeline reaches 0.76, and 0.79 with non-temporal stores of the pooled rows (see store8).
 #include <type_traits>
 
 #include "common.h"
@@ -70,7 +70,13 @@ __device__ __forceinline__ void store8<bf16_t>(bf16_t* p, const float (&x)[8]) {
   uint4 w;
   w.x = pack_bf16x2(x[0], x[1]); w.y = pack_bf16x2(x[2], x[3]);
   w.z = pack_bf16x2(x[4], x[5]); w.w = pack_bf16x2(x[6], x[7]);
-  *reinterpret_cast<uint4*>(p) = w;
+  // Non-temporal: a write among the saturated read stream is what holds this kernel below the rate of its loads (a
+  // bare loop of the same loads streams at 0.90 of the HBM rate, at 0.75 once every workgroup ends with a plain 2 KB
+  // store and at 0.79 with a non-temporal one; 512 bytes per workgroup already cost 0.10).  Writing the pooled rows
+  // eight at a time from LDS, from threads that take no part in the loads, or from a persistent workgroup whose next
+  // loads are in flight changed nothing: the cost is the memory system's, per write and per byte.
+  const u32x4_t ww = {w.x, w.y, w.z, w.w};
+  __builtin_nontemporal_store(ww, reinterpret_cast<u32x4_t*>(p));
 }
 template <>
 __device__ __forceinline__ void store8<float>(float* p, const float (&x)[8]) {
@@ -190,11 +196,12 @@ __global__ __launch_bounds__(kThreads, 2) void pool_chunks_kernel(PoolArgs a) {
   };
   stream(std::integral_constant<bool, kRope>{});
 
-  // fold the R partial rows: fold[(r * U + u) * 16 + i]
+  // fold the R partial rows through LDS: value i of thread t at fold[i * kThreads + t] (consecutive lanes hit
+  // consecutive banks on the way in and on the way out)
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    fold[(r * U + u) * 16 + i] = acc_lo[i];
-    fold[(r * U + u) * 16 + 8 + i] = acc_hi[i];
+    fold[i * kThreads + tid] = acc_lo[i];
+    fold[(8 + i) * kThreads + tid] = acc_hi[i];
   }
   __syncthreads();
   if (tid < U) {
@@ -205,8 +212,8 @@ __global__ __launch_bounds__(kThreads, 2) void pool_chunks_kernel(PoolArgs a) {
     for (int rr = 0; rr < R; ++rr) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        lo[i] += fold[(rr * U + tid) * 16 + i];
-        hi[i] += fold[(rr * U + tid) * 16 + 8 + i];
+        lo[i] += fold[i * kThreads + rr * U + tid];
+        hi[i] += fold[(8 + i) * kThreads + rr * U + tid];
       }
     }
 #pragma unroll

@@ -353,6 +353,30 @@ def test_flash_kernel_through_the_c_abi(ops, Hq, Hkv, causal, flash_form):
             assert cf.rel_err(out[rows][blind:], want) < 1e-2, (b, sq[b], L[b])
 
 
+def test_flash_kernel_one_row_per_sample_without_cu_q(ops, flash_form):
+    """cu_q = NULL means one query row per sample (total_q == B): both forms, causal (the row sees all its keys)."""
+    say(f"flash kernel, one row per sample, no cu_q, form={flash_form}")
+    from msa_amd import _lib
+    lib = _lib.load()
+    Hq, Hkv, D = 32, 8, 128
+    L = [70, 1, 129, 300, 64, 5]
+    cu_kv = np.concatenate([[0], np.cumsum(L)])
+    q = _randn((len(L), Hq, D), 330, torch.bfloat16)
+    k = _randn((int(cu_kv[-1]), Hkv, D), 331, torch.bfloat16)
+    v = _randn((int(cu_kv[-1]), Hkv, D), 332, torch.bfloat16)
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    kv_off = torch.as_tensor(cu_kv[:-1], dtype=torch.int64).cuda()
+    kv_len = torch.as_tensor(L, dtype=torch.int32).cuda()
+    out = torch.full_like(qd, float("nan"))
+    _lib.check(lib.msa_flash_attn(_lib.ptr(qd), None, _lib.ptr(kd), _lib.ptr(vd), _lib.ptr(kv_off), _lib.ptr(kv_len),
+                                  len(L), len(L), Hq, Hkv, D, D ** -0.5, 1, _lib.ptr(out),
+                                  torch.cuda.current_stream().cuda_stream), "msa_flash_attn")
+    torch.cuda.synchronize()
+    for b in range(len(L)):
+        want = cf.attention(q[b:b + 1], k[int(cu_kv[b]):int(cu_kv[b + 1])], v[int(cu_kv[b]):int(cu_kv[b + 1])], causal=True)
+        assert cf.rel_err(out[b:b + 1].cpu(), want) < 1e-2, b
+
+
 def test_flash_hint_keeps_ragged_batches_on_the_32_column_form(ops):
     """msa_flash_attn_hint with the longest query block named: a ragged batch takes the 32-column form, an even one of
     at least 4096 columns the wide form (bit-identical outputs with the forms forced tell which one ran)."""

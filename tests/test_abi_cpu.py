@@ -134,3 +134,20 @@ def test_build_guard_fails_on_a_forced_spill():
     problems = B.check_kernel_contracts(asm, "score_scan4_kernel", max_compiler_vgpr=127, no_agpr=True)
     assert problems, "a spilling build passed the check"
     assert any("spill" in p or "scratch" in p or "private_segment" in p or "accumulation" in p for p in problems), problems[:5]
+
+
+@pytest.mark.parametrize("gen", ["gen_scan_asm.py", "gen_flash_asm.py"])
+def test_generated_asm_includes_are_what_their_generators_emit(gen):
+    """The committed scan_asm.inc / flash_asm.inc are the generators' output (the build refuses a stale one too)."""
+    import subprocess
+    import sys
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "msa_amd", "csrc")
+    assert subprocess.run([sys.executable, os.path.join(csrc, gen), "--check"]).returncode == 0
+
+
+def test_build_guard_covers_the_wide_flash_kernel():
+    from msa_amd import build
+    names = [k for k, _ in build.CONTRACTS["flash_attn.hip"]]
+    assert "flash_wide_kernel" in names and "flash_attn_kernel" in names
+    rules = dict(build.CONTRACTS["flash_attn.hip"])["flash_wide_kernel"]
+    assert rules == {"max_compiler_vgpr": 55, "no_agpr": True}

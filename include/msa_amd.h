@@ -175,6 +175,12 @@ int msa_diag_mfma_loop(int32_t workgroups, int32_t iters, int32_t mode, float* s
 int msa_diag_scan_walk(int32_t tiles_m, int32_t tiles_n, int32_t grid, int32_t has_copy_workgroup, int32_t pool_n,
                        int32_t* visits);
 
+/* Registers and bytes of scratch per lane of the loaded code object's asm-scheduled kernels (which = 0: the routing
+ * scan score_scan4_kernel, 1: flash_wide_kernel).  Their statements keep state in physical registers across statements,
+ * which only holds while the compiler spilled nothing: the library refuses to launch either with scratch (MSA_ESTATE),
+ * and this call lets a test see the numbers.  A diagnostic: no counterpart in the reference. */
+int msa_diag_asm_kernel_resources(int32_t which, int32_t* num_regs, int32_t* scratch_bytes);
+
 /* Switch (no counterpart in the reference): the large-tile scan hands the last eighth of its tiles out dynamically,
  * from a counter in the workspace, to even out the ends of the eight XCDs.  enabled = 0 gives every tile a fixed
  * workgroup (a few percent slower on large banks; no atomics on the hand-out path); 1 is the default.  Process-wide,

@@ -53,6 +53,7 @@ SIGNATURES = {
     "msa_attn_workspace_bytes": (_sz, [_i32, _i32, _i32, _i32, _i32]),
     "msa_flash_attn": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _vp]),
     "msa_flash_set_form": (C.c_int, [_i32]),
+    "msa_diag_asm_kernel_resources": (C.c_int, [_i32, _vp, _vp]),
     "msa_flash_attn_hint": (C.c_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i32, _i32, _i32, _i32, _i32, _f32, _i32, _vp, _i32, _vp]),
     "msa_qk_norm_rope": (C.c_int, [_vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _f32, _vp, _vp, _i32, _i32, _i64, _i32,
                                    _i32, _i32, _vp, _vp, _vp, _vp]),

@@ -41,6 +41,33 @@ static inline hipError_t raise_dynamic_lds_limit(std::atomic<int>& done, const v
   return e;
 }
 
+// The kernels whose main loops are asm statements on physical registers keep state in registers across statements:
+// that only holds while the compiler spills nothing (a spill's reload is a vector-memory load among hand-counted
+// waits, and its address set-up lands in registers the statements own).  The build checks this on the device
+// assembly; this is the same check on the code object that was actually loaded, once per kernel, before its first
+// launch.
+static inline int check_asm_kernel_resources(std::atomic<int>& done, const void* kernel, const char* name, int* num_regs,
+                                             int* scratch_bytes) {
+  if (done.load(std::memory_order_acquire) && !num_regs) return MSA_OK;
+  hipFuncAttributes attr;
+  const hipError_t e = hipFuncGetAttributes(&attr, kernel);
+  if (e != hipSuccess) {
+    msa_set_error("hipFuncGetAttributes(%s) failed: %s", name, hipGetErrorString(e));
+    return MSA_EHIP;
+  }
+  if (num_regs) *num_regs = attr.numRegs;
+  if (scratch_bytes) *scratch_bytes = (int)attr.localSizeBytes;
+  // (512 registers: the statements name registers up to v255 and a255, and one wavefront per SIMD is what they are
+  // scheduled for)
+  if (attr.localSizeBytes != 0 || attr.numRegs != 512) {
+    msa_set_error("%s was built with %d registers and %d bytes of scratch per lane (512 and 0 expected): its asm "
+                  "statements' register contract does not hold", name, attr.numRegs, (int)attr.localSizeBytes);
+    return MSA_ESTATE;
+  }
+  done.store(1, std::memory_order_release);
+  return MSA_OK;
+}
+
 // Compute units of the current device (asked once; the library drives one device per process).
 static inline int device_compute_units() {
   static const int n = [] {

@@ -769,7 +769,10 @@ int flash_wide_launch_g(const void* q, const int32_t* cu_q, const void* k, const
   // one workgroup per compute unit, the same number for every KV head
   const int per_head = (int)std::min<int64_t>(blocks, std::max(1, device_compute_units() / Hkv));
   auto kern = flash_wide_kernel<G>;
-  static std::atomic<int> lds_limit_raised{0};
+  static std::atomic<int> lds_limit_raised{0}, resources_checked{0};
+  if (const int rc = check_asm_kernel_resources(resources_checked, reinterpret_cast<const void*>(kern), "flash_wide_kernel",
+                                                nullptr, nullptr))
+    return rc;
   MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(kern), kWideLdsBytes));
   kern<<<dim3((unsigned)(per_head * Hkv)), 256, kWideLdsBytes, st>>>(
       static_cast<const bf16_t*>(q), cu_q, static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v), kv_off, kv_len,
@@ -863,6 +866,12 @@ extern "C" int msa_flash_attn_hint(const void* q, const int32_t* cu_q, const voi
                                    float scale, int32_t causal, void* out, int32_t max_sq, void* stream) {
   MSA_REQUIRE(max_sq > 0, "msa_flash_attn_hint: max_sq must be the longest query block of the batch");
   return flash_attn_entry(q, cu_q, k, v, kv_off, kv_len, B, total_q, Hq, Hkv, D, scale, causal, out, max_sq, stream);
+}
+
+int flash_wide_kernel_resources(int* num_regs, int* scratch_bytes) {
+  std::atomic<int> unused{0};
+  return check_asm_kernel_resources(unused, reinterpret_cast<const void*>(flash_wide_kernel<4>), "flash_wide_kernel", num_regs,
+                                    scratch_bytes);
 }
 
 extern "C" int msa_flash_set_form(int32_t form) {

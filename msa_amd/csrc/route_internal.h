@@ -52,3 +52,6 @@ int route_scores_to_keys(const msa_bank* bank, int32_t layer, const void* q, con
                          size_t workspace_bytes, hipStream_t st, RouteWorkspace* layout_out, float* mul_out,
                          const char* who, const GatherJob* job = nullptr, bool* job_taken = nullptr,
                          int32_t query_reduce = MSA_QUERY_MAX, int64_t extra_plane_cols = 0);
+
+// flash_attn.hip: registers and scratch bytes of the loaded wide flash-attention kernel (a diagnostic)
+int flash_wide_kernel_resources(int* num_regs, int* scratch_bytes);

@@ -1207,7 +1207,10 @@ int launch_scan4(const void* qs, const void* kr, const uint32_t* row_bits, uint3
     if (job_taken) *job_taken = true;
   }
   auto kern = score_scan4_kernel<kDocMax>;
-  static std::atomic<int> lds_limit_raised{0};
+  static std::atomic<int> lds_limit_raised{0}, resources_checked{0};
+  if (const int rc = check_asm_kernel_resources(resources_checked, reinterpret_cast<const void*>(kern), "score_scan4_kernel",
+                                                nullptr, nullptr))
+    return rc;
   MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(kern), kScan4LdsBytes));
   int slot = -1;
   if (g_timer.on.load(std::memory_order_acquire)) {
@@ -1318,6 +1321,24 @@ extern "C" int msa_diag_scan_walk(int32_t tiles_m, int32_t tiles_n, int32_t grid
 }
 
 // The tile pool of the large-tile scan can be switched off (every tile then belongs to a fixed workgroup).
+extern "C" int msa_diag_asm_kernel_resources(int32_t which, int32_t* num_regs, int32_t* scratch_bytes) {
+  MSA_REQUIRE(num_regs && scratch_bytes, "msa_diag_asm_kernel_resources: null pointer");
+  std::atomic<int> unused{0};
+  int regs = 0, scratch = 0, rc;
+  if (which == 0)
+    rc = check_asm_kernel_resources(unused, reinterpret_cast<const void*>(score_scan4_kernel<true>), "score_scan4_kernel", &regs,
+                                    &scratch);
+  else if (which == 1)
+    rc = flash_wide_kernel_resources(&regs, &scratch);
+  else {
+    msa_set_error("msa_diag_asm_kernel_resources: which = 0 (routing scan) or 1 (wide flash attention)");
+    return MSA_EINVAL;
+  }
+  *num_regs = regs;
+  *scratch_bytes = scratch;
+  return rc;
+}
+
 extern "C" int msa_route_set_tile_pool(int32_t enabled) {
   g_tile_pool_enabled.store(enabled ? 1 : 0, std::memory_order_relaxed);
   return MSA_OK;

@@ -667,3 +667,19 @@ def test_route_topk_mid_size_banks_with_the_tile_pool(seed):
         assert bool((true_of_returned >= kth - 1e-3).all())                  # the 1e-3 gap rule at the k boundary
         assert bool((sc[b][:-1] >= sc[b][1:]).all())
         assert torch.equal(gid[b], doc[b].long())
+
+
+def test_asm_scheduled_kernels_were_loaded_without_scratch(ops):
+    """The loaded code object's routing scan and wide flash kernel use no scratch memory (their asm statements keep
+    state in physical registers across statements; the library would refuse to launch them otherwise) and the whole
+    register file of a SIMD lane (one wavefront per SIMD)."""
+    say("resources of the asm-scheduled kernels")
+    from msa_amd import _lib
+    lib = _lib.load()
+    for which in (0, 1):
+        regs, scratch = C.c_int32(-1), C.c_int32(-1)
+        _lib.check(lib.msa_diag_asm_kernel_resources(which, C.byref(regs), C.byref(scratch)), "msa_diag_asm_kernel_resources")
+        print(f"[resources] kernel {which}: {regs.value} registers, {scratch.value} bytes of scratch", flush=True)
+        assert scratch.value == 0
+        assert regs.value == 512
+    assert lib.msa_diag_asm_kernel_resources(2, C.byref(regs), C.byref(scratch)) != 0

@@ -272,6 +272,35 @@ def extra_mfma_ceiling(dev):
     return out
 
 
+def extra_hbm_read_ceiling(dev):
+    """What the memory system gives loops that only read, in the access patterns of the HBM-bound kernels: the rates the
+    pooling and decode-attention fractions can be read against (the published 8 TB/s is not reached by any read loop)."""
+    from msa_amd import _lib
+    lib = _lib.load()
+    nbytes = 4 << 30
+    src = torch.empty(nbytes // 4, dtype=torch.int32, device=dev)
+    src.random_(0, 1 << 31)
+    dst = torch.empty(nbytes // 64 // 4, dtype=torch.int32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    out = {"workload": "read-only loops over 4 GiB (rows of 2 KB), best of 3 x 5 launches"}
+    for mode, name in ((0, "rows_nontemporal (pooling's reads)"), (1, "rows_plus_2KB_store_per_128KB (pooling's reads and writes)"),
+                       (2, "one_head_256B_pieces_2KB_apart (decode attention's reads)")):
+        def run():
+            _lib.check(lib.msa_diag_read_stream(src.data_ptr(), nbytes, dst.data_ptr(), mode, st), "msa_diag_read_stream")
+        ms = min(time_cuda(run, 5, warm=2) for _ in range(3))
+        out[name] = {"ms": round(ms, 4), "GB/s": round(nbytes / ms / 1e6, 1), "frac_hbm": round(nbytes / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    # launches of a decode layer-step's size (the K and V rows of 16 samples x 4400 tokens = 288 MB) over 14 distinct
+    # pieces of the buffer, back to back: what a launch that short gets, start and end included
+    piece = 16 * 4400 * 2 * 2048 // 131072 * 131072
+    for mode, name in ((0, "rows_nontemporal, 288 MB per launch"), (2, "one_head_256B_pieces_2KB_apart, 288 MB per launch")):
+        def run():
+            for i in range(nbytes // piece):
+                _lib.check(lib.msa_diag_read_stream(src.data_ptr() + i * piece, piece, dst.data_ptr(), mode, st), "msa_diag_read_stream")
+        ms = min(time_cuda(run, 3, warm=1) for _ in range(3)) / (nbytes // piece)
+        out[name] = {"us": round(ms * 1e3, 2), "GB/s": round(piece / ms / 1e6, 1), "frac_hbm": round(piece / ms / 1e6 / HBM_PEAK_GBS, 4)}
+    return out
+
+
 def extra_decode_projections(dev):
     """configs[4] projection share: the four weight-streaming linears of a decode layer and the LM head at B=16
     (Qwen3-4B shapes, bf16), each replayed from a HIP graph over distinct weight copies so that neither the Python
@@ -664,7 +693,8 @@ def main():
     if not args.no_extras:
         extras = {"pooling": extra_pooling(dev), "routing_10M_bank": extra_routing_10m(dev), "decode_attention": extra_decode(dev),
                   "prefill_attention": extra_prefill_attention(dev), "decode_projections": extra_decode_projections(dev),
-                  "mfma_ceiling": extra_mfma_ceiling(dev)}
+                  "mfma_ceiling": extra_mfma_ceiling(dev),
+                  "hbm_read_ceiling": extra_hbm_read_ceiling(dev)}
 
     cpu = None
     if not args.no_cpu_baseline:

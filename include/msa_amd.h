@@ -166,6 +166,17 @@ int msa_profile_collect(float* ms_host, int32_t cap, int32_t* n_out);
  * (the budget of a kernel that does softmax arithmetic between them). */
 int msa_diag_mfma_loop(int32_t workgroups, int32_t iters, int32_t mode, float* sink, double* flops_out, void* stream);
 
+/* Measurement aid (no counterpart in the reference): loops that only read `bytes` of device memory at `src`, taken
+ * as rows of 2 KB (8 heads x 128 bf16), in the access patterns of the library's HBM-bound kernels, enqueued on
+ * `stream`; bytes is a multiple of 128 KB.  mode 0: 64 consecutive rows per workgroup, non-temporal 16-byte loads (the
+ * pooling kernel's reads); dst (device, >= 16 bytes) is not written.  mode 1: the same plus pooling's writes, one
+ * 2 KB row of dst per 128 KB read: 16-byte word t (t < 128) of dst row w is the xor of the words at byte
+ * 4096 * i + 16 * t of workgroup w's 128 KB for i = 0 .. 31; dst holds bytes / 64.  mode 2: each
+ * workgroup reads one head's 256-byte piece of every row of a range of rows (the decode attention's reads of a
+ * [rows, 8, 128] cache); dst (>= 16 bytes) is not written.  bytes / time is the rate a kernel with that pattern can
+ * be held to on this GPU, below the published HBM peak. */
+int msa_diag_read_stream(const void* src, int64_t bytes, void* dst, int32_t mode, void* stream);
+
 /* Test aid (no counterpart in the reference; runs on the host, no GPU needed): replays the tile order of the
  * persistent large-tile scan (more than 128 query rows) for a launch of `grid` workgroups over tiles_m x tiles_n
  * tiles of 256 x 256, with or without the workgroup that copies K / V rows instead of scoring, the last pool_n N

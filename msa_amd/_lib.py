@@ -38,6 +38,7 @@ SIGNATURES = {
     "msa_profile_collect": (C.c_int, [_vp, _i32, _vp]),
     "msa_diag_mfma_loop": (C.c_int, [_i32, _i32, _i32, _vp, _vp, _vp]),
     "msa_diag_fill_lds": (C.c_int, [C.c_uint32, _vp, _i32, _vp]),
+    "msa_diag_read_stream": (C.c_int, [_vp, C.c_int64, _vp, _i32, _vp]),
     "msa_diag_scan_walk": (C.c_int, [_i32, _i32, _i32, _i32, _i32, _vp]),
     "msa_route_set_tile_pool": (C.c_int, [_i32]),
     "msa_gather_plan": (C.c_int, [_vp, _vp, _i32, _i32, _vp]),

@@ -86,6 +86,55 @@ __global__ __launch_bounds__(kThreads) void mfma_loop_kernel(int32_t iters, int3
   sink[tid] = s;
 }
 
+// What the memory system delivers to loops that only read, in the access patterns of the library's HBM-bound kernels.
+// `src` is taken as rows of 2 KB (a token's or a cache row's 8 heads x 128 bf16).  The loaded words are folded with
+// xor so that the loads cannot be dropped.
+// kMode 0: 64 consecutive rows (128 KB) per workgroup of 256 threads, non-temporal 16-byte buffer loads, four per
+//          lane in flight - the pooling kernel's reads.  The fold is stored only if it equals a value it cannot take.
+// kMode 1: the same, and lanes 0 - 127 store their fold: one non-temporal 2 KB row per 128 KB read - pooling's writes.
+template <int kMode>
+__global__ __launch_bounds__(256) void read_rows_kernel(const char* __restrict__ src, char* __restrict__ dst) {
+  const int64_t wg = blockIdx.x;
+  const __amdgpu_buffer_rsrc_t rs =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(src) + wg * (64 * 2048), 0, 64 * 2048, 0x00020000);
+  u32x4_t acc = {0u, 0u, 0u, 0u};
+  for (int i = threadIdx.x * 16; i < 64 * 2048; i += 256 * 16 * 4) {
+    u32x4_t v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = __builtin_amdgcn_raw_buffer_load_b128(rs, i + u * 4096, 0, 2);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc ^= v[u];
+  }
+  if constexpr (kMode == 1) {
+    if (threadIdx.x < 128) __builtin_nontemporal_store(acc, reinterpret_cast<u32x4_t*>(dst + wg * 2048) + threadIdx.x);
+  } else {
+    if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && (acc.x | acc.y) == 0u) *reinterpret_cast<u32x4_t*>(dst) = acc;
+  }
+}
+
+// One KV head's 256-byte piece of every row, 2 KB apart: the decode attention's reads.  Workgroup (head, range) of 512
+// threads, 16 lanes per piece, 32 rows per step and four steps in flight, as in that kernel.
+__global__ __launch_bounds__(512) void read_head_pieces_kernel(const char* __restrict__ src, int64_t rows, int32_t ranges,
+                                                               char* __restrict__ dst) {
+  const int head = blockIdx.x & 7, range = blockIdx.x >> 3;
+  const int64_t per = (rows + ranges - 1) / ranges;
+  const int64_t row0 = range * per, row1 = min(rows, row0 + per);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const char* base = src + head * 256 + (lane & 15) * 16;
+  u32x4_t acc = {0u, 0u, 0u, 0u};
+  for (int64_t r = row0 + wave * 4 + (lane >> 4); r < row1; r += 32 * 4) {
+    u32x4_t v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int64_t rr = r + 32 * u;
+      v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(base + (rr < row1 ? rr : r) * 2048));
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc ^= v[u];
+  }
+  if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u && (acc.x | acc.y) == 0u) *reinterpret_cast<u32x4_t*>(dst) = acc;
+}
+
 // fills the workgroup's dynamic LDS with `word`
 __global__ __launch_bounds__(256) void fill_lds_kernel(uint32_t word, int32_t words, uint32_t* __restrict__ check) {
   extern __shared__ uint32_t lds_words[];
@@ -103,6 +152,27 @@ extern "C" int msa_diag_fill_lds(uint32_t word, uint32_t* check, int32_t workgro
   static std::atomic<int> lds_limit_raised{0};
   MSA_HIP(raise_dynamic_lds_limit(lds_limit_raised, reinterpret_cast<const void*>(fill_lds_kernel), kBytes));
   fill_lds_kernel<<<workgroups, 256, kBytes, as_stream(stream)>>>(word, kBytes / 4, check);
+  MSA_LAUNCH_CHECK();
+  return MSA_OK;
+}
+
+extern "C" int msa_diag_read_stream(const void* src, int64_t bytes, void* dst, int32_t mode, void* stream) {
+  MSA_REQUIRE(src != nullptr && dst != nullptr, "msa_diag_read_stream: null pointer");
+  MSA_REQUIRE(mode >= 0 && mode <= 2, "msa_diag_read_stream: mode %d (0 rows, 1 rows + stores, 2 head pieces)", mode);
+  MSA_REQUIRE(bytes > 0 && bytes % (64 * 2048) == 0 && bytes / (64 * 2048) <= 0x7fffffff,
+              "msa_diag_read_stream: bytes must be a positive multiple of 128 KB");
+  MSA_REQUIRE((((uintptr_t)src | (uintptr_t)dst) & 15) == 0, "msa_diag_read_stream: pointers must be 16-byte aligned");
+  hipStream_t st = as_stream(stream);
+  const unsigned groups = (unsigned)(bytes / (64 * 2048));
+  if (mode == 0) {
+    read_rows_kernel<0><<<groups, 256, 0, st>>>(static_cast<const char*>(src), static_cast<char*>(dst));
+  } else if (mode == 1) {
+    read_rows_kernel<1><<<groups, 256, 0, st>>>(static_cast<const char*>(src), static_cast<char*>(dst));
+  } else {
+    const int ranges = std::max(1, device_compute_units() / 8);       // one workgroup per compute unit
+    read_head_pieces_kernel<<<8 * ranges, 512, 0, st>>>(static_cast<const char*>(src), bytes / 2048, ranges,
+                                                        static_cast<char*>(dst));
+  }
   MSA_LAUNCH_CHECK();
   return MSA_OK;
 }

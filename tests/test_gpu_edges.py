@@ -683,3 +683,32 @@ def test_asm_scheduled_kernels_were_loaded_without_scratch(ops):
         assert scratch.value == 0
         assert regs.value == 512
     assert lib.msa_diag_asm_kernel_resources(2, C.byref(regs), C.byref(scratch)) != 0
+
+
+def test_read_stream_diagnostic_reads_what_it_says(ops):
+    """The measurement aid behind the HBM ceilings: its storing form writes, per 128 KB read, the xor of the 32
+    4 KB slices of that block (so every byte was loaded once); the two non-storing forms leave dst alone; sizes that
+    are no multiple of 128 KB and unknown modes are refused."""
+    say("read-stream diagnostic, 3 x 128 KB")
+    from msa_amd import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    groups = 3
+    src = torch.randint(0, 1 << 31, (groups, 32, 1024), dtype=torch.int32, generator=torch.Generator().manual_seed(5))
+    want = src[:, 0].clone()
+    for i in range(1, 32):
+        want ^= src[:, i]
+    want = want[:, :512]                                     # lanes 0 - 127: 2 KB
+    d_src = src.cuda()
+    dst = torch.full((groups, 512), -7, dtype=torch.int32, device="cuda")
+    _lib.check(lib.msa_diag_read_stream(d_src.data_ptr(), groups * 131072, dst.data_ptr(), 1, st), "msa_diag_read_stream")
+    torch.cuda.synchronize()
+    assert torch.equal(dst.cpu(), want)
+    for mode in (0, 2):
+        dst.fill_(-7)
+        _lib.check(lib.msa_diag_read_stream(d_src.data_ptr(), groups * 131072, dst.data_ptr(), mode, st), "msa_diag_read_stream")
+        torch.cuda.synchronize()
+        assert bool((dst == -7).all())
+    assert lib.msa_diag_read_stream(d_src.data_ptr(), 131072 + 2048, dst.data_ptr(), 0, st) != 0
+    assert lib.msa_diag_read_stream(d_src.data_ptr(), 131072, dst.data_ptr(), 3, st) != 0
+    assert lib.msa_diag_read_stream(None, 131072, dst.data_ptr(), 0, st) != 0

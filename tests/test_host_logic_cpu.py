@@ -236,3 +236,16 @@ def test_compact_cache_in_the_reference_layout():
     want = torch.zeros((B, Hkv, 7, D))
     want.permute(0, 2, 1, 3)[mask] = torch.cat([kc[b, :int(lens[b])] for b in range(B)])
     assert torch.equal(k, want)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU's throughput: a request for several exits with a message that says so, before
+    anything touches a device."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2", "--steps", "1", "--warmup", "0"],
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stdout + r.stderr)
